@@ -1,0 +1,104 @@
+/* exacta_hip.h -- C ABI of libexacta_hip.so: the MI355X (gfx950) backend for the data-parallel
+ * proving path of Exacta/Sable.
+ *
+ * The reference has no FFI: the boundary is drawn inside its Lisp functions.  Each entry point below
+ * names the reference code whose body it replaces (file:line under the reference tree); an SBCL host
+ * binds them with sb-alien (define-alien-routine, pinned (unsigned-byte 32) vectors) and keeps its own
+ * PROVE / VERIFY / CHECK-FINAL API, statements, transcript and proof format.
+ *
+ * Conventions
+ *   - every field value crossing the boundary is a canonical residue in [0, p), p = 2^31 - 2^24 + 1,
+ *     as a little-endian u32; an extension element is D (4 or 8) words in the reference's tower order
+ *     (src/field.lisp:8-11); tables are flat, stride 1 (base) or D (src/sumcheck.lisp:53-59);
+ *   - host buffers are borrowed for the duration of a call only; device tables live behind handles;
+ *   - every function returns EXH_OK or a negative status; exh_last_error() describes the last failure
+ *     of the calling thread in the words of the reference's condition classes (src/conditions.lisp);
+ *   - one context, calls serialised by the caller; every call returns after its small result is on
+ *     the host; nothing calls back into the host language.
+ */
+#ifndef EXACTA_HIP_H
+#define EXACTA_HIP_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EXH_OK 0
+#define EXH_E_PARAM (-1)     /* invalid-parameter        (src/conditions.lisp:96-120) */
+#define EXH_E_DIVZERO (-2)   /* field-division-by-zero   (src/field.lisp:84-96) */
+#define EXH_E_SHAPE (-3)     /* message-shape-error      (src/transcript.lisp:102-114) */
+#define EXH_E_EXHAUSTED (-4) /* transcript-exhausted */
+#define EXH_E_REJECT (-5)    /* verification-failure     (src/conditions.lisp:12-15) */
+#define EXH_E_MALFORMED (-6) /* malformed-proof          (src/conditions.lisp:38-45) */
+#define EXH_E_DEVICE (-7)    /* no usable gfx950 device, or a HIP call failed */
+#define EXH_E_NOMEM (-8)     /* device memory exhausted */
+
+typedef uint64_t exh_table;   /* a device-resident table */
+typedef uint64_t exh_stmt;    /* a compiled statement */
+typedef uint64_t exh_session; /* one sumcheck in progress */
+
+/* ---- context */
+int exh_init(int device);
+void exh_shutdown(void);
+const char *exh_last_error(void);
+/* 1 when a kernel generated for the statement is used, 0 when the interpreter kernel is */
+int exh_stmt_has_generated_kernel(exh_stmt stmt, int degree_d);
+
+/* ---- tables: MAKE-TABLE and the read-back at the end of PROVE (src/sumcheck.lisp:61-70, 564-571) */
+int exh_table_upload(const uint32_t *host, uint64_t n_u32, int stride, exh_table *out);
+int exh_table_alloc(uint64_t n_u32, int stride, exh_table *out);
+/* wrap memory another component already holds on the device (not freed by exh_table_free) */
+int exh_table_wrap(void *device_ptr, uint64_t n_u32, int stride, exh_table *out);
+int exh_table_download(exh_table table, uint64_t offset_u32, uint32_t *host, uint64_t n_u32);
+int exh_table_free(exh_table table);
+void *exh_table_device_ptr(exh_table table);
+/* seeded synthetic table: SplitMix64(seed), 31-bit words, rejected when >= p (the rule of
+   src/transcript.lisp:159-164), generated on the host and uploaded */
+int exh_table_random(uint64_t seed, uint64_t n_u32, int stride, exh_table *out);
+
+/* ---- statements: COMPILE-FORM / ROUND-KERNEL (src/forms.lisp:199-212, src/sumcheck.lisp:270-280).
+   form: the statement's s-expression text, e.g. "(+ (* alpha t0 t1 t2) (* 3 t1))";
+   tables / constants: its variables, in the order the caller passes their values. */
+int exh_stmt_compile(const char *form, const char *const *tables, int n_tables, const char *const *constants,
+                     int n_constants, exh_stmt *out);
+int exh_stmt_degree(exh_stmt stmt); /* STATEMENT-DEGREE, src/sumcheck.lisp:33-35 */
+int exh_stmt_free(exh_stmt stmt);
+
+/* ---- one sumcheck, round by round: the call sites inside PROVE (src/sumcheck.lisp:547-563).
+   tables: n_tables handles of K * 2^n entries each (block-major); eq: n * D words or NULL;
+   block_weights: K * D words or NULL (then K must be 1); constants: n_constants * D words;
+   degree < 0: the statement's degree. */
+int exh_sumcheck_begin(exh_stmt stmt, int degree_d, int n, const exh_table *tables, int n_tables,
+                       const uint32_t *eq, const uint32_t *block_weights, int K, const uint32_t *constants,
+                       int degree, exh_session *out);
+/* the round kernel: (apply kernel flat low high constant-values), src/sumcheck.lisp:556;
+   out_sums: max(degree,1) * D words, the rows of the round message (X = 0, 2, 3, ...) */
+int exh_sumcheck_round(exh_session session, uint32_t *out_sums);
+/* FOLD-FLAT-TABLE of every table by the round's challenge, src/sumcheck.lisp:562, 84-104 */
+int exh_sumcheck_fold(exh_session session, const uint32_t *r);
+/* finals: n_tables * D words (entry 0 of each folded table); folded: NULL, or n_tables pointers to
+   K * D words (src/sumcheck.lisp:564-571).  Ends the session. */
+int exh_sumcheck_finish(exh_session session, uint32_t *finals, uint32_t *const *folded);
+
+/* ---- Reed-Solomon, Merkle, BaseFold kernels (src/rs.lisp:60-101, src/pcs.lisp:44-77, 271-304) */
+/* ENCODE of ncols columns of 2^c base values each (message table: ncols * 2^c words) into codewords
+   of 2^(c+1) words each, bit-reversed order (src/rs.lisp:75-85, src/pcs.lisp:271-273) */
+int exh_rs_encode(exh_table messages, int ncols, int c, exh_table *codewords);
+/* leaf digests + Merkle levels of a class's codewords (src/pcs.lisp:275-277, 293-302): leaf l holds
+   symbols 4l..4l+3 of every column; levels (optional handle out) holds all levels, leaves first, as
+   8-word digests; cap: 32 * cap_rows bytes */
+int exh_merkle_commit(exh_table codewords, int ncols, int c, exh_table *levels, uint8_t *cap, uint64_t *cap_rows);
+/* RS:FOLD of an extension codeword of 2m elements of degree D on twiddle level `level` of the
+   2^n_domain tables (src/rs.lisp:93-101) */
+int exh_rs_fold(exh_table codeword, int degree_d, uint64_t m, int n_domain, int level, const uint32_t *r,
+                exh_table *out);
+
+/* ---- LogUp-GKR layer reductions: FRACTION-TREES (src/gkr.lisp:149-170), one in-block layer:
+   p, q: K * 2^(m+1) EXTs each; out_p, out_q: K * 2^m EXTs (children (b,x), (b,x+2^m)) */
+int exh_gkr_reduce_layer(exh_table p, exh_table q, int degree_d, int K, int m, exh_table *out_p, exh_table *out_q);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,89 @@
+/* exacta_host.h -- C ABI of the host-side mirror of the reference's protocol functions, built into
+ * the same libexacta_hip.so.  An SBCL host does not need these (it keeps its own transcript and
+ * PROVE); they are the stand-in caller that drives the device sessions where no Lisp exists, with
+ * the reference's names, argument meaning and error behaviour, so tests read like the reference's.
+ * Conventions as in exacta_hip.h.
+ */
+#ifndef EXACTA_HOST_H
+#define EXACTA_HOST_H
+#include <stdint.h>
+
+#include "exacta_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint64_t exh_transcript;
+
+/* ---- field helpers on the host (src/field.lisp), for callers without their own arithmetic */
+int exh_ext_mul(int degree_d, const uint32_t *a, const uint32_t *b, uint32_t *out);
+int exh_ext_inv(int degree_d, const uint32_t *a, uint32_t *out); /* EXH_E_DIVZERO on zero (out = 0) */
+int exh_eq_table(int degree_d, int k, const uint32_t *r, uint32_t *out);
+
+/* ---- BLAKE3 and the transcript (src/blake3.lisp, src/transcript.lisp) */
+int exh_blake3(const uint8_t *in, uint64_t len, uint8_t *out, uint64_t out_len);
+/* MAKE-TRANSCRIPT, src/transcript.lisp:75-84; proof != NULL: a verifier replaying the proof's
+   messages (DECODE-PROOF, src/proofio.lisp:53-101; EXH_E_MALFORMED with the reason in last_error) */
+int exh_transcript_new(const uint8_t *label, uint64_t label_len, int degree_d, const uint8_t *proof,
+                       uint64_t proof_len, exh_transcript *out);
+int exh_transcript_free(exh_transcript tr);
+int exh_transcript_absorb(exh_transcript tr, const uint8_t *data, uint64_t len);               /* :95-100 */
+int exh_transcript_send(exh_transcript tr, const uint32_t *vals, int rank, const uint64_t *dims,
+                        uint32_t *out, int absorb);                                              /* :133-148 */
+int exh_transcript_send_bytes(exh_transcript tr, const uint8_t *bytes, int64_t len, uint8_t *out,
+                              uint64_t cap, uint64_t *out_len, int absorb);
+int exh_transcript_challenge_base(exh_transcript tr, int k, uint32_t *out);                      /* :166-172 */
+int exh_transcript_challenge_bits(exh_transcript tr, int nbits, int k, uint64_t *out);          /* :183-187 */
+int exh_transcript_grind(exh_transcript tr, int bits, uint64_t *nonce);                          /* :196-201 */
+int exh_transcript_verify_grind(exh_transcript tr, int bits, uint64_t *nonce);                   /* :203-209 */
+int exh_transcript_digest(exh_transcript tr, uint8_t out[32]);
+int exh_transcript_finished(exh_transcript tr);
+int exh_transcript_message_count(exh_transcript tr, uint64_t *count);
+/* ENCODE-PROOF of the messages so far (src/proofio.lisp:45-49): size in *out_len; bytes written when
+   cap suffices */
+int exh_transcript_proof(exh_transcript tr, uint8_t *out, uint64_t cap, uint64_t *out_len);
+
+/* ---- sumcheck (src/sumcheck.lisp) */
+/* HYPERCUBE-SUM, :112-127: the honest claim, computed on the device */
+int exh_hypercube_sum(exh_stmt stmt, int degree_d, int n, const exh_table *tables, int n_tables,
+                      const uint32_t *eq, const uint32_t *constants, uint32_t *out);
+/* PROVE, :512-571.  out_challenges: n * D; out_finals: n_tables * D; out_folded: NULL or n_tables
+   pointers to K * D words */
+int exh_prove(exh_transcript tr, int n, exh_stmt stmt, const exh_table *tables, int n_tables,
+              const uint32_t *eq, const uint32_t *constants, const uint8_t *label, uint64_t label_len,
+              const uint32_t *block_weights, int K, int degree, uint32_t *out_challenges, uint32_t *out_finals,
+              uint32_t *const *out_folded);
+/* VERIFY, :147-163 */
+int exh_verify(exh_transcript tr, int n, exh_stmt stmt, const uint32_t *claim, const uint32_t *eq,
+               const uint32_t *constants, int blocks, const uint8_t *label, uint64_t label_len, int degree,
+               uint32_t *out_challenges, uint32_t *out_reduced);
+/* CHECK-FINAL, :165-172 */
+int exh_check_final(exh_stmt stmt, int degree_d, const uint32_t *reduced, const uint32_t *finals,
+                    const uint32_t *constants);
+
+/* ---- LogUp-GKR (src/gkr.lisp) */
+/* PROVE-UPPER, :215-272.  leaves: 2 * lookups tables (p, q per lookup) of K * 2^n EXTs */
+int exh_gkr_prove_upper(exh_transcript tr, int n, int K, int lookups, const exh_table *leaves,
+                        const uint8_t *label, uint64_t label_len, uint32_t *out_ri, uint32_t *out_rb,
+                        uint32_t *out_cp, uint32_t *out_cq);
+/* VERIFY-UPPER, :91-145 */
+int exh_gkr_verify_upper(exh_transcript tr, int n, int K, int lookups, const uint8_t *label, uint64_t label_len,
+                         uint32_t *out_roots, uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp,
+                         uint32_t *out_cq);
+
+/* ---- commitment (src/pcs.lisp:279-304, 581-657) */
+/* PCS-COMMIT of one class: encode + leaves + Merkle + send-bytes of the cap on the transcript */
+int exh_pcs_commit(exh_transcript tr, exh_table columns, int ncols, int c, exh_table *codewords,
+                   exh_table *levels);
+/* BASEFOLD of one class of 2^nv EXT8s h (device) at the point rr (nv EXT8s), value v */
+int exh_basefold_prove(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, exh_table h,
+                       int grind_bits, int queries, uint64_t *out_qs, uint32_t *out_challenges,
+                       uint32_t *out_final);
+int exh_basefold_verify(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits,
+                        int queries, uint64_t *out_qs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

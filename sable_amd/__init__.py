@@ -1,0 +1,394 @@
+"""sable_amd -- host-side mirror of the reference's proving-path interface over libexacta_hip.so.
+
+The names and argument meaning follow the reference's Lisp functions (make-transcript, prove, verify,
+check-final, hypercube-sum, prove-upper, verify-upper, encode, pcs-commit, basefold) so that tests read
+like the reference's own.  All compute happens in the HIP library on an MI355X; this module only
+marshals numpy arrays of canonical u32 residues across the C ABI.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import lib as _l
+from .lib import (DeviceError, ExactaError, FieldDivisionByZero, InvalidParameter, MalformedProof,  # noqa: F401
+                  MessageShapeError, TranscriptExhausted, VerificationFailure, check, init, load)
+
+P = 2130706433
+u32p = C.POINTER(C.c_uint32)
+u8p = C.POINTER(C.c_uint8)
+u64p = C.POINTER(C.c_uint64)
+
+
+def _u32(a):
+    a = np.asarray(a, dtype=np.uint64)
+    out = np.empty(a.shape, np.uint32)
+    out[...] = a % P
+    return out
+
+
+def _p(a):
+    return a.ctypes.data_as(u32p) if a is not None else None
+
+
+def _bytes(label):
+    return label.encode() if isinstance(label, str) else bytes(label)
+
+
+# ------------------------------------------------------------------ device tables
+class Table:
+    """A table resident in HBM: base values (stride 1) or extension elements (stride D)."""
+
+    def __init__(self, handle, n_u32, stride):
+        self.handle, self.n_u32, self.stride = handle, n_u32, stride
+
+    @classmethod
+    def upload(cls, values):
+        """make-table (src/sumcheck.lisp:61-70): a 1-d array of base values or a 2-d array of EXTs."""
+        init()
+        a = np.ascontiguousarray(values, dtype=np.uint32)
+        stride = 1 if a.ndim == 1 else a.shape[-1]
+        h = C.c_uint64()
+        check(load().exh_table_upload(_p(a), C.c_uint64(a.size), stride, C.byref(h)))
+        return cls(h.value, a.size, stride)
+
+    @classmethod
+    def random(cls, seed, entries, stride=1):
+        init()
+        h = C.c_uint64()
+        check(load().exh_table_random(C.c_uint64(seed), C.c_uint64(entries * stride), stride, C.byref(h)))
+        return cls(h.value, entries * stride, stride)
+
+    def download(self, offset_u32=0, n_u32=None):
+        n = self.n_u32 - offset_u32 if n_u32 is None else n_u32
+        out = np.zeros(n, np.uint32)
+        check(load().exh_table_download(C.c_uint64(self.handle), C.c_uint64(offset_u32), _p(out), C.c_uint64(n)))
+        return out if self.stride == 1 else out.reshape(-1, self.stride)
+
+    def free(self):
+        if self.handle:
+            load().exh_table_free(C.c_uint64(self.handle))
+            self.handle = 0
+
+    @property
+    def entries(self):
+        return self.n_u32 // self.stride
+
+    def device_ptr(self):
+        return load().exh_table_device_ptr(C.c_uint64(self.handle))
+
+
+def _handles(tables):
+    return (C.c_uint64 * len(tables))(*[t.handle for t in tables])
+
+
+# ------------------------------------------------------------------ statements
+class Statement:
+    """A statement form compiled for the device (compile-form / round-kernel of the reference)."""
+
+    def __init__(self, form, tables, constants=()):
+        self.form, self.tables, self.constants = form, list(tables), list(constants)
+        t = (C.c_char_p * len(self.tables))(*[s.encode() for s in self.tables])
+        c = (C.c_char_p * max(len(self.constants), 1))(*[s.encode() for s in self.constants])
+        h = C.c_uint64()
+        check(load().exh_stmt_compile(form.encode(), t, len(self.tables), c, len(self.constants), C.byref(h)))
+        self.handle = h.value
+        self.degree = load().exh_stmt_degree(C.c_uint64(self.handle))
+
+    def has_generated_kernel(self, d):
+        return load().exh_stmt_has_generated_kernel(C.c_uint64(self.handle), d) == 1
+
+
+# ------------------------------------------------------------------ transcript
+class Transcript:
+    """make-transcript (src/transcript.lisp:75-84); with `proof`, a verifier replaying its messages."""
+
+    def __init__(self, label, degree, proof=None):
+        label = _bytes(label)
+        h = C.c_uint64()
+        check(load().exh_transcript_new(label, C.c_uint64(len(label)), degree, proof,
+                                        C.c_uint64(len(proof) if proof is not None else 0), C.byref(h)))
+        self.handle, self.degree = h.value, degree
+
+    def __del__(self):
+        if getattr(self, "handle", 0):
+            load().exh_transcript_free(C.c_uint64(self.handle))
+            self.handle = 0
+
+    @property
+    def h(self):
+        return C.c_uint64(self.handle)
+
+    def absorb(self, data):
+        data = _bytes(data)
+        check(load().exh_transcript_absorb(self.h, data, C.c_uint64(len(data))))
+
+    def _field(self, value, shape, absorb):
+        if value is not None:
+            a = _u32(value)
+            dims = (C.c_uint64 * 8)(*a.shape)
+            check(load().exh_transcript_send(self.h, _p(a), a.ndim, dims, None, absorb))
+            return a
+        out = np.zeros(shape, np.uint32)
+        dims = (C.c_uint64 * 8)(*shape)
+        check(load().exh_transcript_send(self.h, None, len(shape), dims, _p(out), absorb))
+        return out
+
+    def send(self, value=None, shape=None): return self._field(value, shape, 1)
+    def record(self, value=None, shape=None): return self._field(value, shape, 0)
+
+    def _bytes_msg(self, value, length, absorb):
+        if value is not None:
+            value = bytes(value)
+            check(load().exh_transcript_send_bytes(self.h, value, C.c_int64(len(value)), None, C.c_uint64(0), None,
+                                                   absorb))
+            return value
+        n = C.c_uint64()
+        cap = 1 << 22
+        out = (C.c_uint8 * cap)()
+        check(load().exh_transcript_send_bytes(self.h, None, C.c_int64(-1 if length is None else length), out,
+                                               C.c_uint64(cap), C.byref(n), absorb))
+        return bytes(out[:n.value])
+
+    def send_bytes(self, value=None, length=None): return self._bytes_msg(value, length, 1)
+    def record_bytes(self, value=None, length=None): return self._bytes_msg(value, length, 0)
+
+    def challenge_base(self, k):
+        out = np.zeros(k, np.uint32)
+        check(load().exh_transcript_challenge_base(self.h, k, _p(out)))
+        return out
+
+    def challenge(self, degree=None): return self.challenge_base(degree or self.degree)
+
+    def challenges(self, k, degree=None):
+        d = degree or self.degree
+        return self.challenge_base(d * k).reshape(k, d)
+
+    def challenge_bits(self, nbits, k):
+        out = np.zeros(k, np.uint64)
+        check(load().exh_transcript_challenge_bits(self.h, nbits, k, out.ctypes.data_as(u64p)))
+        return [int(x) for x in out]
+
+    def grind(self, bits):
+        nonce = C.c_uint64()
+        check(load().exh_transcript_grind(self.h, bits, C.byref(nonce)))
+        return nonce.value
+
+    def verify_grind(self, bits):
+        nonce = C.c_uint64()
+        check(load().exh_transcript_verify_grind(self.h, bits, C.byref(nonce)))
+        return nonce.value
+
+    def state_digest(self):
+        out = (C.c_uint8 * 32)()
+        check(load().exh_transcript_digest(self.h, out))
+        return bytes(out)
+
+    def finished(self): return load().exh_transcript_finished(self.h) == 1
+
+    def proof(self):
+        """encode-proof of the messages so far (src/proofio.lisp:45-49)."""
+        n = C.c_uint64()
+        check(load().exh_transcript_proof(self.h, None, C.c_uint64(0), C.byref(n)))
+        out = (C.c_uint8 * max(n.value, 1))()
+        check(load().exh_transcript_proof(self.h, out, n, C.byref(n)))
+        return bytes(out[:n.value])
+
+
+def blake3(data, n=32):
+    out = (C.c_uint8 * n)()
+    check(load().exh_blake3(bytes(data), C.c_uint64(len(data)), out, C.c_uint64(n)))
+    return bytes(out)
+
+
+def ext_mul(a, b):
+    a, b = _u32(a), _u32(b)
+    out = np.zeros_like(a)
+    check(load().exh_ext_mul(len(a), _p(a), _p(b), _p(out)))
+    return out
+
+
+def ext_inv(a):
+    a = _u32(a)
+    out = np.zeros_like(a)
+    check(load().exh_ext_inv(len(a), _p(a), _p(out)))
+    return out
+
+
+def eq_table(r, d):
+    r = _u32(r).reshape(-1, d)
+    out = np.zeros((1 << len(r), d), np.uint32)
+    check(load().exh_eq_table(d, len(r), _p(r), _p(out)))
+    return out
+
+
+# ------------------------------------------------------------------ sumcheck (src/sumcheck.lisp)
+def _opt(a, d):
+    return None if a is None else _u32(a).reshape(-1, d)
+
+
+def _consts(constants, d):
+    if constants is None or len(constants) == 0:
+        return np.zeros((1, d), np.uint32)
+    return _u32(constants).reshape(-1, d)
+
+
+def hypercube_sum(st, n, tables, d, eq=None, constants=None):
+    eqa, ca = _opt(eq, d), _consts(constants, d)
+    out = np.zeros(d, np.uint32)
+    check(load().exh_hypercube_sum(C.c_uint64(st.handle), d, n, _handles(tables), len(tables), _p(eqa), _p(ca),
+                                   _p(out)))
+    return out
+
+
+def prove(tr, n, st, tables, eq=None, constants=None, label="sc", block_weights=None, degree=None):
+    """prove: returns (challenges (n, D), finals (T, D), folded: T arrays (K, D))."""
+    d = tr.degree
+    eqa, ca, bw = _opt(eq, d), _consts(constants, d), _opt(block_weights, d)
+    K = len(bw) if bw is not None else 1
+    chal = np.zeros((n, d), np.uint32)
+    finals = np.zeros((len(tables), d), np.uint32)
+    folded = [np.zeros((K, d), np.uint32) for _ in tables]
+    fptr = (u32p * len(tables))(*[_p(a) for a in folded])
+    label = _bytes(label)
+    check(load().exh_prove(tr.h, n, C.c_uint64(st.handle), _handles(tables), len(tables), _p(eqa), _p(ca), label,
+                           C.c_uint64(len(label)), _p(bw), K, -1 if degree is None else degree, _p(chal), _p(finals),
+                           fptr))
+    return chal, finals, folded
+
+
+def verify(tr, n, st, claim, eq=None, constants=None, blocks=1, label="sc", degree=None):
+    d = tr.degree
+    eqa, ca, claim = _opt(eq, d), _consts(constants, d), _u32(claim)
+    chal = np.zeros((n, d), np.uint32)
+    reduced = np.zeros(d, np.uint32)
+    label = _bytes(label)
+    check(load().exh_verify(tr.h, n, C.c_uint64(st.handle), _p(claim), _p(eqa), _p(ca), blocks, label,
+                            C.c_uint64(len(label)), -1 if degree is None else degree, _p(chal), _p(reduced)))
+    return chal, reduced
+
+
+def check_final(reduced, st, finals, constants=None):
+    reduced = _u32(reduced)
+    d = len(reduced)
+    f, ca = _u32(finals).reshape(-1, d), _consts(constants, d)
+    check(load().exh_check_final(C.c_uint64(st.handle), d, _p(reduced), _p(f), _p(ca)))
+    return True
+
+
+class SumcheckSession:
+    """The round-by-round entry points an SBCL host binds inside its own PROVE."""
+
+    def __init__(self, st, d, n, tables, eq=None, constants=None, block_weights=None, degree=None):
+        self.d, self.points, self.T = d, max(st.degree if degree is None else degree, 1), len(tables)
+        eqa, ca, bw = _opt(eq, d), _consts(constants, d), _opt(block_weights, d)
+        self.K = len(bw) if bw is not None else 1
+        h = C.c_uint64()
+        check(load().exh_sumcheck_begin(C.c_uint64(st.handle), d, n, _handles(tables), len(tables), _p(eqa), _p(bw),
+                                        self.K, _p(ca), -1 if degree is None else degree, C.byref(h)))
+        self.handle = h.value
+
+    def round(self):
+        out = np.zeros((self.points, self.d), np.uint32)
+        check(load().exh_sumcheck_round(C.c_uint64(self.handle), _p(out)))
+        return out
+
+    def fold(self, r):
+        r = _u32(r)
+        check(load().exh_sumcheck_fold(C.c_uint64(self.handle), _p(r)))
+
+    def finish(self):
+        finals = np.zeros((self.T, self.d), np.uint32)
+        folded = [np.zeros((self.K, self.d), np.uint32) for _ in range(self.T)]
+        fptr = (u32p * self.T)(*[_p(a) for a in folded])
+        check(load().exh_sumcheck_finish(C.c_uint64(self.handle), _p(finals), fptr))
+        return finals, folded
+
+
+# ------------------------------------------------------------------ LogUp-GKR (src/gkr.lisp)
+def _block_bits(k):
+    return (k - 1).bit_length()
+
+
+def gkr_reduce_layer(p, q, d, k, m):
+    hp, hq = C.c_uint64(), C.c_uint64()
+    check(load().exh_gkr_reduce_layer(C.c_uint64(p.handle), C.c_uint64(q.handle), d, k, m, C.byref(hp), C.byref(hq)))
+    n = (k << m) * d
+    return Table(hp.value, n, d), Table(hq.value, n, d)
+
+
+def prove_upper(tr, n, k, leaves, label="gkr"):
+    """prove-upper: leaves is a list per lookup of (p, q) device Tables of K * 2^n EXTs."""
+    d = tr.degree
+    flat = [t for pq in leaves for t in pq]
+    L, lk = len(leaves), _block_bits(k)
+    ri, rb = np.zeros((max(n - 1, 0), d), np.uint32), np.zeros((lk, d), np.uint32)
+    cp, cq = np.zeros((L, d), np.uint32), np.zeros((L, d), np.uint32)
+    label = _bytes(label)
+    check(load().exh_gkr_prove_upper(tr.h, n, k, L, _handles(flat), label, C.c_uint64(len(label)), _p(ri), _p(rb),
+                                     _p(cp), _p(cq)))
+    return ri, rb, cp, cq
+
+
+def verify_upper(tr, n, k, lookups, label="gkr"):
+    d = tr.degree
+    lk = _block_bits(k)
+    roots = np.zeros((lookups, 2, d), np.uint32)
+    ri, rb = np.zeros((max(n - 1, 0), d), np.uint32), np.zeros((lk, d), np.uint32)
+    cp, cq = np.zeros((lookups, d), np.uint32), np.zeros((lookups, d), np.uint32)
+    label = _bytes(label)
+    check(load().exh_gkr_verify_upper(tr.h, n, k, lookups, label, C.c_uint64(len(label)), _p(roots), _p(ri), _p(rb),
+                                      _p(cp), _p(cq)))
+    return roots, ri, rb, cp, cq
+
+
+# ------------------------------------------------------------------ commitment (src/rs.lisp, src/pcs.lisp)
+def encode(messages, ncols, c):
+    """encode of ncols columns of 2^c base values (a Table of ncols * 2^c words) -> codewords Table."""
+    h = C.c_uint64()
+    check(load().exh_rs_encode(C.c_uint64(messages.handle), ncols, c, C.byref(h)))
+    return Table(h.value, ncols << (c + 1), 1)
+
+
+def merkle_commit(codewords, ncols, c, want_levels=True):
+    h = C.c_uint64()
+    cap = np.zeros((128, 32), np.uint8)
+    rows = C.c_uint64()
+    check(load().exh_merkle_commit(C.c_uint64(codewords.handle), ncols, c, C.byref(h) if want_levels else None,
+                                   cap.ctypes.data_as(u8p), C.byref(rows)))
+    nleaves = 1 << (c - 1)
+    levels = Table(h.value, (2 * nleaves - 1) * 8, 8) if want_levels else None
+    return levels, cap[:rows.value].copy()
+
+
+def rs_fold(codeword, d, n_domain, level, r):
+    m = codeword.entries // 2
+    r = _u32(r)
+    h = C.c_uint64()
+    check(load().exh_rs_fold(C.c_uint64(codeword.handle), d, C.c_uint64(m), n_domain, level, _p(r), C.byref(h)))
+    return Table(h.value, m * d, d)
+
+
+def pcs_commit(tr, columns, ncols, c):
+    """pcs-commit of one class: encode, leaf digests, Merkle levels; the cap is sent on the transcript."""
+    hc, hl = C.c_uint64(), C.c_uint64()
+    check(load().exh_pcs_commit(tr.h, C.c_uint64(columns.handle), ncols, c, C.byref(hc), C.byref(hl)))
+    nleaves = 1 << (c - 1)
+    return Table(hc.value, ncols << (c + 1), 1), Table(hl.value, (2 * nleaves - 1) * 8, 8)
+
+
+def basefold_prove(tr, nv, rr, v, h, grind_bits=4, queries=6):
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    fl = max(0, nv - 5)
+    qs = np.zeros(queries, np.uint64)
+    chal = np.zeros((max(fl, 1), 8), np.uint32)
+    final = np.zeros((1 << (nv - fl), 8), np.uint32)
+    check(load().exh_basefold_prove(tr.h, nv, _p(rr), _p(v), C.c_uint64(h.handle), grind_bits, queries,
+                                    qs.ctypes.data_as(u64p), _p(chal), _p(final)))
+    return [int(q) for q in qs], chal[:fl], final
+
+
+def basefold_verify(tr, nv, rr, v, grind_bits=4, queries=6):
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    qs = np.zeros(queries, np.uint64)
+    check(load().exh_basefold_verify(tr.h, nv, _p(rr), _p(v), grind_bits, queries, qs.ctypes.data_as(u64p)))
+    return [int(q) for q in qs]

@@ -1,0 +1,567 @@
+// api.hip -- the C ABI (include/exacta_hip.h, include/exacta_host.h) over the C++ internals.
+#include <string.h>
+
+#include <map>
+#include <memory>
+
+#include "../../include/exacta_host.h"
+#include "commit.hpp"
+#include "context.hpp"
+#include "gkr.hpp"
+#include "hostfield.hpp"
+#include "prover.hpp"
+#include "sumcheck.hpp"
+#include "transcript.hpp"
+
+using namespace exh;
+
+namespace {
+std::map<uint64_t, std::unique_ptr<Statement>> g_stmts;
+std::map<uint64_t, std::unique_ptr<SumcheckSession>> g_sessions;
+std::map<uint64_t, std::unique_ptr<Transcript>> g_transcripts;
+uint64_t g_next = 1;
+
+Statement *stmt_of(exh_stmt h) {
+  auto it = g_stmts.find(h);
+  if (it == g_stmts.end()) {
+    set_error("invalid-parameter: unknown statement handle");
+    return nullptr;
+  }
+  return it->second.get();
+}
+Transcript *tr_of(exh_transcript h) {
+  auto it = g_transcripts.find(h);
+  if (it == g_transcripts.end()) {
+    set_error("invalid-parameter: unknown transcript handle");
+    return nullptr;
+  }
+  return it->second.get();
+}
+DeviceTable *table_of(exh_table h) {
+  auto it = ctx().tables.find(h);
+  if (it == ctx().tables.end()) {
+    set_error("invalid-parameter: unknown table handle");
+    return nullptr;
+  }
+  return &it->second;
+}
+exh_table add_table(uint32_t *ptr, uint64_t n_u32, int stride, bool owned) {
+  Context &c = ctx();
+  uint64_t h = c.next_handle++;
+  c.tables[h] = DeviceTable{ptr, n_u32, stride, owned};
+  return h;
+}
+// device pointers and strides of a list of table handles, each checked against `entries`
+int gather_tables(const exh_table *tables, int n, int D, uint64_t entries, std::vector<const uint32_t *> *ptrs,
+                  std::vector<int> *strides) {
+  ptrs->clear();
+  strides->clear();
+  for (int t = 0; t < n; t++) {
+    DeviceTable *dt = table_of(tables[t]);
+    if (!dt) return E_PARAM;
+    if (dt->stride != 1 && dt->stride != D) {
+      set_error("invalid-parameter: table stride must be 1 or the transcript's degree");
+      return E_PARAM;
+    }
+    if (dt->n_u32 != entries * (uint64_t)dt->stride) {
+      set_error("invalid-parameter: table size: expected " + std::to_string(entries) + " entries");
+      return E_PARAM;
+    }
+    ptrs->push_back(dt->ptr);
+    strides->push_back(dt->stride);
+  }
+  return OK;
+}
+}  // namespace
+
+extern "C" {
+
+// ------------------------------------------------------------------ context
+int exh_init(int device) { return ctx_init(device); }
+void exh_shutdown(void) {
+  g_sessions.clear();
+  ctx_shutdown();
+}
+const char *exh_last_error(void) { return last_error(); }
+
+// ------------------------------------------------------------------ tables
+int exh_table_alloc(uint64_t n_u32, int stride, exh_table *out) {
+  int status = ctx().require();
+  if (status) return status;
+  if (stride < 1 || stride > 8 || n_u32 % stride) {
+    set_error("invalid-parameter: table stride");
+    return E_PARAM;
+  }
+  void *ptr = nullptr;
+  hipError_t e = hipMalloc(&ptr, n_u32 ? n_u32 * 4 : 4);
+  if (e != hipSuccess) {
+    set_error(std::string("device-out-of-memory: ") + hipGetErrorString(e));
+    return E_NOMEM;
+  }
+  *out = add_table((uint32_t *)ptr, n_u32, stride, true);
+  return OK;
+}
+
+int exh_table_upload(const uint32_t *host, uint64_t n_u32, int stride, exh_table *out) {
+  for (uint64_t i = 0; i < n_u32; i++)
+    if (host[i] >= P) {
+      set_error("invalid-parameter: table values must be canonical (below p)");
+      return E_PARAM;
+    }
+  int status = exh_table_alloc(n_u32, stride, out);
+  if (status) return status;
+  DeviceTable *dt = table_of(*out);
+  EXH_HIP(hipMemcpy(dt->ptr, host, n_u32 * 4, hipMemcpyHostToDevice));
+  return OK;
+}
+
+int exh_table_wrap(void *device_ptr, uint64_t n_u32, int stride, exh_table *out) {
+  int status = ctx().require();
+  if (status) return status;
+  if (!device_ptr || stride < 1 || stride > 8 || ((uintptr_t)device_ptr & 15)) {
+    set_error("invalid-parameter: wrapped table must be a 16-byte aligned device pointer");
+    return E_PARAM;
+  }
+  *out = add_table((uint32_t *)device_ptr, n_u32, stride, false);
+  return OK;
+}
+
+int exh_table_download(exh_table table, uint64_t offset_u32, uint32_t *host, uint64_t n_u32) {
+  DeviceTable *dt = table_of(table);
+  if (!dt) return E_PARAM;
+  if (offset_u32 + n_u32 > dt->n_u32) {
+    set_error("invalid-parameter: download beyond the table");
+    return E_PARAM;
+  }
+  EXH_HIP(hipStreamSynchronize(ctx().stream));
+  EXH_HIP(hipMemcpy(host, dt->ptr + offset_u32, n_u32 * 4, hipMemcpyDeviceToHost));
+  return OK;
+}
+
+int exh_table_free(exh_table table) {
+  DeviceTable *dt = table_of(table);
+  if (!dt) return E_PARAM;
+  (void)hipStreamSynchronize(ctx().stream);
+  if (dt->owned && dt->ptr) EXH_HIP(hipFree(dt->ptr));
+  ctx().tables.erase(table);
+  return OK;
+}
+
+void *exh_table_device_ptr(exh_table table) {
+  DeviceTable *dt = table_of(table);
+  return dt ? dt->ptr : nullptr;
+}
+
+int exh_table_random(uint64_t seed, uint64_t n_u32, int stride, exh_table *out) {
+  std::vector<uint32_t> host(n_u32);
+  uint64_t x = seed;
+  for (uint64_t i = 0; i < n_u32;) {
+    x += 0x9E3779B97F4A7C15ull;  // SplitMix64
+    uint64_t z = x;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    uint32_t w = (uint32_t)(z >> 33);
+    if (w < P) host[i++] = w;
+  }
+  int status = exh_table_alloc(n_u32, stride, out);
+  if (status) return status;
+  EXH_HIP(hipMemcpy(table_of(*out)->ptr, host.data(), n_u32 * 4, hipMemcpyHostToDevice));
+  return OK;
+}
+
+// ------------------------------------------------------------------ statements
+int exh_stmt_compile(const char *form, const char *const *tables, int n_tables, const char *const *constants,
+                     int n_constants, exh_stmt *out) {
+  auto st = std::make_unique<Statement>();
+  std::vector<std::string> tn, cn;
+  for (int i = 0; i < n_tables; i++) tn.push_back(tables[i]);
+  for (int i = 0; i < n_constants; i++) cn.push_back(constants[i]);
+  int status = compile_statement(form, tn, cn, st.get());
+  if (status) return status;
+  *out = g_next++;
+  g_stmts[*out] = std::move(st);
+  return OK;
+}
+int exh_stmt_degree(exh_stmt stmt) {
+  Statement *st = stmt_of(stmt);
+  return st ? st->degree : E_PARAM;
+}
+int exh_stmt_free(exh_stmt stmt) {
+  if (!stmt_of(stmt)) return E_PARAM;
+  g_stmts.erase(stmt);
+  return OK;
+}
+int exh_stmt_has_generated_kernel(exh_stmt stmt, int D) {
+  Statement *st = stmt_of(stmt);
+  if (!st) return E_PARAM;
+  Statement copy = *st;
+  copy.plan(copy.degree > 1 ? copy.degree : 1);
+  return find_kernels(copy.key(), D) ? 1 : 0;
+}
+
+// ------------------------------------------------------------------ sumcheck sessions
+int exh_sumcheck_begin(exh_stmt stmt, int D, int n, const exh_table *tables, int n_tables, const uint32_t *eq,
+                       const uint32_t *bw, int K, const uint32_t *constants, int degree, exh_session *out) {
+  Statement *st = stmt_of(stmt);
+  if (!st) return E_PARAM;
+  if (n_tables != st->T() || (!bw && K != 1) || K < 1 || n < 0 || n > 40) {
+    set_error("invalid-parameter: sumcheck arguments");
+    return E_PARAM;
+  }
+  std::vector<const uint32_t *> ptrs;
+  std::vector<int> strides;
+  int status = gather_tables(tables, n_tables, D, (uint64_t)K << n, &ptrs, &strides);
+  if (status) return status;
+  auto s = std::make_unique<SumcheckSession>();
+  if ((status = s->begin(*st, D, n, ptrs.data(), strides.data(), eq, bw, K, constants, degree))) return status;
+  *out = g_next++;
+  g_sessions[*out] = std::move(s);
+  return OK;
+}
+static SumcheckSession *session_of(exh_session h) {
+  auto it = g_sessions.find(h);
+  if (it == g_sessions.end()) {
+    set_error("invalid-parameter: unknown session handle");
+    return nullptr;
+  }
+  return it->second.get();
+}
+int exh_sumcheck_round(exh_session session, uint32_t *out_sums) {
+  SumcheckSession *s = session_of(session);
+  return s ? s->round_sums(out_sums) : E_PARAM;
+}
+int exh_sumcheck_fold(exh_session session, const uint32_t *r) {
+  SumcheckSession *s = session_of(session);
+  return s ? s->fold(r) : E_PARAM;
+}
+int exh_sumcheck_finish(exh_session session, uint32_t *finals, uint32_t *const *folded) {
+  SumcheckSession *s = session_of(session);
+  if (!s) return E_PARAM;
+  int status = s->finish(finals, folded);
+  g_sessions.erase(session);
+  return status;
+}
+
+// ------------------------------------------------------------------ host field helpers
+int exh_ext_mul(int D, const uint32_t *a, const uint32_t *b, uint32_t *out) {
+  if (D != 4 && D != 8) return E_PARAM;
+  hf::mul_raw(D, a, b, out);
+  return OK;
+}
+int exh_ext_inv(int D, const uint32_t *a, uint32_t *out) {
+  if (D != 4 && D != 8) return E_PARAM;
+  hf::E x = hf::from(a, D);
+  if (hf::is_zero(x)) {
+    memset(out, 0, 4 * D);
+    set_error("field-division-by-zero: ext-inv");
+    return E_DIVZERO;
+  }
+  hf::E r = hf::inv(x);
+  memcpy(out, r.data(), 4 * D);
+  return OK;
+}
+int exh_eq_table(int D, int k, const uint32_t *r, uint32_t *out) {
+  if ((D != 4 && D != 8) || k < 0 || k > 24) return E_PARAM;
+  std::vector<uint32_t> t = hf::eq_table(r, k, D);
+  memcpy(out, t.data(), t.size() * 4);
+  return OK;
+}
+
+// ------------------------------------------------------------------ transcript
+int exh_blake3(const uint8_t *in, uint64_t len, uint8_t *out, uint64_t out_len) {
+  blake3_hash(in, len, out, out_len);
+  return OK;
+}
+int exh_transcript_new(const uint8_t *label, uint64_t label_len, int D, const uint8_t *proof, uint64_t proof_len,
+                       exh_transcript *out) {
+  if (D != 4 && D != 8) {
+    set_error("invalid-parameter: degree: expected 4 or 8");
+    return E_PARAM;
+  }
+  auto tr = std::make_unique<Transcript>(label, label_len, D);
+  if (proof) {
+    int status = tr->load_proof(proof, proof_len);
+    if (status) {
+      static const char *reasons[] = {"", "magic", "truncated", "trailing-bytes", "unknown-tag", "value-range", "rank",
+                                      "dimension"};
+      set_error(std::string("malformed-proof: ") + reasons[tr->malformed_reason]);
+      return status;
+    }
+  }
+  *out = g_next++;
+  g_transcripts[*out] = std::move(tr);
+  return OK;
+}
+int exh_transcript_free(exh_transcript h) {
+  if (!tr_of(h)) return E_PARAM;
+  g_transcripts.erase(h);
+  return OK;
+}
+int exh_transcript_absorb(exh_transcript h, const uint8_t *data, uint64_t len) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  tr->absorb(data, len);
+  return OK;
+}
+int exh_transcript_send(exh_transcript h, const uint32_t *vals, int rank, const uint64_t *dims, uint32_t *out,
+                        int absorb) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  int status = tr->send(vals, rank, dims, out, absorb != 0);
+  if (status == E_SHAPE) set_error("message-shape-error");
+  if (status == E_EXHAUSTED) set_error("transcript-exhausted");
+  return status;
+}
+int exh_transcript_send_bytes(exh_transcript h, const uint8_t *bytes, int64_t len, uint8_t *out, uint64_t cap,
+                              uint64_t *out_len, int absorb) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  std::vector<uint8_t> got;
+  int status = tr->send_bytes(bytes, len, &got, absorb != 0);
+  if (status == E_SHAPE) set_error("message-shape-error");
+  if (status == E_EXHAUSTED) set_error("transcript-exhausted");
+  if (status) return status;
+  if (out_len) *out_len = got.size();
+  if (out) memcpy(out, got.data(), got.size() < cap ? got.size() : cap);
+  return OK;
+}
+int exh_transcript_challenge_base(exh_transcript h, int k, uint32_t *out) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  tr->challenge_base(k, out);
+  return OK;
+}
+int exh_transcript_challenge_bits(exh_transcript h, int nbits, int k, uint64_t *out) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  tr->challenge_bits(nbits, k, out);
+  return OK;
+}
+int exh_transcript_grind(exh_transcript h, int bits, uint64_t *nonce) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  *nonce = tr->grind(bits);
+  return OK;
+}
+int exh_transcript_verify_grind(exh_transcript h, int bits, uint64_t *nonce) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  int status = tr->verify_grind(bits, nonce);
+  if (status == E_REJECT) set_error("verification-failure: proof-of-work");
+  return status;
+}
+int exh_transcript_digest(exh_transcript h, uint8_t out[32]) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  tr->state.digest(out, 32);
+  return OK;
+}
+int exh_transcript_finished(exh_transcript h) {
+  Transcript *tr = tr_of(h);
+  return tr ? (tr->finished() ? 1 : 0) : E_PARAM;
+}
+int exh_transcript_message_count(exh_transcript h, uint64_t *count) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  *count = tr->messages.size();
+  return OK;
+}
+int exh_transcript_proof(exh_transcript h, uint8_t *out, uint64_t cap, uint64_t *out_len) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  std::vector<uint8_t> bytes = tr->encode_proof();
+  *out_len = bytes.size();
+  if (out && cap >= bytes.size()) memcpy(out, bytes.data(), bytes.size());
+  return OK;
+}
+
+// ------------------------------------------------------------------ sumcheck protocol
+int exh_hypercube_sum(exh_stmt stmt, int D, int n, const exh_table *tables, int n_tables, const uint32_t *eq,
+                      const uint32_t *constants, uint32_t *out) {
+  Statement *st = stmt_of(stmt);
+  if (!st) return E_PARAM;
+  if (n_tables != st->T()) {
+    set_error("invalid-parameter: table count");
+    return E_PARAM;
+  }
+  std::vector<const uint32_t *> ptrs;
+  std::vector<int> strides;
+  int status = gather_tables(tables, n_tables, D, (uint64_t)1 << n, &ptrs, &strides);
+  if (status) return status;
+  if (n == 0) {  // one row: the statement at the tables' only entries
+    std::vector<uint32_t> tv((size_t)n_tables * D, 0);
+    for (int t = 0; t < n_tables; t++)
+      EXH_HIP(hipMemcpy(&tv[(size_t)t * D], ptrs[t], 4 * strides[t], hipMemcpyDeviceToHost));
+    evaluate_statement(*st, D, tv.data(), constants, out);
+    return OK;
+  }
+  SumcheckSession s;
+  if ((status = s.begin(*st, D, n, ptrs.data(), strides.data(), eq, nullptr, 1, constants, -1, true))) return status;
+  uint32_t sums[16 * 8];
+  if ((status = s.round_sums(sums))) return status;
+  memcpy(out, sums, 4 * D);
+  return OK;
+}
+
+int exh_prove(exh_transcript h, int n, exh_stmt stmt, const exh_table *tables, int n_tables, const uint32_t *eq,
+              const uint32_t *constants, const uint8_t *label, uint64_t label_len, const uint32_t *bw, int K,
+              int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded) {
+  Transcript *tr = tr_of(h);
+  Statement *st = stmt_of(stmt);
+  if (!tr || !st) return E_PARAM;
+  if (n_tables != st->T() || (!bw && K != 1) || K < 1) {
+    set_error("invalid-parameter: prove arguments");
+    return E_PARAM;
+  }
+  std::vector<const uint32_t *> ptrs;
+  std::vector<int> strides;
+  int status = gather_tables(tables, n_tables, tr->D, (uint64_t)K << n, &ptrs, &strides);
+  if (status) return status;
+  return sumcheck_prove(*tr, n, *st, ptrs.data(), strides.data(), eq, constants,
+                        std::string((const char *)label, label_len), bw, K, degree, out_chal, out_finals, out_folded);
+}
+
+int exh_verify(exh_transcript h, int n, exh_stmt stmt, const uint32_t *claim, const uint32_t *eq,
+               const uint32_t *constants, int blocks, const uint8_t *label, uint64_t label_len, int degree,
+               uint32_t *out_chal, uint32_t *out_reduced) {
+  Transcript *tr = tr_of(h);
+  Statement *st = stmt_of(stmt);
+  if (!tr || !st) return E_PARAM;
+  return sumcheck_verify(*tr, n, *st, claim, eq, constants, blocks, std::string((const char *)label, label_len),
+                         degree, out_chal, out_reduced);
+}
+
+int exh_check_final(exh_stmt stmt, int D, const uint32_t *reduced, const uint32_t *finals, const uint32_t *constants) {
+  Statement *st = stmt_of(stmt);
+  if (!st) return E_PARAM;
+  return check_final(*st, D, reduced, finals, constants);
+}
+
+// ------------------------------------------------------------------ GKR
+int exh_gkr_reduce_layer(exh_table p, exh_table q, int D, int K, int m, exh_table *out_p, exh_table *out_q) {
+  DeviceTable *dp = table_of(p), *dq = table_of(q);
+  if (!dp || !dq) return E_PARAM;
+  uint64_t in_entries = (uint64_t)K << (m + 1);
+  if ((D != 4 && D != 8) || dp->stride != D || dq->stride != D || dp->n_u32 != in_entries * D ||
+      dq->n_u32 != in_entries * D) {
+    set_error("invalid-parameter: layer tables must hold K * 2^(m+1) extension elements");
+    return E_PARAM;
+  }
+  int status;
+  if ((status = exh_table_alloc((in_entries / 2) * D, D, out_p))) return status;
+  if ((status = exh_table_alloc((in_entries / 2) * D, D, out_q))) return status;
+  return gkr_reduce_layer(D, K, m, dp->ptr, dq->ptr, table_of(*out_p)->ptr, table_of(*out_q)->ptr);
+}
+
+int exh_gkr_prove_upper(exh_transcript h, int n, int K, int lookups, const exh_table *leaves, const uint8_t *label,
+                        uint64_t label_len, uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp, uint32_t *out_cq) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  std::vector<const uint32_t *> ptrs;
+  std::vector<int> strides;
+  int status = gather_tables(leaves, 2 * lookups, tr->D, (uint64_t)K << n, &ptrs, &strides);
+  if (status) return status;
+  for (int s : strides)
+    if (s != tr->D) {
+      set_error("invalid-parameter: GKR leaves are extension elements");
+      return E_PARAM;
+    }
+  return gkr_prove_upper(*tr, n, K, lookups, ptrs.data(), std::string((const char *)label, label_len), out_ri, out_rb,
+                         out_cp, out_cq);
+}
+
+int exh_gkr_verify_upper(exh_transcript h, int n, int K, int lookups, const uint8_t *label, uint64_t label_len,
+                         uint32_t *out_roots, uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp,
+                         uint32_t *out_cq) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  return gkr_verify_upper(*tr, n, K, lookups, std::string((const char *)label, label_len), out_roots, out_ri, out_rb,
+                          out_cp, out_cq);
+}
+
+// ------------------------------------------------------------------ Reed-Solomon, Merkle, BaseFold
+int exh_rs_encode(exh_table messages, int ncols, int c, exh_table *codewords) {
+  DeviceTable *m = table_of(messages);
+  if (!m) return E_PARAM;
+  if (ncols < 1 || c < 0 || c > 23 || m->stride != 1 || m->n_u32 != ((uint64_t)ncols << c)) {
+    set_error("invalid-parameter: messages must hold ncols * 2^c base values, c <= 23");
+    return E_PARAM;
+  }
+  int status = exh_table_alloc((uint64_t)ncols << (c + 1), 1, codewords);
+  if (status) return status;
+  return rs_encode_columns(m->ptr, ncols, c, table_of(*codewords)->ptr);
+}
+
+int exh_merkle_commit(exh_table codewords, int ncols, int c, exh_table *levels, uint8_t *cap, uint64_t *cap_rows) {
+  DeviceTable *cw = table_of(codewords);
+  if (!cw) return E_PARAM;
+  if (ncols < 1 || c < 1 || c > 23 || cw->n_u32 != ((uint64_t)ncols << (c + 1))) {
+    set_error("invalid-parameter: codewords must hold ncols * 2^(c+1) symbols, 1 <= c <= 23");
+    return E_PARAM;
+  }
+  uint64_t nleaves = (uint64_t)1 << (c - 1);
+  exh_table lv;
+  int status = exh_table_alloc((2 * nleaves - 1) * 8, 8, &lv);
+  if (status) return status;
+  status = merkle_commit_columns(cw->ptr, ncols, c, table_of(lv)->ptr, cap, cap_rows);
+  if (status || !levels)
+    exh_table_free(lv);
+  else
+    *levels = lv;
+  return status;
+}
+
+int exh_rs_fold(exh_table codeword, int D, uint64_t m, int n_domain, int level, const uint32_t *r, exh_table *out) {
+  DeviceTable *cw = table_of(codeword);
+  if (!cw) return E_PARAM;
+  if ((D != 4 && D != 8) || cw->n_u32 != 2 * m * D || n_domain < 1 || n_domain > 24 || level < 0 ||
+      m != ((uint64_t)1 << (n_domain - 1 - level))) {
+    set_error("invalid-parameter: codeword of 2m extension elements on level `level` of the 2^n_domain tables");
+    return E_PARAM;
+  }
+  int status = exh_table_alloc(m * D, D, out);
+  if (status) return status;
+  return rs_fold_device(D, m, n_domain, level, cw->ptr, r, table_of(*out)->ptr);
+}
+
+int exh_pcs_commit(exh_transcript h, exh_table columns, int ncols, int c, exh_table *codewords, exh_table *levels) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  exh_table cw;
+  int status = exh_rs_encode(columns, ncols, c, &cw);
+  if (status) return status;
+  std::vector<uint8_t> cap(32 * ((size_t)1 << 7));
+  uint64_t rows = 0;
+  if ((status = exh_merkle_commit(cw, ncols, c, levels, cap.data(), &rows))) {
+    exh_table_free(cw);
+    return status;
+  }
+  status = tr->send_bytes(cap.data(), (int64_t)(32 * rows), nullptr);
+  if (codewords)
+    *codewords = cw;
+  else
+    exh_table_free(cw);
+  return status;
+}
+
+int exh_basefold_prove(exh_transcript h, int nv, const uint32_t *rr, const uint32_t *v, exh_table table, int grind_bits,
+                       int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final) {
+  Transcript *tr = tr_of(h);
+  DeviceTable *dt = table_of(table);
+  if (!tr || !dt) return E_PARAM;
+  if (nv < 1 || nv > 23 || dt->stride != 8 || dt->n_u32 != ((uint64_t)8 << nv)) {
+    set_error("invalid-parameter: BaseFold takes 2^nv EXT8s, 1 <= nv <= 23");
+    return E_PARAM;
+  }
+  return basefold_prove(*tr, nv, rr, v, dt->ptr, grind_bits, queries, out_qs, out_chal, out_final);
+}
+
+int exh_basefold_verify(exh_transcript h, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,
+                        uint64_t *out_qs) {
+  Transcript *tr = tr_of(h);
+  if (!tr) return E_PARAM;
+  return basefold_verify(*tr, nv, rr, v, grind_bits, queries, out_qs);
+}
+
+}  // extern "C"

@@ -1,0 +1,667 @@
+// commit.hip -- see commit.hpp.
+#include "commit.hpp"
+
+#include <string.h>
+
+#include <algorithm>
+#include <map>
+#include <vector>
+
+#include "blake3.cuh"
+#include "context.hpp"
+#include "hostfield.hpp"
+#include "sumcheck_kernels.cuh"
+
+namespace exh {
+
+// ------------------------------------------------------------------ twiddle tables of a domain
+// Level l of the 2^n tables (src/rs.lisp:44-55) holds x_s = w_n^(2^l bitrev_{n-1-l}(s)) for the
+// 2^(n-1-l) position pairs of the level-l codeword.  Both x (for the encoder's butterflies) and
+// 1/(2x) (for folding) are kept on the device in Montgomery form, levels concatenated.
+struct Domain {
+  int n = 0;
+  uint32_t *tw = nullptr, *tw_inv2 = nullptr;
+  uint64_t off[32];
+};
+static std::map<int, Domain> g_domains;
+
+struct LevelOffsets {
+  uint64_t off[32];
+  int levels, n;
+};
+
+__device__ __forceinline__ uint32_t bitrev_dev(uint32_t v, int bits) { return bits ? __brev(v) >> (32 - bits) : 0; }
+
+// pw: w_n^e for e < 4096, then w_n^(4096 e) for e < 4096 (Montgomery form); pw_inv the same for
+// the inverse root times 1/2 folded into the first table
+__global__ __launch_bounds__(BLOCK) void twiddle_kernel(LevelOffsets lv, const uint32_t *pw, const uint32_t *pw_inv,
+                                                        uint32_t *tw, uint32_t *tw_inv2, uint64_t total) {
+  uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid >= total) return;
+  int l = 0;
+  while (l + 1 < lv.levels && gid >= lv.off[l + 1]) l++;
+  uint32_t s = (uint32_t)(gid - lv.off[l]);
+  uint32_t e = bitrev_dev(s, lv.n - 1 - l) << l;  // exponent of w_n, below 2^(n-1)
+  // mont_mul of two Montgomery-form values is the Montgomery form of the product
+  tw[gid] = mont_mul(pw[e & 4095], pw[4096 + (e >> 12)]);
+  tw_inv2[gid] = mont_mul(pw_inv[e & 4095], pw_inv[4096 + (e >> 12)]);
+}
+
+static int get_domain(int n, Domain **out) {
+  auto it = g_domains.find(n);
+  if (it != g_domains.end()) {
+    *out = &it->second;
+    return OK;
+  }
+  Context &c = ctx();
+  Domain d;
+  d.n = n;
+  int levels = n - 1 > 1 ? n - 1 : 1;
+  uint64_t total = 0, len = (uint64_t)1 << (n - 1);
+  LevelOffsets lv;
+  memset(&lv, 0, sizeof(lv));
+  for (int l = 0; l < levels; l++, len /= 2) {
+    d.off[l] = lv.off[l] = total;
+    total += len;
+  }
+  lv.levels = levels;
+  lv.n = n;
+  uint32_t w = fpow(3, (uint64_t)(P - 1) >> n), winv = finv(w);
+  std::vector<uint32_t> pw(8192), pwi(8192);
+  uint32_t x = 1, xi = INV2;  // the 1/2 of 1/(2x) rides on the low table
+  for (int e = 0; e < 4096; e++) {
+    pw[e] = to_mont(x), pwi[e] = to_mont(xi);
+    x = fmul(x, w), xi = fmul(xi, winv);
+  }
+  uint32_t w4096 = fpow(w, 4096), wi4096 = fpow(winv, 4096);
+  x = 1, xi = 1;
+  for (int e = 0; e < 4096; e++) {
+    pw[4096 + e] = to_mont(x), pwi[4096 + e] = to_mont(xi);
+    x = fmul(x, w4096), xi = fmul(xi, wi4096);
+  }
+  uint32_t *d_pw = nullptr;
+  EXH_HIP(hipMalloc((void **)&d_pw, 2 * 8192 * 4));
+  EXH_HIP(hipMemcpy(d_pw, pw.data(), 8192 * 4, hipMemcpyHostToDevice));
+  EXH_HIP(hipMemcpy(d_pw + 8192, pwi.data(), 8192 * 4, hipMemcpyHostToDevice));
+  EXH_HIP(hipMalloc((void **)&d.tw, total * 4));
+  EXH_HIP(hipMalloc((void **)&d.tw_inv2, total * 4));
+  uint32_t grid = (uint32_t)((total + BLOCK - 1) / BLOCK);
+  hipLaunchKernelGGL(twiddle_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, lv, d_pw, d_pw + 8192, d.tw, d.tw_inv2,
+                     total);
+  EXH_HIP(hipGetLastError());
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  EXH_HIP(hipFree(d_pw));
+  g_domains[n] = d;
+  *out = &g_domains[n];
+  return OK;
+}
+
+// ------------------------------------------------------------------ the encoder
+// One pass of the butterflies (src/rs.lisp:60-73) for the stages b = b_hi .. b_lo over tiles held
+// in LDS.  An index is (top | mid | low) with mid the bits b_lo..b_hi; a workgroup takes one top,
+// all 2^S mids and C consecutive lows (C = tile / 2^S), so its loads are segments of C words and
+// every butterfly of these stages stays inside the tile.  With `first` the input is the message
+// m, read as m || m (src/rs.lisp:81).
+constexpr int NTT_TILE_BITS = 12;
+
+__global__ __launch_bounds__(BLOCK) void ntt_pass_kernel(const uint32_t *in, uint32_t *out, int n, int b_hi, int b_lo,
+                                                         int tile_bits, const uint32_t *tw, LevelOffsets lv,
+                                                         int first, uint64_t in_stride, uint64_t out_stride) {
+  __shared__ uint32_t lds[1 << NTT_TILE_BITS];
+  const int S = b_hi - b_lo + 1, cbits = tile_bits - S;
+  const uint32_t tile = 1u << tile_bits, C = 1u << cbits;
+  in += (uint64_t)blockIdx.y * in_stride;
+  out += (uint64_t)blockIdx.y * out_stride;
+  const uint64_t chunks_per_top = ((uint64_t)1 << b_lo) >> cbits;
+  const uint64_t top = blockIdx.x / chunks_per_top, chunk = blockIdx.x % chunks_per_top;
+  const uint64_t base = (top << (b_hi + 1)) | (chunk << cbits);
+  const uint64_t msg_mask = ((uint64_t)1 << (n - 1)) - 1;
+  for (uint32_t e = threadIdx.x; e < tile; e += BLOCK) {
+    uint64_t g = base | ((uint64_t)(e >> cbits) << b_lo) | (e & (C - 1));
+    lds[e] = first ? in[g & msg_mask] : in[g];
+  }
+  __syncthreads();
+  for (int b = b_hi; b >= b_lo; b--) {
+    const int d = b - b_lo;
+    const uint32_t *level = tw + lv.off[b];
+    for (uint32_t u = threadIdx.x; u < tile / 2; u += BLOCK) {
+      uint32_t cc = u & (C - 1), mm = u >> cbits;
+      uint32_t mid_lo = mm & ((1u << d) - 1), mid_hi = mm >> d;
+      uint32_t ia = ((((mid_hi << (d + 1)) | mid_lo)) << cbits) | cc, ib = ia + (1u << (d + cbits));
+      uint64_t k = (top << (b_hi - b)) | mid_hi;
+      uint32_t a = lds[ia], tc = mont_mul(level[k], lds[ib]);
+      lds[ia] = fadd(a, tc);
+      lds[ib] = fsub(a, tc);
+    }
+    __syncthreads();
+  }
+  for (uint32_t e = threadIdx.x; e < tile; e += BLOCK) {
+    uint64_t g = base | ((uint64_t)(e >> cbits) << b_lo) | (e & (C - 1));
+    out[g] = lds[e];
+  }
+}
+
+// m || m for the degenerate domains with no butterfly stage
+__global__ void dup_kernel(const uint32_t *in, uint32_t *out, uint64_t half, uint64_t in_stride, uint64_t out_stride) {
+  uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid < 2 * half) out[blockIdx.y * out_stride + gid] = in[blockIdx.y * in_stride + (gid % half)];
+}
+
+int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_codewords) {
+  Context &cx = ctx();
+  int status = cx.require();
+  if (status) return status;
+  int n = c + 1;
+  uint64_t len = (uint64_t)1 << n;
+  if (n < 2) {
+    hipLaunchKernelGGL(dup_kernel, dim3(1, ncols), dim3(64), 0, cx.stream, d_messages, d_codewords, len / 2, len / 2, len);
+    EXH_HIP(hipGetLastError());
+    return OK;
+  }
+  Domain *dom;
+  if ((status = get_domain(n, &dom))) return status;
+  LevelOffsets lv;
+  memset(&lv, 0, sizeof(lv));
+  lv.levels = n - 1, lv.n = n;
+  for (int l = 0; l < n - 1; l++) lv.off[l] = dom->off[l];
+  int tile_bits = n - 1 < NTT_TILE_BITS ? n - 1 : NTT_TILE_BITS;  // a tile never spans two tops
+  // stages n-2 .. 0: the last pass takes the low tile_bits stages, earlier passes up to 7 each
+  int b = n - 2;
+  bool first = true;
+  while (b >= 0) {
+    int b_lo;
+    if (b < tile_bits)
+      b_lo = 0;
+    else {
+      int remaining = b - tile_bits + 1;  // stages above the last pass
+      int take = remaining > 7 ? (remaining > 14 ? 7 : (remaining + 1) / 2) : remaining;
+      b_lo = b - take + 1;
+    }
+    uint32_t grid = (uint32_t)(len >> tile_bits);
+    hipLaunchKernelGGL(ntt_pass_kernel, dim3(grid, ncols), dim3(BLOCK), 0, cx.stream,
+                       first ? d_messages : d_codewords, d_codewords, n, b, b_lo, tile_bits, dom->tw, lv, first ? 1 : 0,
+                       first ? len / 2 : len, len);
+    first = false;
+    b = b_lo - 1;
+  }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+// ------------------------------------------------------------------ codeword folding
+// pair (a, b) at twiddle x: f0 = (a + b)/2, f1 = (a - b)/(2x), out = f0 + r (f1 - f0)
+template <int D>
+__global__ __launch_bounds__(BLOCK) void rs_fold_kernel(const uint32_t *cw, const uint32_t *tw_inv2, uint32_t *out,
+                                                        uint64_t m, RoundArgs<D> args) {
+  uint64_t s = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (s >= m) return;
+  Ext<D> r;
+#pragma unroll
+  for (int c = 0; c < D; c++) r.c[c] = args.r_mont[c];
+  Ext<D> a = load_ext<D>(cw + 2 * s * D), b = load_ext<D>(cw + (2 * s + 1) * D);
+  Ext<D> f0 = ext_scale_mont<D>(ext_add<D>(a, b), mont_mul(INV2, R2));
+  Ext<D> f1 = ext_scale_mont<D>(ext_sub<D>(a, b), tw_inv2[s]);
+  store_ext<D>(out + s * D, ext_add<D>(f0, ext_mul_mont<D>(r, ext_sub<D>(f1, f0))));
+}
+
+static int rs_fold_launch(int D, uint64_t m, const uint32_t *tw_inv2_level, const uint32_t *d_cw, const uint32_t *r,
+                          uint32_t *d_out) {
+  Context &c = ctx();
+  uint32_t grid = (uint32_t)((m + BLOCK - 1) / BLOCK);
+  if (D == 4) {
+    RoundArgs<4> a;
+    memset(&a, 0, sizeof(a));
+    for (int k = 0; k < 4; k++) a.r_mont[k] = to_mont(r[k] % P);
+    hipLaunchKernelGGL(rs_fold_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, d_cw, tw_inv2_level, d_out, m, a);
+  } else {
+    RoundArgs<8> a;
+    memset(&a, 0, sizeof(a));
+    for (int k = 0; k < 8; k++) a.r_mont[k] = to_mont(r[k] % P);
+    hipLaunchKernelGGL(rs_fold_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, d_cw, tw_inv2_level, d_out, m, a);
+  }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d_cw, const uint32_t *r, uint32_t *d_out) {
+  int status = ctx().require();
+  if (status) return status;
+  Domain *dom;
+  if ((status = get_domain(n_domain, &dom))) return status;
+  return rs_fold_launch(D, m, dom->tw_inv2 + dom->off[level], d_cw, r, d_out);
+}
+
+// ------------------------------------------------------------------ Merkle trees
+// LEAF-DIGEST (src/pcs.lisp:44-52) of leaf l of ncols codewords: one row of 4 symbols per column,
+// rows hashed 64 at a time and chained h = BLAKE3(h || d).  A thread per leaf.
+__global__ __launch_bounds__(BLOCK) void leaf_kernel(const uint32_t *cw, int ncols, uint64_t cw_len, uint64_t nleaves,
+                                                     uint32_t *digests) {
+  uint64_t l = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (l >= nleaves) return;
+  uint32_t h[8], d[8], m[16];
+  bool have = false;
+  for (int start = 0; start < ncols; start += 64) {
+    int rows = ncols - start < 64 ? ncols - start : 64;
+    int nblocks = (rows + 3) / 4;
+    b3_iv(d);
+    for (int b = 0; b < nblocks; b++) {
+      int have_rows = rows - 4 * b < 4 ? rows - 4 * b : 4;
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (k < have_rows) v = *reinterpret_cast<const uint4 *>(cw + (uint64_t)(start + 4 * b + k) * cw_len + 4 * l);
+        m[4 * k] = v.x, m[4 * k + 1] = v.y, m[4 * k + 2] = v.z, m[4 * k + 3] = v.w;
+      }
+      uint32_t flags = (b == 0 ? B3_CHUNK_START : 0u) | (b == nblocks - 1 ? (B3_CHUNK_END | B3_ROOT) : 0u);
+      b3_compress(d, m, 0, (uint32_t)(16 * have_rows), flags, d, 0);
+    }
+    if (have)
+      b3_node(h, d, h);
+    else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) h[i] = d[i];
+      have = true;
+    }
+  }
+  uint4 *o = reinterpret_cast<uint4 *>(digests + l * 8);
+  o[0] = make_uint4(h[0], h[1], h[2], h[3]);
+  o[1] = make_uint4(h[4], h[5], h[6], h[7]);
+}
+
+// leaf l of an oracle codeword of EXT8s: one row per coordinate, symbols 4l..4l+3
+// (ORACLE-ROWS, src/pcs.lisp:577-579): 128 bytes, two blocks
+__global__ __launch_bounds__(BLOCK) void oracle_leaf_kernel(const uint32_t *cw, uint64_t nleaves, uint32_t *digests) {
+  uint64_t l = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (l >= nleaves) return;
+  uint32_t sym[4][8];
+#pragma unroll
+  for (int s = 0; s < 4; s++) {
+    Ext<8> e = load_ext<8>(cw + (4 * l + s) * 8);
+#pragma unroll
+    for (int d = 0; d < 8; d++) sym[s][d] = e.c[d];
+  }
+  uint32_t h[8], m[16];
+  b3_iv(h);
+#pragma unroll
+  for (int b = 0; b < 2; b++) {
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+#pragma unroll
+      for (int s = 0; s < 4; s++) m[4 * k + s] = sym[s][4 * b + k];
+    uint32_t flags = b == 0 ? B3_CHUNK_START : (B3_CHUNK_END | B3_ROOT);
+    b3_compress(h, m, 0, 64, flags, h, 0);
+  }
+  uint4 *o = reinterpret_cast<uint4 *>(digests + l * 8);
+  o[0] = make_uint4(h[0], h[1], h[2], h[3]);
+  o[1] = make_uint4(h[4], h[5], h[6], h[7]);
+}
+
+// one level of nodes: node = BLAKE3(left || right) (src/pcs.lisp:54-55, 64-77)
+__global__ __launch_bounds__(BLOCK) void node_kernel(const uint32_t *level, uint32_t *next, uint64_t n_next) {
+  uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (i >= n_next) return;
+  const uint4 *p = reinterpret_cast<const uint4 *>(level + 16 * i);
+  uint4 a = p[0], b = p[1], c = p[2], d = p[3];
+  uint32_t left[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w}, right[8] = {c.x, c.y, c.z, c.w, d.x, d.y, d.z, d.w}, h[8];
+  b3_node(left, right, h);
+  uint4 *o = reinterpret_cast<uint4 *>(next + 8 * i);
+  o[0] = make_uint4(h[0], h[1], h[2], h[3]);
+  o[1] = make_uint4(h[4], h[5], h[6], h[7]);
+}
+
+static int cap_level_of(uint64_t leaves) {  // src/pcs.lisp:57-59
+  int il = 0;
+  for (uint64_t v = leaves; v; v >>= 1) il++;
+  return il - 1 - 7 > 0 ? il - 1 - 7 : 0;
+}
+
+// the levels above the leaf digests already at d_levels; returns the cap
+static int merkle_levels_device(uint32_t *d_levels, uint64_t nleaves, uint8_t *cap, uint64_t *cap_rows) {
+  Context &c = ctx();
+  uint32_t *level = d_levels;
+  uint64_t n = nleaves;
+  int lc = cap_level_of(nleaves), l = 0;
+  const uint32_t *cap_ptr = d_levels;
+  while (n > 1) {
+    uint32_t *next = level + 8 * n;
+    uint32_t grid = (uint32_t)((n / 2 + BLOCK - 1) / BLOCK);
+    hipLaunchKernelGGL(node_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, level, next, n / 2);
+    level = next;
+    n /= 2;
+    l++;
+    if (l == lc) cap_ptr = level;
+  }
+  EXH_HIP(hipGetLastError());
+  *cap_rows = nleaves >> lc;
+  EXH_HIP(hipMemcpyAsync(cap, cap_ptr, 32 * *cap_rows, hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  return OK;
+}
+
+int merkle_commit_columns(const uint32_t *d_codewords, int ncols, int c, uint32_t *d_levels, uint8_t *cap,
+                          uint64_t *cap_rows) {
+  Context &cx = ctx();
+  int status = cx.require();
+  if (status) return status;
+  uint64_t nleaves = (uint64_t)1 << (c - 1), cw_len = (uint64_t)1 << (c + 1);
+  uint32_t grid = (uint32_t)((nleaves + BLOCK - 1) / BLOCK);
+  hipLaunchKernelGGL(leaf_kernel, dim3(grid), dim3(BLOCK), 0, cx.stream, d_codewords, ncols, cw_len, nleaves, d_levels);
+  return merkle_levels_device(d_levels, nleaves, cap, cap_rows);
+}
+
+// ------------------------------------------------------------------ BaseFold
+// DOT-PAIRS (src/pcs.lisp:473-483) for the three parities at once: sums over pairs of
+// pick(tt) pick(et), pick = even entry, odd entry, 2 odd - even.  Partials per workgroup.
+__global__ __launch_bounds__(BLOCK) void dot_pairs_kernel(const uint32_t *tt, const uint32_t *et, uint64_t n_pairs,
+                                                          uint32_t *partials) {
+  Acc96 acc[3][8];
+#pragma unroll
+  for (int k = 0; k < 3; k++)
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc_zero(acc[k][c]);
+  for (uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x; i < n_pairs; i += (uint64_t)gridDim.x * BLOCK) {
+    Ext<8> t0 = load_ext<8>(tt + 2 * i * 8), t1 = load_ext<8>(tt + (2 * i + 1) * 8);
+    Ext<8> e0 = load_ext<8>(et + 2 * i * 8), e1 = load_ext<8>(et + (2 * i + 1) * 8);
+    ext_mul_acc<8>(acc[0], t0, e0);
+    ext_mul_acc<8>(acc[1], t1, e1);
+    Ext<8> t2 = ext_sub<8>(ext_add<8>(t1, t1), t0), e2 = ext_sub<8>(ext_add<8>(e1, e1), e0);
+    ext_mul_acc<8>(acc[2], t2, e2);
+  }
+  __shared__ uint32_t lds[BLOCK / 64][24];
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < 3; k++)
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+      uint32_t v = wave_sum(acc_reduce(acc[k][c]));
+      if (lane == 0) lds[wave][k * 8 + c] = v;
+    }
+  __syncthreads();
+  if (threadIdx.x < 24) {
+    uint32_t v = lds[0][threadIdx.x];
+    for (int w = 1; w < BLOCK / 64; w++) v = fadd(v, lds[w][threadIdx.x]);
+    partials[(uint64_t)blockIdx.x * 24 + threadIdx.x] = v;
+  }
+}
+
+__global__ __launch_bounds__(BLOCK) void sum_columns_kernel(const uint32_t *partials, uint32_t nblocks, uint32_t width,
+                                                            uint32_t *sums) {
+  __shared__ uint32_t lds[BLOCK / 64];
+  uint32_t o = blockIdx.x, v = 0;
+  for (uint32_t b = threadIdx.x; b < nblocks; b += BLOCK) v = fadd(v, partials[(uint64_t)b * width + o]);
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < BLOCK / 64; w++) v = fadd(v, lds[w]);
+    sums[o] = v;
+  }
+}
+
+// FOLD-TABLE (src/field.lisp:365-370) of EXT8 tables
+__global__ __launch_bounds__(BLOCK) void fold8_kernel(const uint32_t *in, uint32_t *out, uint64_t n_out,
+                                                      RoundArgs<8> args) {
+  uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (i >= n_out) return;
+  Ext<8> r;
+#pragma unroll
+  for (int c = 0; c < 8; c++) r.c[c] = args.r_mont[c];
+  store_ext<8>(out + i * 8, fold_ext<8>(load_ext<8>(in + 2 * i * 8), load_ext<8>(in + (2 * i + 1) * 8), r));
+}
+
+// EXT8 table (entries x 8) <-> 8 coordinate columns, for ENCODE-EXT (src/pcs.lisp:569-575)
+__global__ __launch_bounds__(BLOCK) void split_coords_kernel(const uint32_t *table, uint32_t *cols, uint64_t len) {
+  uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (i >= len) return;
+  Ext<8> e = load_ext<8>(table + i * 8);
+#pragma unroll
+  for (int d = 0; d < 8; d++) cols[(uint64_t)d * len + i] = e.c[d];
+}
+__global__ __launch_bounds__(BLOCK) void join_coords_kernel(const uint32_t *cols, uint32_t *table, uint64_t len) {
+  uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (i >= len) return;
+  Ext<8> e;
+#pragma unroll
+  for (int d = 0; d < 8; d++) e.c[d] = cols[(uint64_t)d * len + i];
+  store_ext<8>(table + i * 8, e);
+}
+
+// eq(rr, x) for all x of nv bits as one table (weights of the BaseFold sumcheck)
+struct EqOne {
+  int bits;
+};
+__global__ __launch_bounds__(BLOCK) void eq8_kernel(const uint32_t *factors, int bits, uint32_t *out, uint64_t total) {
+  uint64_t x = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (x >= total) return;
+  Ext<8> e = ext_lift<8>(1);
+  for (int b = 0; b < bits; b++)
+    e = ext_mul_mont<8>(e, load_ext<8>(factors + ((size_t)b * 2 + (((x >> b) & 1) ? 0 : 1)) * 8));
+  store_ext<8>(out + x * 8, e);
+}
+
+// copy `count` segments of `words` words each from src + offsets[i] to out
+__global__ void gather_kernel(const uint32_t *src, const uint64_t *offsets, uint32_t words, uint32_t count,
+                              uint32_t *out) {
+  uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (uint64_t)words * count) return;
+  uint32_t seg = (uint32_t)(gid / words), w = (uint32_t)(gid % words);
+  out[gid] = src[offsets[seg] + w];
+}
+
+namespace {
+struct Owned {
+  std::vector<void *> ptrs;
+  ~Owned() {
+    for (void *p : ptrs) (void)hipFree(p);
+  }
+  uint32_t *alloc(uint64_t words) {
+    void *p = nullptr;
+    if (hipMalloc(&p, words ? words * 4 : 4) != hipSuccess) {
+      set_error("device-out-of-memory: BaseFold buffers");
+      return nullptr;
+    }
+    ptrs.push_back(p);
+    return (uint32_t *)p;
+  }
+};
+struct OracleTree {
+  int level;
+  uint32_t *cw, *levels;
+  uint64_t cw_len, nleaves;
+  int lc;
+};
+}  // namespace
+
+static int gather_to_host(const uint32_t *src, const std::vector<uint64_t> &offsets, uint32_t words,
+                          std::vector<uint32_t> *out) {
+  Context &c = ctx();
+  out->assign((size_t)offsets.size() * words, 0);
+  if (offsets.empty()) return OK;
+  uint64_t *d_off = nullptr;
+  uint32_t *d_out = nullptr;
+  EXH_HIP(hipMalloc((void **)&d_off, offsets.size() * 8));
+  EXH_HIP(hipMalloc((void **)&d_out, out->size() * 4));
+  EXH_HIP(hipMemcpy(d_off, offsets.data(), offsets.size() * 8, hipMemcpyHostToDevice));
+  uint64_t total = out->size();
+  hipLaunchKernelGGL(gather_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, c.stream, src, d_off, words,
+                     (uint32_t)offsets.size(), d_out);
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  EXH_HIP(hipMemcpy(out->data(), d_out, total * 4, hipMemcpyDeviceToHost));
+  EXH_HIP(hipFree(d_off));
+  EXH_HIP(hipFree(d_out));
+  return OK;
+}
+
+int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
+                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  const int fl = nv - 5 > 0 ? nv - 5 : 0;
+  const uint64_t len = (uint64_t)1 << nv;
+  Owned mem;
+  uint32_t *tt = mem.alloc(len * 8), *tt2 = mem.alloc(len * 4 + 8), *et = mem.alloc(len * 8),
+           *et2 = mem.alloc(len * 4 + 8), *cw = mem.alloc(2 * len * 8), *cw2 = mem.alloc(len * 8);
+  uint32_t *cols = mem.alloc(len * 8), *cwcols = mem.alloc(2 * len * 8);
+  const uint32_t max_grid = 1024;
+  uint32_t *partials = mem.alloc((uint64_t)max_grid * 24 + 24), *factors = mem.alloc((uint64_t)nv * 16 + 16);
+  if (!tt || !tt2 || !et || !et2 || !cw || !cw2 || !cols || !cwcols || !partials || !factors) return E_NOMEM;
+  uint32_t *sums = partials + (uint64_t)max_grid * 24;
+  uint32_t grid_len = (uint32_t)((len + BLOCK - 1) / BLOCK);
+  // tt = H, cw = ENCODE-EXT(H), et = eq-table(rr)
+  EXH_HIP(hipMemcpyAsync(tt, d_h, len * 32, hipMemcpyDeviceToDevice, c.stream));
+  hipLaunchKernelGGL(split_coords_kernel, dim3(grid_len), dim3(BLOCK), 0, c.stream, d_h, cols, len);
+  if ((status = rs_encode_columns(cols, 8, nv, cwcols))) return status;
+  hipLaunchKernelGGL(join_coords_kernel, dim3(2 * grid_len), dim3(BLOCK), 0, c.stream, cwcols, cw, 2 * len);
+  {
+    std::vector<uint32_t> f((size_t)nv * 16);
+    for (int b = 0; b < nv; b++)
+      for (int k = 0; k < 8; k++) {
+        uint32_t r = rr[(size_t)b * 8 + k] % P;
+        f[((size_t)b * 2) * 8 + k] = to_mont(r);
+        f[((size_t)b * 2 + 1) * 8 + k] = to_mont(fsub(k == 0 ? 1u : 0u, r));
+      }
+    EXH_HIP(hipMemcpy(factors, f.data(), f.size() * 4, hipMemcpyHostToDevice));
+    hipLaunchKernelGGL(eq8_kernel, dim3(grid_len), dim3(BLOCK), 0, c.stream, factors, nv, et, len);
+  }
+  EXH_HIP(hipGetLastError());
+  Domain *dom;
+  if ((status = get_domain(nv + 1, &dom))) return status;
+
+  hf::E prf = hf::lift(1, 8), claim = hf::from(v, 8);
+  std::vector<OracleTree> oracles;
+  for (int i = 0; i < fl; i++) {
+    uint64_t cur = len >> i, n_pairs = cur / 2;
+    uint32_t grid = (uint32_t)std::min<uint64_t>((n_pairs + BLOCK - 1) / BLOCK, max_grid);
+    hipLaunchKernelGGL(dot_pairs_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, tt, et, n_pairs, partials);
+    hipLaunchKernelGGL(sum_columns_kernel, dim3(24), dim3(BLOCK), 0, c.stream, partials, grid, 24u, sums);
+    uint32_t ev[24];
+    EXH_HIP(hipMemcpyAsync(ev, sums, 96, hipMemcpyDeviceToHost, c.stream));
+    EXH_HIP(hipStreamSynchronize(c.stream));
+    // every class has joined at level 0, so the a = prf * ysum term of the reference is zero
+    uint64_t dims[2] = {3, 8};
+    if ((status = tr.send(ev, 2, dims, nullptr))) return status;
+    if (hf::add(hf::from(ev, 8), hf::from(ev + 8, 8)) != claim) {
+      set_error("verification-failure: pcs: basefold sumcheck round " + std::to_string(i) + " failed");
+      return E_REJECT;
+    }
+    uint32_t x[8];
+    tr.challenge(8, x);
+    if (out_chal) memcpy(out_chal + 8 * i, x, 32);
+    claim = hf::lagrange({hf::from(ev, 8), hf::from(ev + 8, 8), hf::from(ev + 16, 8)}, hf::from(x, 8));
+    prf = hf::mul(prf, hf::eq1(hf::from(rr + 8 * i, 8), hf::from(x, 8)));
+    RoundArgs<8> a;
+    memset(&a, 0, sizeof(a));
+    for (int k = 0; k < 8; k++) a.r_mont[k] = to_mont(x[k]);
+    uint32_t gfold = (uint32_t)((n_pairs + BLOCK - 1) / BLOCK);
+    hipLaunchKernelGGL(fold8_kernel, dim3(gfold), dim3(BLOCK), 0, c.stream, tt, tt2, n_pairs, a);
+    hipLaunchKernelGGL(fold8_kernel, dim3(gfold), dim3(BLOCK), 0, c.stream, et, et2, n_pairs, a);
+    std::swap(tt, tt2);
+    std::swap(et, et2);
+    if ((status = rs_fold_launch(8, cur, dom->tw_inv2 + dom->off[i], cw, x, cw2))) return status;
+    std::swap(cw, cw2);
+    int l = i + 1;
+    if (l >= 2 && l < fl && l % 2 == 0) {  // an oracle tree over the folded codeword
+      OracleTree o;
+      o.level = l;
+      o.cw_len = cur;
+      o.nleaves = cur / 4;
+      o.lc = cap_level_of(o.nleaves);
+      o.cw = mem.alloc(cur * 8);
+      o.levels = mem.alloc((2 * o.nleaves) * 8);
+      if (!o.cw || !o.levels) return E_NOMEM;
+      EXH_HIP(hipMemcpyAsync(o.cw, cw, cur * 32, hipMemcpyDeviceToDevice, c.stream));
+      uint32_t gl = (uint32_t)((o.nleaves + BLOCK - 1) / BLOCK);
+      hipLaunchKernelGGL(oracle_leaf_kernel, dim3(gl), dim3(BLOCK), 0, c.stream, o.cw, o.nleaves, o.levels);
+      std::vector<uint8_t> cap(32 * 128);
+      uint64_t rows = 0;
+      if ((status = merkle_levels_device(o.levels, o.nleaves, cap.data(), &rows))) return status;
+      if ((status = tr.send_bytes(cap.data(), (int64_t)(32 * rows), nullptr))) return status;
+      oracles.push_back(o);
+    }
+  }
+  // the final table in the clear, the final claim, grinding, the query positions
+  uint64_t mlen = len >> fl;
+  std::vector<uint32_t> m(mlen * 8);
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  EXH_HIP(hipMemcpy(m.data(), tt, mlen * 32, hipMemcpyDeviceToHost));
+  uint64_t dims[2] = {mlen, 8};
+  if ((status = tr.send(m.data(), 2, dims, nullptr))) return status;
+  if (out_final) memcpy(out_final, m.data(), mlen * 32);
+  hf::E mval = fl < nv ? hf::mle_eval(m.data(), nv - fl, rr + 8 * fl, 8) : hf::from(m.data(), 8);
+  if (hf::mul(prf, mval) != claim) {
+    set_error("verification-failure: pcs: basefold final claim");
+    return E_REJECT;
+  }
+  tr.grind(grind_bits);
+  std::vector<uint64_t> qs(queries);
+  tr.challenge_bits(nv - 1, queries, qs.data());
+  if (out_qs) memcpy(out_qs, qs.data(), 8 * (size_t)queries);
+  for (const OracleTree &o : oracles) {  // the oracle openings, recorded (src/pcs.lisp:651-655)
+    std::vector<uint64_t> leaf_off, path_off;
+    for (int q = 0; q < queries; q++) {
+      uint64_t li = qs[q] >> o.level;
+      for (int s = 0; s < 4; s++) leaf_off.push_back((4 * li + s) * 8);
+      uint64_t level_start = 0, n = o.nleaves, idx = li;
+      for (int d = 0; d < o.lc; d++) {
+        path_off.push_back((level_start + (idx ^ 1)) * 8);
+        level_start += n;
+        n /= 2;
+        idx >>= 1;
+      }
+    }
+    std::vector<uint32_t> syms, path;
+    if ((status = gather_to_host(o.cw, leaf_off, 8, &syms))) return status;
+    if ((status = gather_to_host(o.levels, path_off, 8, &path))) return status;
+    std::vector<uint32_t> leaves((size_t)queries * 32);  // (Q, 8 rows, 4 symbols): row d holds coordinate d
+    for (int q = 0; q < queries; q++)
+      for (int d = 0; d < 8; d++)
+        for (int s = 0; s < 4; s++) leaves[((size_t)q * 8 + d) * 4 + s] = syms[((size_t)q * 4 + s) * 8 + d];
+    uint64_t d3[3] = {(uint64_t)queries, 8, 4};
+    if ((status = tr.send(leaves.data(), 3, d3, nullptr, false))) return status;
+    if ((status = tr.send_bytes((const uint8_t *)path.data(), (int64_t)path.size() * 4, nullptr, false))) return status;
+  }
+  return OK;
+}
+
+int basefold_verify(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,
+                    uint64_t *out_qs) {
+  const int fl = nv - 5 > 0 ? nv - 5 : 0;
+  int status;
+  hf::E prf = hf::lift(1, 8), claim = hf::from(v, 8);
+  for (int i = 0; i < fl; i++) {
+    uint32_t ev[24], x[8];
+    uint64_t dims[2] = {3, 8};
+    if ((status = tr.send(nullptr, 2, dims, ev))) return status;
+    if (hf::add(hf::from(ev, 8), hf::from(ev + 8, 8)) != claim) {
+      set_error("verification-failure: pcs: basefold sumcheck round " + std::to_string(i) + " failed");
+      return E_REJECT;
+    }
+    tr.challenge(8, x);
+    claim = hf::lagrange({hf::from(ev, 8), hf::from(ev + 8, 8), hf::from(ev + 16, 8)}, hf::from(x, 8));
+    prf = hf::mul(prf, hf::eq1(hf::from(rr + 8 * i, 8), hf::from(x, 8)));
+    int l = i + 1;
+    if (l >= 2 && l < fl && l % 2 == 0) {
+      uint64_t nleaves = ((uint64_t)1 << (nv + 1 - l)) / 4;
+      uint64_t rows = nleaves >> cap_level_of(nleaves);
+      if ((status = tr.send_bytes(nullptr, (int64_t)(32 * rows), nullptr))) return status;
+    }
+  }
+  uint64_t mlen = (uint64_t)1 << (nv - fl);
+  std::vector<uint32_t> m(mlen * 8);
+  uint64_t dims[2] = {mlen, 8};
+  if ((status = tr.send(nullptr, 2, dims, m.data()))) return status;
+  hf::E mval = fl < nv ? hf::mle_eval(m.data(), nv - fl, rr + 8 * fl, 8) : hf::from(m.data(), 8);
+  if (hf::mul(prf, mval) != claim) {
+    set_error("verification-failure: pcs: basefold final claim");
+    return E_REJECT;
+  }
+  uint64_t nonce;
+  if ((status = tr.verify_grind(grind_bits, &nonce))) return status;
+  std::vector<uint64_t> qs(queries);
+  tr.challenge_bits(nv - 1, queries, qs.data());
+  if (out_qs) memcpy(out_qs, qs.data(), 8 * (size_t)queries);
+  return OK;
+}
+
+}  // namespace exh

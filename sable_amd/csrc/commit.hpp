@@ -1,0 +1,25 @@
+// commit.hpp -- the commitment's data-parallel part on the device: rate-1/2 Reed-Solomon encoding
+// (src/rs.lisp:60-85), codeword folding (src/rs.lisp:93-101), BLAKE3 leaf digests and Merkle levels
+// with caps (src/pcs.lisp:44-77, 271-304) and the BaseFold loop (src/pcs.lisp:581-657).
+#pragma once
+#include <stdint.h>
+
+#include "transcript.hpp"
+
+namespace exh {
+
+// ncols messages of 2^c base values (contiguous) -> ncols codewords of 2^(c+1) symbols
+int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_codewords);
+// fold a codeword of 2m elements of degree D on level `level` of the 2^n_domain twiddle tables
+int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d_codeword, const uint32_t *r,
+                   uint32_t *d_out);
+// leaf digests and all Merkle levels (8-word digests, leaves first) of ncols codewords of
+// 2^(c+1) symbols; cap: the level max(0, log2(leaves) - 7), as bytes
+int merkle_commit_columns(const uint32_t *d_codewords, int ncols, int c, uint32_t *d_levels, uint8_t *cap,
+                          uint64_t *cap_rows);
+int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
+                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final);
+int basefold_verify(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,
+                    uint64_t *out_qs);
+
+}  // namespace exh

@@ -1,0 +1,90 @@
+// context.hip -- see context.hpp.
+#include "context.hpp"
+
+namespace exh {
+
+static Context g_ctx;
+Context &ctx() { return g_ctx; }
+
+int Arena::reserve(size_t need) {
+  if (need <= bytes) return OK;
+  if (ptr) {
+    hipError_t e = hipFree(ptr);
+    ptr = nullptr;
+    bytes = 0;
+    if (e != hipSuccess) {
+      set_error(std::string("device-error: hipFree: ") + hipGetErrorString(e));
+      return E_DEVICE;
+    }
+  }
+  size_t rounded = (need + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+  hipError_t e = hipMalloc(&ptr, rounded);
+  if (e != hipSuccess) {
+    ptr = nullptr;
+    set_error(std::string("device-out-of-memory: ") + std::to_string(rounded) + " bytes: " + hipGetErrorString(e));
+    return E_NOMEM;
+  }
+  bytes = rounded;
+  return OK;
+}
+
+void Arena::release() {
+  if (ptr) (void)hipFree(ptr);
+  ptr = nullptr;
+  bytes = 0;
+}
+
+int Context::require() {
+  if (!ready) {
+    set_error("device-error: the library is not initialised (exh_init), or no MI355X is visible");
+    return E_DEVICE;
+  }
+  return OK;
+}
+
+int ctx_init(int device) {
+  Context &c = g_ctx;
+  if (c.ready) return OK;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0) {
+    set_error(std::string("device-error: no HIP device: ") + (e == hipSuccess ? "count 0" : hipGetErrorString(e)));
+    return E_DEVICE;
+  }
+  if (device < 0 || device >= count) {
+    set_error("invalid-parameter: device index");
+    return E_PARAM;
+  }
+  EXH_HIP(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  EXH_HIP(hipGetDeviceProperties(&prop, device));
+  if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0) {
+    set_error(std::string("device-error: kernels are built for gfx950, found ") + prop.gcnArchName);
+    return E_DEVICE;
+  }
+  EXH_HIP(hipStreamCreate(&c.stream));
+  c.host_pinned_words = 1 << 16;
+  EXH_HIP(hipHostMalloc((void **)&c.host_pinned, c.host_pinned_words * 4, hipHostMallocDefault));
+  c.device = device;
+  c.ready = true;
+  return OK;
+}
+
+void ctx_shutdown() {
+  Context &c = g_ctx;
+  if (!c.ready) return;
+  (void)hipStreamSynchronize(c.stream);
+  for (auto &kv : c.tables)
+    if (kv.second.owned && kv.second.ptr) (void)hipFree(kv.second.ptr);
+  c.tables.clear();
+  c.fold_a.release();
+  c.fold_b.release();
+  c.misc.release();
+  if (c.host_pinned) (void)hipHostFree(c.host_pinned);
+  c.host_pinned = nullptr;
+  (void)hipStreamDestroy(c.stream);
+  c.stream = nullptr;
+  c.ready = false;
+}
+
+}  // namespace exh

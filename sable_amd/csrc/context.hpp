@@ -1,0 +1,56 @@
+// context.hpp -- the library's one device context: the HIP device and stream, device tables behind
+// opaque handles, and a grow-only workspace so the proving loop does not allocate per round.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "transcript.hpp"
+
+namespace exh {
+
+#define EXH_HIP(call)                                                                              \
+  do {                                                                                             \
+    hipError_t exh_err__ = (call);                                                                 \
+    if (exh_err__ != hipSuccess) {                                                                 \
+      ::exh::set_error(std::string("device-error: ") + #call + ": " + hipGetErrorString(exh_err__)); \
+      return ::exh::E_DEVICE;                                                                      \
+    }                                                                                              \
+  } while (0)
+
+struct DeviceTable {
+  uint32_t *ptr = nullptr;
+  uint64_t n_u32 = 0;
+  int stride = 1;     // 1: base values, D: extension elements
+  bool owned = true;  // allocated by the library (freed by exh_table_free)
+};
+
+// A device buffer that only grows; contents are scratch between calls.
+struct Arena {
+  void *ptr = nullptr;
+  size_t bytes = 0;
+  int reserve(size_t need);
+  void release();
+};
+
+struct Context {
+  bool ready = false;
+  int device = -1;
+  hipStream_t stream = nullptr;
+  std::map<uint64_t, DeviceTable> tables;
+  uint64_t next_handle = 1;
+  Arena fold_a, fold_b;  // the two generations of folded tables
+  Arena misc;            // weights, partial sums, small results
+  uint32_t *host_pinned = nullptr;  // small pinned buffer for per-round results
+  size_t host_pinned_words = 0;
+  int require();  // OK, or E_DEVICE with the reason when the library is not initialised
+};
+
+Context &ctx();
+int ctx_init(int device);
+void ctx_shutdown();
+
+}  // namespace exh

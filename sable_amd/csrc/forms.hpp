@@ -1,0 +1,63 @@
+// forms.hpp -- statements as data: the s-expression forms of the reference (src/forms.lisp) parsed,
+// expanded into the canonical sum of monomials, and compiled into the table-monomial groups the
+// round kernels are generated from.
+#pragma once
+#include <stdint.h>
+
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace exh {
+
+struct Term {  // coefficient * product of variables (names upper-cased, sorted)
+  std::vector<std::string> vars;
+  uint32_t coeff;
+};
+
+// EXPAND (src/forms.lisp:57-78): like terms merged, zero terms dropped, graded order.
+// Returns OK or E_PARAM (malformed form; message in last_error()).
+int expand_form(const std::string &text, std::vector<Term> *out);
+
+// One group of a compiled statement: a multiset of tables with the constant-side of every term
+// over it, so that  statement = sum_g coefficient_g(constants) * prod_{t in g} table_t.
+struct Group {
+  std::vector<int> tabs;  // table indices, sorted; empty: the constant group
+  struct Part {
+    uint32_t coeff;
+    std::vector<int> consts;  // constant indices (with repetition)
+  };
+  std::vector<Part> parts;
+  // evaluation points of the group's round polynomial computed on the device (X values); the host
+  // extrapolates to the wire points when the group's degree is below the statement's
+  std::vector<int> evalx;
+  int acc_base = 0;  // index of its first accumulator
+};
+
+struct Statement {
+  std::string text;
+  std::vector<std::string> tables, constants;
+  std::vector<Term> terms;
+  int degree = 0;  // in the tables (src/sumcheck.lisp:33-35)
+  int T() const { return (int)tables.size(); }
+  int C() const { return (int)constants.size(); }
+  std::vector<Group> groups;  // constant group (if any) included
+  int nacc = 0;               // accumulators per round over all groups
+  // the device evaluation points are chosen for POINTS = max(header degree, 1) wire points
+  void plan(int points);
+  // every group at X = 0 and X = 1 only: what the honest claim (HYPERCUBE-SUM) needs
+  void plan_claim();
+  int planned_points = -1;
+  std::string key() const;  // canonical description of the table groups, for kernel lookup
+};
+
+int compile_statement(const std::string &text, const std::vector<std::string> &tables,
+                      const std::vector<std::string> &constants, Statement *out);
+
+// the statement over F_p^D at the given table and constant values (exact, host side)
+void evaluate_statement(const Statement &st, int D, const uint32_t *table_vals, const uint32_t *const_vals,
+                        uint32_t *out);
+// the groups' coefficients at the constants: out[g*D .. g*D+D)
+void group_coefficients(const Statement &st, int D, const uint32_t *const_vals, uint32_t *out);
+
+}  // namespace exh

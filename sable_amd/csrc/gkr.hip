@@ -1,0 +1,425 @@
+// gkr.hip -- see gkr.hpp.
+#include "gkr.hpp"
+
+#include <string.h>
+
+#include <vector>
+
+#include "context.hpp"
+#include "forms.hpp"
+#include "hostfield.hpp"
+#include "prover.hpp"
+#include "sumcheck_kernels.cuh"
+
+namespace exh {
+
+// parent (b, x) of children (b, x) and (b, x + 2^m): p = p0 q1 + p1 q0, q = q0 q1
+template <int D>
+__global__ __launch_bounds__(BLOCK) void gkr_reduce_kernel(const uint32_t *p, const uint32_t *q, uint32_t *pp,
+                                                           uint32_t *qq, uint32_t m, uint64_t n_out) {
+  uint64_t o = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (o >= n_out) return;
+  uint64_t half = (uint64_t)1 << m, b = o >> m, x = o & (half - 1);
+  uint64_t c0 = (b << (m + 1)) + x, c1 = c0 + half;
+  Ext<D> p0 = load_ext<D>(p + c0 * D), p1 = load_ext<D>(p + c1 * D);
+  Ext<D> q0 = load_ext<D>(q + c0 * D), q1 = load_ext<D>(q + c1 * D);
+  // products carry 1/R; multiplying one factor of each product by R^2 first makes them exact
+  Ext<D> q1r, q0r;
+#pragma unroll
+  for (int c = 0; c < D; c++) q1r.c[c] = mont_mul(q1.c[c], R2), q0r.c[c] = mont_mul(q0.c[c], R2);
+  store_ext<D>(pp + o * D, ext_add<D>(ext_mul_mont<D>(p0, q1r), ext_mul_mont<D>(p1, q0r)));
+  store_ext<D>(qq + o * D, ext_mul_mont<D>(q0, q1r));
+}
+
+int gkr_reduce_layer(int D, int K, int m, const uint32_t *p, const uint32_t *q, uint32_t *pp, uint32_t *qq) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  uint64_t n_out = (uint64_t)K << m;
+  uint32_t grid = (uint32_t)((n_out + BLOCK - 1) / BLOCK);
+  if (D == 4)
+    hipLaunchKernelGGL(gkr_reduce_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, p, q, pp, qq, (uint32_t)m, n_out);
+  else
+    hipLaunchKernelGGL(gkr_reduce_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, p, q, pp, qq, (uint32_t)m, n_out);
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+// the lower and upper halves of each block, as K contiguous blocks each (HALVES-PER-BLOCK,
+// src/gkr.lisp:190-197); only needed when K > 1: with one block the halves are views
+template <int D>
+__global__ __launch_bounds__(BLOCK) void halves_kernel(const uint32_t *v, uint32_t *lower, uint32_t *upper,
+                                                       uint32_t size_bits, uint64_t n_out) {
+  uint64_t o = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (o >= n_out) return;
+  uint64_t size = (uint64_t)1 << size_bits, b = o >> size_bits, x = o & (size - 1);
+  store_ext<D>(lower + o * D, load_ext<D>(v + (b * 2 * size + x) * D));
+  store_ext<D>(upper + o * D, load_ext<D>(v + (b * 2 * size + size + x) * D));
+}
+
+namespace {
+
+int block_bits(int k) {  // src/gkr.lisp:23-25
+  int b = 0;
+  for (int v = k - 1; v > 0; v >>= 1) b++;
+  return b;
+}
+
+// LAYER-STATEMENT (src/gkr.lisp:30-41) as a form; with_bw: (* bw statement)
+Statement layer_statement(int lookups, bool with_bw) {
+  std::string form = "(+";
+  std::vector<std::string> tables, constants;
+  if (with_bw) tables.push_back("BW");
+  for (int l = 0; l < lookups; l++) {
+    std::string s = std::to_string(l);
+    form += " (* A" + s + " P0-" + s + " Q1-" + s + ") (* A" + s + " P1-" + s + " Q0-" + s + ") (* AL" + s + " Q0-" + s +
+            " Q1-" + s + ")";
+    for (const char *name : {"P0-", "P1-", "Q0-", "Q1-"}) tables.push_back(name + s);
+    constants.push_back("A" + s);
+    constants.push_back("AL" + s);
+  }
+  form += ")";
+  if (with_bw) form = "(* BW " + form + ")";
+  Statement st;
+  compile_statement(form, tables, constants, &st);
+  return st;
+}
+
+// a_l for each lookup from one challenge stream, then lambda; constants a_l, a_l lambda (:43-51)
+void layer_challenges(Transcript &tr, int D, int L, std::vector<uint32_t> &consts, std::vector<hf::E> &as,
+                      hf::E &lam) {
+  std::vector<uint32_t> raw((size_t)L * D);
+  tr.challenges(L, D, raw.data());
+  lam.assign(D, 0);
+  tr.challenge(D, lam.data());
+  consts.assign((size_t)2 * L * D, 0);
+  as.clear();
+  for (int l = 0; l < L; l++) {
+    hf::E a(raw.begin() + (size_t)l * D, raw.begin() + (size_t)(l + 1) * D);
+    hf::E al = hf::mul(a, lam);
+    memcpy(&consts[(size_t)(2 * l) * D], a.data(), 4 * D);
+    memcpy(&consts[(size_t)(2 * l + 1) * D], al.data(), 4 * D);
+    as.push_back(a);
+  }
+}
+
+hf::E layer_claim(int D, const std::vector<hf::E> &as, const hf::E &lam, const std::vector<hf::E> &cp,
+                  const std::vector<hf::E> &cq) {  // :53-55
+  hf::E acc = hf::zero(D);
+  for (size_t l = 0; l < as.size(); l++) acc = hf::add(acc, hf::mul(as[l], hf::add(cp[l], hf::mul(lam, cq[l]))));
+  return acc;
+}
+
+hf::E fold_pair(const hf::E &lo, const hf::E &hi, const hf::E &r) { return hf::add(lo, hf::mul(r, hf::sub(hi, lo))); }
+
+void next_claims(int D, int L, const uint32_t *finals, const hf::E &tt, std::vector<hf::E> &cp,
+                 std::vector<hf::E> &cq) {  // :57-63
+  for (int l = 0; l < L; l++) {
+    const uint32_t *f = finals + (size_t)(4 * l) * D;
+    cp[l] = fold_pair(hf::from(f, D), hf::from(f + D, D), tt);
+    cq[l] = fold_pair(hf::from(f + 2 * D, D), hf::from(f + 3 * D, D), tt);
+  }
+}
+
+hf::E padded_mass(int D, int lk, int K, const std::vector<uint32_t> &rb) {  // :68-71
+  std::vector<uint32_t> e = hf::eq_table(rb.data(), lk, D);
+  hf::E mass = hf::zero(D);
+  for (size_t b = K; b < ((size_t)1 << lk); b++) mass = hf::add(mass, hf::from(&e[b * D], D));
+  return mass;
+}
+
+std::vector<uint32_t> block_weights(int D, int K, const std::vector<uint32_t> &rb) {  // :73-77
+  if (rb.empty()) {
+    std::vector<uint32_t> one((size_t)D, 0);
+    one[0] = 1;
+    return one;
+  }
+  std::vector<uint32_t> e = hf::eq_table(rb.data(), (int)(rb.size() / D), D);
+  e.resize((size_t)K * D);
+  return e;
+}
+
+int send_finals(Transcript &tr, int D, int ntables, const uint32_t *finals, hf::E &tt) {  // :208-213
+  uint64_t dims[2] = {1, (uint64_t)D};
+  for (int t = 0; t < ntables; t++) {
+    int status = tr.send(finals + (size_t)t * D, 2, dims, nullptr);
+    if (status) return status;
+  }
+  tt.assign(D, 0);
+  tr.challenge(D, tt.data());
+  return OK;
+}
+
+struct DeviceBuffers {  // frees what it allocated when the proof ends
+  std::vector<void *> owned;
+  ~DeviceBuffers() {
+    for (void *p : owned) (void)hipFree(p);
+  }
+  uint32_t *alloc(uint64_t words) {
+    void *p = nullptr;
+    if (hipMalloc(&p, words ? words * 4 : 4) != hipSuccess) return nullptr;
+    owned.push_back(p);
+    return (uint32_t *)p;
+  }
+};
+
+}  // namespace
+
+int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *leaves, const std::string &label,
+                    uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp, uint32_t *out_cq) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  int D = tr.D, lk = block_bits(K), NT = 4 * L;
+  if (L < 1 || NT + 1 > MAXT || n < 0 || n > 30 || K < 1) {
+    set_error("invalid-parameter: GKR shape");
+    return E_PARAM;
+  }
+  uint64_t Kp = (uint64_t)1 << lk;
+  DeviceBuffers bufs;
+  // FRACTION-TREES: every in-block layer, bottom up, kept on the device
+  std::vector<std::vector<const uint32_t *>> layers(n + 1, std::vector<const uint32_t *>(2 * L));
+  for (int i = 0; i < 2 * L; i++) layers[n][i] = leaves[i];
+  for (int m = n - 1; m >= 0; m--)
+    for (int l = 0; l < L; l++) {
+      uint64_t words = ((uint64_t)K << m) * D;
+      uint32_t *pp = bufs.alloc(words), *qq = bufs.alloc(words);
+      if (!pp || !qq) {
+        set_error("device-out-of-memory: GKR layers");
+        return E_NOMEM;
+      }
+      if ((status = gkr_reduce_layer(D, K, m, layers[m + 1][2 * l], layers[m + 1][2 * l + 1], pp, qq))) return status;
+      layers[m][2 * l] = pp;
+      layers[m][2 * l + 1] = qq;
+    }
+  // the per-block roots, and the top tree over the block index on the host (2^lk entries)
+  std::vector<std::vector<std::vector<uint32_t>>> top(lk + 1, std::vector<std::vector<uint32_t>>(2 * L));
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  for (int l = 0; l < L; l++) {
+    std::vector<uint32_t> p(Kp * D, 0), q(Kp * D, 0);
+    EXH_HIP(hipMemcpy(p.data(), layers[0][2 * l], (size_t)K * D * 4, hipMemcpyDeviceToHost));
+    EXH_HIP(hipMemcpy(q.data(), layers[0][2 * l + 1], (size_t)K * D * 4, hipMemcpyDeviceToHost));
+    for (uint64_t b = K; b < Kp; b++) q[b * D] = 1;  // padded with 0/1
+    top[lk][2 * l] = p;
+    top[lk][2 * l + 1] = q;
+  }
+  for (int j = lk - 1; j >= 0; j--)
+    for (int l = 0; l < L; l++) {
+      uint64_t len = (uint64_t)1 << j;
+      const std::vector<uint32_t> &p = top[j + 1][2 * l], &q = top[j + 1][2 * l + 1];
+      std::vector<uint32_t> pp(len * D), qq(len * D);
+      for (uint64_t b = 0; b < len; b++) {
+        hf::E p0 = hf::from(&p[b * D], D), p1 = hf::from(&p[(b + len) * D], D);
+        hf::E q0 = hf::from(&q[b * D], D), q1 = hf::from(&q[(b + len) * D], D);
+        hf::E np = hf::add(hf::mul(p0, q1), hf::mul(p1, q0)), nq = hf::mul(q0, q1);
+        memcpy(&pp[b * D], np.data(), 4 * D);
+        memcpy(&qq[b * D], nq.data(), 4 * D);
+      }
+      top[j][2 * l] = pp;
+      top[j][2 * l + 1] = qq;
+    }
+
+  Statement st = layer_statement(L, false), st_blk = layer_statement(L, true);
+  std::vector<hf::E> cp(L), cq(L), as;
+  hf::E lam, tt;
+  std::vector<uint32_t> consts, finals((size_t)(NT + 1) * D), rho((size_t)(n + lk + 1) * D);
+  std::vector<uint32_t> r, ri;
+  uint64_t dims2[2] = {2, (uint64_t)D};
+  for (int l = 0; l < L; l++) {  // the roots
+    uint32_t root[16];
+    memcpy(root, top[0][2 * l].data(), 4 * D);
+    memcpy(root + D, top[0][2 * l + 1].data(), 4 * D);
+    if ((status = tr.send(root, 2, dims2, nullptr))) return status;
+    cp[l] = hf::from(root, D);
+    cq[l] = hf::from(root + D, D);
+  }
+  std::vector<int> strides(NT + 1, D);
+  for (int j = 0; j < lk; j++) {  // the top tree
+    layer_challenges(tr, D, L, consts, as, lam);
+    uint64_t size = (uint64_t)1 << j;
+    std::vector<const uint32_t *> tabs(NT);
+    for (int l = 0; l < L; l++)
+      for (int w = 0; w < 2; w++) {
+        uint32_t *d = bufs.alloc(2 * size * D);
+        if (!d) return E_NOMEM;
+        EXH_HIP(hipMemcpy(d, top[j + 1][2 * l + w].data(), 2 * size * D * 4, hipMemcpyHostToDevice));
+        tabs[4 * l + 2 * w] = d;                 // lower half: children b
+        tabs[4 * l + 2 * w + 1] = d + size * D;  // upper half: children b + 2^j
+      }
+    status = sumcheck_prove(tr, j, st, tabs.data(), strides.data(), j > 0 ? r.data() : nullptr, consts.data(),
+                            label + "-top", nullptr, 1, j > 0 ? 2 : 0, rho.data(), finals.data(), nullptr);
+    if (status) return status;
+    if ((status = send_finals(tr, D, NT, finals.data(), tt))) return status;
+    next_claims(D, L, finals.data(), tt, cp, cq);
+    r.assign(rho.begin(), rho.begin() + (size_t)j * D);
+    r.insert(r.end(), tt.begin(), tt.end());
+  }
+  std::vector<uint32_t> rb = r;
+  if (Kp != (uint64_t)K) {
+    hf::E mass = padded_mass(D, lk, K, rb);
+    for (int l = 0; l < L; l++) cq[l] = hf::sub(cq[l], mass);
+  }
+  for (int layer = 0; layer < n - 1; layer++) {  // the in-block layers
+    layer_challenges(tr, D, L, consts, as, lam);
+    std::vector<uint32_t> bw = block_weights(D, K, rb);
+    uint64_t size = (uint64_t)1 << layer;
+    std::vector<const uint32_t *> tabs(NT);
+    for (int l = 0; l < L; l++)
+      for (int w = 0; w < 2; w++) {
+        const uint32_t *v = layers[layer + 1][2 * l + w];
+        if (K == 1) {  // the halves are views
+          tabs[4 * l + 2 * w] = v;
+          tabs[4 * l + 2 * w + 1] = v + size * D;
+        } else {
+          uint32_t *lo = bufs.alloc(K * size * D), *hi = bufs.alloc(K * size * D);
+          if (!lo || !hi) return E_NOMEM;
+          uint64_t n_out = K * size;
+          uint32_t grid = (uint32_t)((n_out + BLOCK - 1) / BLOCK);
+          if (D == 4)
+            hipLaunchKernelGGL(halves_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, v, lo, hi, (uint32_t)layer,
+                               n_out);
+          else
+            hipLaunchKernelGGL(halves_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, v, lo, hi, (uint32_t)layer,
+                               n_out);
+          tabs[4 * l + 2 * w] = lo;
+          tabs[4 * l + 2 * w + 1] = hi;
+        }
+      }
+    std::vector<std::vector<uint32_t>> folded(NT, std::vector<uint32_t>(Kp * D, 0));  // zero padded to 2^lk
+    std::vector<uint32_t *> fptr(NT);
+    for (int t = 0; t < NT; t++) fptr[t] = folded[t].data();
+    status = sumcheck_prove(tr, layer, st, tabs.data(), strides.data(), layer > 0 ? ri.data() : nullptr,
+                            consts.data(), label, bw.data(), K, layer > 0 ? 2 : 0, rho.data(), finals.data(),
+                            fptr.data());
+    if (status) return status;
+    std::vector<uint32_t> rbn;
+    if (lk > 0) {  // bind the block index: the blocks' values and weights, padded with zeros
+      std::vector<const uint32_t *> btabs(NT + 1);
+      std::vector<uint32_t> bwp(Kp * D, 0);
+      memcpy(bwp.data(), bw.data(), (size_t)K * D * 4);
+      for (int t = 0; t <= NT; t++) {
+        uint32_t *d = bufs.alloc(Kp * D);
+        if (!d) return E_NOMEM;
+        EXH_HIP(hipMemcpy(d, t == 0 ? bwp.data() : folded[t - 1].data(), Kp * D * 4, hipMemcpyHostToDevice));
+        btabs[t] = d;
+      }
+      std::vector<uint32_t> f2((size_t)(NT + 1) * D);
+      rbn.assign((size_t)lk * D, 0);
+      status = sumcheck_prove(tr, lk, st_blk, btabs.data(), strides.data(), nullptr, consts.data(), label + "-blk",
+                              nullptr, 1, -1, rbn.data(), f2.data(), nullptr);
+      if (status) return status;
+      memcpy(finals.data(), f2.data() + D, (size_t)NT * D * 4);  // bw's final comes first
+    }
+    if ((status = send_finals(tr, D, NT, finals.data(), tt))) return status;
+    next_claims(D, L, finals.data(), tt, cp, cq);
+    ri.assign(rho.begin(), rho.begin() + (size_t)layer * D);
+    ri.insert(ri.end(), tt.begin(), tt.end());
+    rb = rbn;
+  }
+  if (out_ri && !ri.empty()) memcpy(out_ri, ri.data(), ri.size() * 4);
+  if (out_rb && !rb.empty()) memcpy(out_rb, rb.data(), rb.size() * 4);
+  for (int l = 0; l < L; l++) {
+    if (out_cp) memcpy(out_cp + (size_t)l * D, cp[l].data(), 4 * D);
+    if (out_cq) memcpy(out_cq + (size_t)l * D, cq[l].data(), 4 * D);
+  }
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  return OK;
+}
+
+int gkr_verify_upper(Transcript &tr, int n, int K, int L, const std::string &label, uint32_t *out_roots,
+                     uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp, uint32_t *out_cq) {
+  int D = tr.D, lk = block_bits(K), NT = 4 * L, status;
+  if (L < 1 || NT + 1 > MAXT || n < 0 || K < 1) {
+    set_error("invalid-parameter: GKR shape");
+    return E_PARAM;
+  }
+  uint64_t Kp = (uint64_t)1 << lk;
+  std::vector<hf::E> cp(L), cq(L), as;
+  hf::E lam, tt;
+  uint64_t dims2[2] = {2, (uint64_t)D}, dims1[2] = {1, (uint64_t)D};
+  for (int l = 0; l < L; l++) {
+    uint32_t root[16];
+    if ((status = tr.send(nullptr, 2, dims2, root))) return status;
+    if (out_roots) memcpy(out_roots + (size_t)l * 2 * D, root, 8 * D);
+    cp[l] = hf::from(root, D);
+    cq[l] = hf::from(root + D, D);
+  }
+  Statement st = layer_statement(L, false), st_blk = layer_statement(L, true);
+  std::vector<uint32_t> consts, finals((size_t)NT * D), rho((size_t)(n + lk + 1) * D), r, ri, rb;
+  uint32_t reduced[8], expected[8];
+  auto receive_finals = [&]() -> int {  // :84-89
+    for (int t = 0; t < NT; t++) {
+      int s = tr.send(nullptr, 2, dims1, &finals[(size_t)t * D]);
+      if (s) return s;
+    }
+    tt.assign(D, 0);
+    tr.challenge(D, tt.data());
+    return OK;
+  };
+  for (int j = 0; j < lk; j++) {  // the top tree
+    layer_challenges(tr, D, L, consts, as, lam);
+    hf::E claim = layer_claim(D, as, lam, cp, cq);
+    if ((status = sumcheck_verify(tr, j, st, claim.data(), j > 0 ? r.data() : nullptr, consts.data(), 1,
+                                  label + "-top", j > 0 ? 2 : 0, rho.data(), reduced)))
+      return status;
+    if ((status = receive_finals())) return status;
+    evaluate_statement(st, D, finals.data(), consts.data(), expected);
+    if (memcmp(reduced, expected, 4 * D)) {
+      set_error("verification-failure: gkr-top: layer " + std::to_string(j) + " of the top tree");
+      return E_REJECT;
+    }
+    next_claims(D, L, finals.data(), tt, cp, cq);
+    r.assign(rho.begin(), rho.begin() + (size_t)j * D);
+    r.insert(r.end(), tt.begin(), tt.end());
+  }
+  rb = r;
+  if (Kp != (uint64_t)K) {
+    hf::E mass = padded_mass(D, lk, K, rb);
+    for (int l = 0; l < L; l++) cq[l] = hf::sub(cq[l], mass);
+  }
+  for (int layer = 0; layer < n - 1; layer++) {  // the in-block layers
+    layer_challenges(tr, D, L, consts, as, lam);
+    std::vector<uint32_t> bw = block_weights(D, K, rb);
+    hf::E claim = layer_claim(D, as, lam, cp, cq);
+    if ((status = sumcheck_verify(tr, layer, st, claim.data(), layer > 0 ? ri.data() : nullptr, consts.data(), K,
+                                  label, layer > 0 ? 2 : 0, rho.data(), reduced)))
+      return status;
+    std::vector<uint32_t> rbn;
+    if (lk > 0) {
+      rbn.assign((size_t)lk * D, 0);
+      uint32_t red2[8];
+      if ((status = sumcheck_verify(tr, lk, st_blk, reduced, nullptr, consts.data(), 1, label + "-blk", -1,
+                                    rbn.data(), red2)))
+        return status;
+      memcpy(reduced, red2, 4 * D);
+    }
+    if ((status = receive_finals())) return status;
+    hf::E weight = hf::zero(D);
+    if (K > 1) {  // sum_b bw_b eq(rbn, b)
+      std::vector<uint32_t> e = hf::eq_table(rbn.data(), lk, D);
+      for (int b = 0; b < K; b++)
+        weight = hf::add(weight, hf::mul(hf::from(&bw[(size_t)b * D], D), hf::from(&e[(size_t)b * D], D)));
+    } else {
+      weight = hf::from(bw.data(), D);
+    }
+    evaluate_statement(st, D, finals.data(), consts.data(), expected);
+    hf::E want = hf::mul(weight, hf::from(expected, D));
+    if (memcmp(reduced, want.data(), 4 * D)) {
+      set_error("verification-failure: gkr-layer: in-block layer " + std::to_string(layer));
+      return E_REJECT;
+    }
+    next_claims(D, L, finals.data(), tt, cp, cq);
+    ri.assign(rho.begin(), rho.begin() + (size_t)layer * D);
+    ri.insert(ri.end(), tt.begin(), tt.end());
+    rb = rbn;
+  }
+  if (out_ri && !ri.empty()) memcpy(out_ri, ri.data(), ri.size() * 4);
+  if (out_rb && !rb.empty()) memcpy(out_rb, rb.data(), rb.size() * 4);
+  for (int l = 0; l < L; l++) {
+    if (out_cp) memcpy(out_cp + (size_t)l * D, cp[l].data(), 4 * D);
+    if (out_cq) memcpy(out_cq + (size_t)l * D, cq[l].data(), 4 * D);
+  }
+  return OK;
+}
+
+}  // namespace exh

@@ -1,0 +1,104 @@
+// prover.cpp -- see prover.hpp.
+#include "prover.hpp"
+
+#include <string.h>
+
+#include "hostfield.hpp"
+
+namespace exh {
+
+// label | n u16 | degree u16 | blocks u32, little-endian (src/sumcheck.lisp:24-27)
+void absorb_header(Transcript &tr, const std::string &label, int n, int degree, int blocks) {
+  std::string h = label + "|";
+  h.push_back((char)(n & 0xff)), h.push_back((char)((n >> 8) & 0xff));
+  h.push_back((char)(degree & 0xff)), h.push_back((char)((degree >> 8) & 0xff));
+  for (int i = 0; i < 4; i++) h.push_back((char)(((uint32_t)blocks >> (8 * i)) & 0xff));
+  tr.absorb((const uint8_t *)h.data(), h.size());
+}
+
+int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables, const int *strides,
+                   const uint32_t *eq, const uint32_t *consts, const std::string &label, const uint32_t *bw, int K,
+                   int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded) {
+  int D = tr.D;
+  if (degree < 0) degree = st.degree;
+  int points = degree > 1 ? degree : 1;
+  SumcheckSession s;
+  int status = s.begin(st, D, n, d_tables, strides, eq, bw, K, consts, degree);
+  if (status) return status;
+  absorb_header(tr, label, n, degree, bw ? K : 1);
+  uint32_t sums[16 * 8];
+  for (int j = 0; j < n; j++) {
+    if ((status = s.round_sums(sums))) return status;
+    uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
+    if ((status = tr.send(sums, 2, dims, nullptr))) return status;
+    uint32_t *r = out_chal + (size_t)j * D;
+    tr.challenge(D, r);
+    if ((status = s.fold(r))) return status;
+  }
+  return s.finish(out_finals, out_folded);
+}
+
+// g(X) at x from the message (g at 0, 2, 3, ...) and the claim, which gives g(1)
+// (NEXT-CLAIM, src/sumcheck.lisp:137-145)
+static int next_claim(int D, int points, hf::E &claim, const uint32_t *message, const uint32_t *eq_rj,
+                      const uint32_t *x) {
+  std::vector<hf::E> vals;
+  hf::E g0 = hf::from(message, D), g1;
+  if (eq_rj) {  // claim = (1 - r) g(0) + r g(1)
+    hf::E r = hf::from(eq_rj, D);
+    if (hf::is_zero(r)) {
+      set_error("field-division-by-zero: ext-inv of the eq point's coordinate");
+      return E_DIVZERO;
+    }
+    g1 = hf::mul(hf::sub(claim, hf::mul(hf::sub(hf::lift(1, D), r), g0)), hf::inv(r));
+  } else {
+    g1 = hf::sub(claim, g0);
+  }
+  vals.push_back(g0);
+  vals.push_back(g1);
+  for (int k = 1; k < points; k++) vals.push_back(hf::from(message + (size_t)k * D, D));
+  claim = hf::lagrange(vals, hf::from(x, D));
+  return OK;
+}
+
+int sumcheck_verify(Transcript &tr, int n, const Statement &st, const uint32_t *claim_in, const uint32_t *eq,
+                    const uint32_t *consts, int blocks, const std::string &label, int degree, uint32_t *out_chal,
+                    uint32_t *out_reduced) {
+  (void)consts;
+  int D = tr.D;
+  if (degree < 0) degree = st.degree;
+  int points = degree > 1 ? degree : 1;
+  if (points > 16) {
+    set_error("invalid-parameter: degree");
+    return E_PARAM;
+  }
+  hf::E claim(D);
+  for (int k = 0; k < D; k++) claim[k] = claim_in[k] % P;
+  absorb_header(tr, label, n, degree, blocks);
+  for (int j = 0; j < n; j++) {
+    uint32_t message[16 * 8];
+    uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
+    int status = tr.send(nullptr, 2, dims, message);
+    if (status) {
+      set_error(status == E_EXHAUSTED ? "transcript-exhausted: round message" : "message-shape-error: round message");
+      return status;
+    }
+    uint32_t *r = out_chal + (size_t)j * D;
+    tr.challenge(D, r);
+    if ((status = next_claim(D, points, claim, message, eq ? eq + (size_t)j * D : nullptr, r))) return status;
+  }
+  memcpy(out_reduced, claim.data(), 4 * D);
+  return OK;
+}
+
+int check_final(const Statement &st, int D, const uint32_t *reduced, const uint32_t *finals, const uint32_t *consts) {
+  uint32_t expected[8];
+  evaluate_statement(st, D, finals, consts, expected);
+  if (memcmp(expected, reduced, 4 * D) != 0) {
+    set_error("verification-failure: sumcheck-final: reduced claim differs from the statement at the final values");
+    return E_REJECT;
+  }
+  return OK;
+}
+
+}  // namespace exh

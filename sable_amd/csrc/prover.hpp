@@ -1,0 +1,24 @@
+// prover.hpp -- the host side of the protocols over the device sessions: PROVE / VERIFY / CHECK-FINAL
+// of the sumcheck with the reference's argument meaning (src/sumcheck.lisp:131-172, 512-571).
+#pragma once
+#include <stdint.h>
+
+#include <string>
+
+#include "forms.hpp"
+#include "sumcheck.hpp"
+#include "transcript.hpp"
+
+namespace exh {
+
+// tables: device pointers, K * 2^n entries of stride 1 or D each, block-major.
+int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables, const int *strides,
+                   const uint32_t *eq, const uint32_t *consts, const std::string &label, const uint32_t *bw, int K,
+                   int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded);
+int sumcheck_verify(Transcript &tr, int n, const Statement &st, const uint32_t *claim, const uint32_t *eq,
+                    const uint32_t *consts, int blocks, const std::string &label, int degree, uint32_t *out_chal,
+                    uint32_t *out_reduced);
+int check_final(const Statement &st, int D, const uint32_t *reduced, const uint32_t *finals, const uint32_t *consts);
+void absorb_header(Transcript &tr, const std::string &label, int n, int degree, int blocks);
+
+}  // namespace exh

@@ -1,0 +1,522 @@
+// sumcheck.hip -- sumcheck session: weight tables, round launches, partial-sum reduction, folds.
+#include "sumcheck.hpp"
+
+#include <string.h>
+
+#include <map>
+
+#include "context.hpp"
+#include "hostfield.hpp"
+
+namespace exh {
+
+// ------------------------------------------------------------------ small kernels
+
+// eq weights for every round in one launch.  Table k covers the eq point's variables
+// [first, first + bits): entry x = prod_b (x_b ? r_b : 1 - r_b) (src/field.lisp:354-363: bit b of the
+// index pairs with the b-th variable).  factors[v] = (r_v R, (1 - r_v) R): each product is exact.
+struct EqTables {
+  int count;
+  uint64_t off[64];  // in EXTs
+  int first[64], bits[64];
+};
+
+template <int D>
+__global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const uint32_t *factors, uint32_t *out,
+                                                          uint64_t total) {
+  uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid >= total) return;
+  int k = 0;
+  uint64_t start = 0;
+  while (k + 1 < tabs.count && gid >= start + ((uint64_t)1 << tabs.bits[k])) {
+    start += (uint64_t)1 << tabs.bits[k];
+    k++;
+  }
+  uint64_t x = gid - start;
+  Ext<D> e = ext_lift<D>(1);
+  for (int b = 0; b < tabs.bits[k]; b++) {
+    const uint32_t *f = factors + ((size_t)(tabs.first[k] + b) * 2 + (((x >> b) & 1) ? 0 : 1)) * D;
+    e = ext_mul_mont<D>(e, load_ext<D>(f));
+  }
+  store_ext<D>(out + (tabs.off[k] + x) * D, e);
+}
+
+template <int D>
+__global__ __launch_bounds__(BLOCK) void fill_ones_kernel(uint32_t *out, uint64_t n) {
+  uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid < n) store_ext<D>(out + gid * D, ext_lift<D>(1));
+}
+
+// base values lifted to (v, 0, ..., 0) (src/sumcheck.lisp:75-82)
+template <int D>
+__global__ __launch_bounds__(BLOCK) void lift_kernel(const uint32_t *in, uint32_t *out, uint64_t n) {
+  uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid < n) store_ext<D>(out + gid * D, ext_lift<D>(in[gid]));
+}
+
+// one fold without sums (the last round): thread per folded entry
+template <int D, bool IN_BASE>
+__global__ __launch_bounds__(BLOCK) void fold_kernel(const uint32_t *in, uint32_t *out, uint64_t n_out,
+                                                     RoundArgs<D> args) {
+  uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid >= n_out) return;
+  Ext<D> r;
+#pragma unroll
+  for (int c = 0; c < D; c++) r.c[c] = args.r_mont[c];
+  Ext<D> o;
+  if constexpr (IN_BASE) {
+    uint2 e = *reinterpret_cast<const uint2 *>(in + 2 * gid);
+    o = fold_base<D>(e.x, e.y, r);
+  } else {
+    o = fold_ext<D>(load_ext<D>(in + 2 * gid * D), load_ext<D>(in + (2 * gid + 1) * D), r);
+  }
+  store_ext<D>(out + gid * D, o);
+}
+
+// sums[o] = sum over the workgroups' partials: one workgroup per output word
+__global__ __launch_bounds__(BLOCK) void reduce_partials_kernel(const uint32_t *partials, uint32_t nblocks,
+                                                                uint32_t width, uint32_t *sums) {
+  __shared__ uint32_t lds[BLOCK / 64];
+  uint32_t o = blockIdx.x, v = 0;
+  for (uint32_t b = threadIdx.x; b < nblocks; b += BLOCK) v = fadd(v, partials[(uint64_t)b * width + o]);
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < BLOCK / 64; w++) v = fadd(v, lds[w]);
+    sums[o] = v;
+  }
+}
+
+// the interpreter's launchers
+template <int D>
+static void launch_interp(const RoundArgs<D> &a, const StmtDesc &d, bool in_base, bool fold, uint32_t grid,
+                          hipStream_t s) {
+  if (in_base && fold)
+    hipLaunchKernelGGL((round_kernel_interp<D, true, true>), dim3(grid), dim3(BLOCK), 0, s, a, d);
+  else if (in_base)
+    hipLaunchKernelGGL((round_kernel_interp<D, true, false>), dim3(grid), dim3(BLOCK), 0, s, a, d);
+  else if (fold)
+    hipLaunchKernelGGL((round_kernel_interp<D, false, true>), dim3(grid), dim3(BLOCK), 0, s, a, d);
+  else
+    hipLaunchKernelGGL((round_kernel_interp<D, false, false>), dim3(grid), dim3(BLOCK), 0, s, a, d);
+}
+
+// ------------------------------------------------------------------ registry of generated kernels
+static std::map<std::pair<std::string, int>, KernelSet> &registry() {
+  static std::map<std::pair<std::string, int>, KernelSet> r;
+  return r;
+}
+void register_kernels(const std::string &key, int D, KernelSet set) { registry()[{key, D}] = set; }
+const KernelSet *find_kernels(const std::string &key, int D) {
+  auto it = registry().find({key, D});
+  return it == registry().end() ? nullptr : &it->second;
+}
+
+StmtDesc make_desc(const Statement &st) {
+  StmtDesc d;
+  memset(&d, 0, sizeof(d));
+  d.T = st.T();
+  int g = 0, maxx = 0;
+  for (const Group &grp : st.groups) {
+    if (grp.tabs.empty()) continue;
+    d.deg[g] = (int)grp.tabs.size();
+    for (size_t j = 0; j < grp.tabs.size(); j++) d.tab[g][j] = grp.tabs[j];
+    d.nev[g] = (int)grp.evalx.size();
+    for (size_t k = 0; k < grp.evalx.size(); k++) {
+      d.ev[g][k] = grp.evalx[k];
+      if (grp.evalx[k] > maxx) maxx = grp.evalx[k];
+    }
+    g++;
+  }
+  d.G = g;
+  d.nacc = st.nacc;
+  d.maxx = maxx;
+  return d;
+}
+
+// ------------------------------------------------------------------ the session
+static inline uint32_t next_pow2(uint64_t v) {
+  uint32_t p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uint32_t *const *tables,
+                           const int *strides, const uint32_t *eq, const uint32_t *bw, int K_, const uint32_t *consts,
+                           int degree, bool claim_mode_) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  D = D_, n = n_, K = K_;
+  if ((D != 4 && D != 8) || n < 0 || n > 40 || K < 1) {
+    set_error("invalid-parameter: sumcheck shape");
+    return E_PARAM;
+  }
+  st = statement;
+  if (degree < 0) degree = st.degree;
+  points = degree > 1 ? degree : 1;
+  claim_mode = claim_mode_;
+  if (claim_mode)
+    st.plan_claim();
+  else
+    st.plan(points);
+  eq0.clear();
+  if (eq && n > 0) eq0.assign(eq, eq + D);
+  int T = st.T(), real_groups = 0;
+  for (const Group &g : st.groups) {
+    if (g.tabs.empty()) continue;
+    real_groups++;
+    if ((int)g.tabs.size() > MAXDEG || (int)g.evalx.size() > MAXEV || g.evalx.back() > MAXX) {
+      set_error("invalid-parameter: statement degree beyond the kernels' limit");
+      return E_PARAM;
+    }
+  }
+  if (T < 1 || T > MAXT || real_groups > MAXG || st.nacc > MAXACC || points > 16) {
+    set_error("invalid-parameter: statement beyond the kernels' limits");
+    return E_PARAM;
+  }
+  desc = make_desc(st);
+  kernels = find_kernels(st.key(), D);
+  generated = kernels != nullptr;
+  has_eq = eq != nullptr;
+  has_bw = bw != nullptr;
+  size = (uint64_t)K << n;
+  round = 0;
+  pending_fold = false;
+  generation = 0;
+  group_coef.assign(st.groups.size() * D, 0);
+  group_coefficients(st, D, consts, group_coef.data());
+  bw_sum.assign(D, 0);
+  if (has_bw) {
+    for (int b = 0; b < K; b++)
+      for (int k = 0; k < D; k++) bw_sum[k] = fadd(bw_sum[k], bw[(size_t)b * D + k] % P);
+  }
+
+  // ---- layout of the misc arena: eq factors | weight tables | bw | ones | partials | sums | lifted
+  low_off.assign(n, 0), high_off.assign(n, 0), low_bits.assign(n, 0), n_high.assign(n, 0);
+  EqTables eqt;
+  memset(&eqt, 0, sizeof(eqt));
+  uint64_t pos = (uint64_t)2 * n;  // in EXTs: the eq factors come first
+  uint64_t bw_off = 0, ones_off = 0, ones_len = 0, total_eq = 0;
+  if (has_bw) {
+    bw_off = pos;
+    pos += K;
+  }
+  for (int j = 0; j < n; j++) {
+    int from = j + 1, middle = has_bw ? n : from + (n - from) / 2;
+    low_bits[j] = middle - from;
+    n_high[j] = has_bw ? (uint64_t)K : (uint64_t)1 << (n - middle);
+    if (has_eq) {
+      if (eqt.count + 2 > 64) {
+        set_error("invalid-parameter: too many rounds");
+        return E_PARAM;
+      }
+      low_off[j] = pos;
+      eqt.off[eqt.count] = pos, eqt.first[eqt.count] = from, eqt.bits[eqt.count] = middle - from;
+      eqt.count++;
+      pos += (uint64_t)1 << (middle - from);
+      total_eq += (uint64_t)1 << (middle - from);
+      if (!has_bw) {
+        high_off[j] = pos;
+        eqt.off[eqt.count] = pos, eqt.first[eqt.count] = middle, eqt.bits[eqt.count] = n - middle;
+        eqt.count++;
+        pos += (uint64_t)1 << (n - middle);
+        total_eq += (uint64_t)1 << (n - middle);
+      }
+    } else {
+      ones_len = std::max(ones_len, std::max((uint64_t)1 << low_bits[j], n_high[j]));
+    }
+    if (has_bw) high_off[j] = bw_off;
+  }
+  if (!has_eq && n > 0) {
+    ones_off = pos;
+    pos += ones_len;
+    for (int j = 0; j < n; j++) {
+      low_off[j] = ones_off;
+      if (!has_bw) high_off[j] = ones_off;
+    }
+  }
+  uint64_t pairs0 = size / 2;
+  max_grid = pairs0 ? (pairs0 + BLOCK - 1) / BLOCK : 1;
+  if (max_grid > 8192) max_grid = 8192;
+  uint64_t partial_off = pos * D;  // from here in words
+  uint64_t words = partial_off + (max_grid + 1) * (uint64_t)std::max(st.nacc, 1) * D + 64;
+  // mixed base / extension inputs: lift the base ones
+  bool any_base = false, all_base = true;
+  for (int t = 0; t < T; t++) {
+    if (strides[t] == 1)
+      any_base = true;
+    else if (strides[t] == D)
+      all_base = false;
+    else {
+      set_error("invalid-parameter: table stride must be 1 or D");
+      return E_PARAM;
+    }
+  }
+  uint64_t lifted_off = words;
+  if (any_base && !all_base)
+    for (int t = 0; t < T; t++)
+      if (strides[t] == 1) words += size * D;
+  if ((status = c.misc.reserve(words * 4))) return status;
+  uint32_t *base = (uint32_t *)c.misc.ptr;
+  d_weights = base;
+  d_partials = base + partial_off;
+  d_sums = d_partials + max_grid * (uint64_t)std::max(st.nacc, 1) * D;
+
+  cur.assign(T, nullptr);
+  cur_base = all_base;
+  for (int t = 0; t < T; t++) cur[t] = tables[t];
+  if (any_base && !all_base) {
+    uint32_t *dst = base + lifted_off;
+    for (int t = 0; t < T; t++)
+      if (strides[t] == 1) {
+        uint32_t grid = (uint32_t)((size + BLOCK - 1) / BLOCK);
+        if (D == 4)
+          hipLaunchKernelGGL(lift_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, tables[t], dst, size);
+        else
+          hipLaunchKernelGGL(lift_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, tables[t], dst, size);
+        cur[t] = dst;
+        dst += size * D;
+      }
+  }
+
+  // ---- upload the eq factors and block weights, build the weight tables
+  std::vector<uint32_t> host((size_t)(2 * n + (has_bw ? K : 0)) * D, 0);
+  if (has_eq)
+    for (int v = 0; v < n; v++)
+      for (int k = 0; k < D; k++) {
+        uint32_t r = eq[(size_t)v * D + k] % P, one_minus = fsub(k == 0 ? 1u : 0u, r);
+        host[((size_t)v * 2) * D + k] = to_mont(r);
+        host[((size_t)v * 2 + 1) * D + k] = to_mont(one_minus);
+      }
+  if (has_bw)
+    for (size_t i = 0; i < (size_t)K * D; i++) host[(size_t)2 * n * D + i] = bw[i] % P;
+  if (!host.empty()) EXH_HIP(hipMemcpyAsync(base, host.data(), host.size() * 4, hipMemcpyHostToDevice, c.stream));
+  EXH_HIP(hipStreamSynchronize(c.stream));  // host vector goes out of scope
+  if (has_eq && total_eq) {
+    uint32_t grid = (uint32_t)((total_eq + BLOCK - 1) / BLOCK);
+    // tables are laid out in launch order, so thread gid maps to table k by running sums; the
+    // offsets themselves may skip the block weights, so they are taken from eqt.off
+    if (D == 4)
+      hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, total_eq);
+    else
+      hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, total_eq);
+  }
+  if (!has_eq && ones_len) {
+    uint32_t grid = (uint32_t)((ones_len + BLOCK - 1) / BLOCK);
+    if (D == 4)
+      hipLaunchKernelGGL(fill_ones_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, base + ones_off * D, ones_len);
+    else
+      hipLaunchKernelGGL(fill_ones_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, base + ones_off * D, ones_len);
+  }
+  // the folded generations: the first holds half the input, the second a quarter
+  if (n > 0) {
+    if ((status = c.fold_a.reserve((size_t)T * (size / 2) * D * 4))) return status;
+    if (n > 1 && (status = c.fold_b.reserve((size_t)T * (size / 4) * D * 4))) return status;
+  }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+template <int D>
+static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::vector<uint32_t *> &outs,
+                        uint64_t n_pairs, int j) {
+  Context &c = ctx();
+  RoundArgs<D> a;
+  memset(&a, 0, sizeof(a));
+  int T = s.st.T();
+  for (int t = 0; t < T; t++) {
+    a.in[t] = s.cur[t];
+    a.out[t] = fold ? outs[t] : nullptr;
+  }
+  a.n_pairs = n_pairs;
+  a.do_sums = do_sums ? 1 : 0;
+  uint32_t ppt = 1;
+  if (do_sums) {
+    a.low = s.d_weights + s.low_off[j] * D;
+    a.high = s.d_weights + s.high_off[j] * D;
+    a.low_bits = (uint32_t)s.low_bits[j];
+  }
+  while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > s.max_grid) ppt *= 2;
+  a.pairs_per_thread = ppt;
+  a.deferred = do_sums && ((uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits)) ? 1 : 0;
+  a.partials = s.d_partials;
+  if (fold)
+    for (int k = 0; k < D; k++) a.r_mont[k] = to_mont(s.pending_r[k]);
+  uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
+  if (s.generated)
+    s.kernels->launch(&a, s.cur_base, fold, grid, c.stream);
+  else
+    launch_interp<D>(a, s.desc, s.cur_base, fold, grid, c.stream);
+  if (do_sums) {
+    uint32_t width = (uint32_t)s.st.nacc * D;
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3(width), dim3(BLOCK), 0, c.stream, s.d_partials, grid, width,
+                       s.d_sums);
+  }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+int SumcheckSession::round_sums(uint32_t *out) {
+  Context &c = ctx();
+  if (round >= n) {
+    set_error("invalid-parameter: no rounds left");
+    return E_PARAM;
+  }
+  if (round > 0 && !pending_fold) {
+    set_error("invalid-parameter: fold the previous round's challenge first");
+    return E_PARAM;
+  }
+  int T = st.T(), j = round, status;
+  uint64_t n_pairs;
+  if (pending_fold) {  // fused: fold round j-1's variable, then sum round j
+    uint64_t out_size = size / 2;
+    Arena &dst = (generation % 2 == 0) ? c.fold_a : c.fold_b;
+    out_buf.assign(T, nullptr);
+    for (int t = 0; t < T; t++) out_buf[t] = (uint32_t *)dst.ptr + (uint64_t)t * out_size * D;
+    n_pairs = out_size / 2;
+    status = D == 4 ? launch_round<4>(*this, true, true, out_buf, n_pairs, j)
+                    : launch_round<8>(*this, true, true, out_buf, n_pairs, j);
+    if (status) return status;
+    for (int t = 0; t < T; t++) cur[t] = out_buf[t];
+    cur_base = false;
+    size = out_size;
+    generation++;
+    pending_fold = false;
+  } else {
+    n_pairs = size / 2;
+    status = D == 4 ? launch_round<4>(*this, false, true, out_buf, n_pairs, j)
+                    : launch_round<8>(*this, false, true, out_buf, n_pairs, j);
+    if (status) return status;
+  }
+  size_t words = (size_t)st.nacc * D;
+  if (words) EXH_HIP(hipMemcpyAsync(c.host_pinned, d_sums, words * 4, hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipStreamSynchronize(c.stream));
+
+  // ---- the message rows from the groups' sums
+  // total weight of the pairs, for the constant group
+  hf::E wsum = hf::lift(1, D);
+  {
+    uint64_t nl = (uint64_t)1 << low_bits[j];
+    if (!has_eq) wsum = hf::lift((uint32_t)(nl % P), D);
+    if (has_bw)
+      wsum = hf::mul(wsum, bw_sum);
+    else if (!has_eq)
+      wsum = hf::scale(wsum, (uint32_t)(n_high[j] % P));
+  }
+  if (claim_mode) {  // sum_g coef_g ((1 - r_0) G(0) + r_0 G(1)), or G(0) + G(1) without eq
+    hf::E total = hf::zero(D), one = hf::lift(1, D);
+    for (size_t g = 0; g < st.groups.size(); g++) {
+      const Group &grp = st.groups[g];
+      hf::E coef(group_coef.begin() + g * D, group_coef.begin() + (g + 1) * D);
+      if (grp.tabs.empty()) {
+        total = hf::add(total, hf::mul(coef, has_eq ? wsum : hf::scale(wsum, 2)));
+        continue;
+      }
+      uint32_t fix = fpow(R1, grp.tabs.size());
+      hf::E g0(c.host_pinned + (size_t)grp.acc_base * D, c.host_pinned + (size_t)(grp.acc_base + 1) * D);
+      hf::E g1(c.host_pinned + (size_t)(grp.acc_base + 1) * D, c.host_pinned + (size_t)(grp.acc_base + 2) * D);
+      g0 = hf::scale(g0, fix), g1 = hf::scale(g1, fix);
+      hf::E v = has_eq ? hf::add(hf::mul(hf::sub(one, eq0), g0), hf::mul(eq0, g1)) : hf::add(g0, g1);
+      total = hf::add(total, hf::mul(coef, v));
+    }
+    memcpy(out, total.data(), 4 * D);
+    return OK;
+  }
+  std::vector<int> wire(points);
+  for (int k = 0; k < points; k++) wire[k] = k == 0 ? 0 : k + 1;
+  std::vector<hf::E> rows(points, hf::zero(D));
+  for (size_t g = 0; g < st.groups.size(); g++) {
+    const Group &grp = st.groups[g];
+    hf::E coef(group_coef.begin() + g * D, group_coef.begin() + (g + 1) * D);
+    if (grp.tabs.empty()) {
+      hf::E v = hf::mul(coef, wsum);
+      for (int k = 0; k < points; k++) rows[k] = hf::add(rows[k], v);
+      continue;
+    }
+    uint32_t fix = fpow(R1, grp.tabs.size());  // the kernel's sums carry R^-degree
+    std::vector<hf::E> vals;
+    for (size_t k = 0; k < grp.evalx.size(); k++) {
+      hf::E v(c.host_pinned + (size_t)(grp.acc_base + k) * D, c.host_pinned + (size_t)(grp.acc_base + k + 1) * D);
+      vals.push_back(hf::scale(v, fix));
+    }
+    bool direct = (int)grp.tabs.size() >= points;
+    for (int k = 0; k < points; k++) {
+      hf::E gv = direct ? vals[k] : hf::interpolate(grp.evalx, vals, hf::lift((uint32_t)wire[k], D));
+      rows[k] = hf::add(rows[k], hf::mul(coef, gv));
+    }
+  }
+  for (int k = 0; k < points; k++) memcpy(out + (size_t)k * D, rows[k].data(), 4 * D);
+  return OK;
+}
+
+int SumcheckSession::fold(const uint32_t *r) {
+  if (round >= n || pending_fold) {
+    set_error("invalid-parameter: nothing to fold");
+    return E_PARAM;
+  }
+  for (int k = 0; k < D; k++) pending_r[k] = r[k] % P;
+  pending_fold = true;
+  round++;
+  return OK;
+}
+
+int SumcheckSession::flush() {
+  Context &c = ctx();
+  if (!pending_fold) return OK;
+  int T = st.T();
+  uint64_t out_size = size / 2;
+  Arena &dst = (generation % 2 == 0) ? c.fold_a : c.fold_b;
+  RoundArgs<4> a4;
+  RoundArgs<8> a8;
+  memset(&a4, 0, sizeof(a4));
+  memset(&a8, 0, sizeof(a8));
+  for (int k = 0; k < D; k++) a4.r_mont[k % 4] = a8.r_mont[k] = to_mont(pending_r[k]);
+  uint32_t grid = (uint32_t)((out_size + BLOCK - 1) / BLOCK);
+  for (int t = 0; t < T; t++) {
+    uint32_t *o = (uint32_t *)dst.ptr + (uint64_t)t * out_size * D;
+    if (D == 4 && cur_base)
+      hipLaunchKernelGGL((fold_kernel<4, true>), dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], o, out_size, a4);
+    else if (D == 4)
+      hipLaunchKernelGGL((fold_kernel<4, false>), dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], o, out_size, a4);
+    else if (cur_base)
+      hipLaunchKernelGGL((fold_kernel<8, true>), dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], o, out_size, a8);
+    else
+      hipLaunchKernelGGL((fold_kernel<8, false>), dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], o, out_size, a8);
+    cur[t] = o;
+  }
+  EXH_HIP(hipGetLastError());
+  cur_base = false;
+  size = out_size;
+  generation++;
+  pending_fold = false;
+  return OK;
+}
+
+int SumcheckSession::finish(uint32_t *finals, uint32_t *const *folded) {
+  Context &c = ctx();
+  int status = flush();
+  if (status) return status;
+  int T = st.T();
+  // each table's current entries (K of them after n rounds), lifted if still base
+  std::vector<uint32_t> tmp;
+  for (int t = 0; t < T; t++) {
+    uint64_t words = size * (cur_base ? 1 : D);
+    tmp.resize(words);
+    EXH_HIP(hipMemcpyAsync(tmp.data(), cur[t], words * 4, hipMemcpyDeviceToHost, c.stream));
+    EXH_HIP(hipStreamSynchronize(c.stream));
+    for (uint64_t x = 0; x < size; x++) {
+      uint32_t e[8] = {0};
+      if (cur_base)
+        e[0] = tmp[x];
+      else
+        memcpy(e, &tmp[x * D], 4 * D);
+      if (x == 0 && finals) memcpy(finals + (size_t)t * D, e, 4 * D);
+      if (folded && folded[t]) memcpy(folded[t] + x * D, e, 4 * D);
+    }
+  }
+  return OK;
+}
+
+}  // namespace exh

@@ -1,0 +1,63 @@
+// sumcheck.hpp -- the device side of the sumcheck prover as a session: the tables stay in HBM, each
+// round returns its message rows, each fold takes the round's challenge.  It replaces the bodies of
+// the reference's round kernel call and FOLD-FLAT-TABLE inside PROVE (src/sumcheck.lisp:547-563).
+#pragma once
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "forms.hpp"
+#include "sumcheck_kernels.cuh"
+
+namespace exh {
+
+struct KernelSet {  // the launchers generated for one statement and one degree D
+  void (*launch)(const void *args, bool in_base, bool fold, uint32_t grid, hipStream_t stream);
+};
+void register_kernels(const std::string &key, int D, KernelSet set);
+const KernelSet *find_kernels(const std::string &key, int D);
+StmtDesc make_desc(const Statement &st);
+
+struct SumcheckSession {
+  int D = 4, n = 0, K = 1, points = 1;
+  Statement st;
+  bool generated = false;  // a kernel generated for the statement is in use (else the interpreter)
+  const KernelSet *kernels = nullptr;
+  StmtDesc desc;
+  std::vector<const uint32_t *> cur;  // current tables (device)
+  bool cur_base = false;
+  uint64_t size = 0;  // entries per table now
+  int round = 0;
+  bool has_eq = false, has_bw = false;
+  std::vector<uint32_t> group_coef;  // G * D
+  std::vector<uint32_t> bw_sum;      // sum of the block weights (D), for the constant group
+  // per-round weight tables on the device
+  uint32_t *d_weights = nullptr;
+  std::vector<uint64_t> low_off, high_off;
+  std::vector<int> low_bits;
+  std::vector<uint64_t> n_high;
+  uint32_t *d_partials = nullptr, *d_sums = nullptr, *d_lifted = nullptr;
+  uint64_t max_grid = 0;
+  bool pending_fold = false;
+  uint32_t pending_r[8];
+  int generation = 0;
+  std::vector<uint32_t *> out_buf;  // scratch for the launch
+
+  // tables[t]: K * 2^n entries of stride strides[t] (1 or D), block-major, on the device.
+  // eq: n * D host words or null; bw: K * D host words or null; consts: C * D host words.
+  int begin(const Statement &statement, int D, int n, const uint32_t *const *tables, const int *strides,
+            const uint32_t *eq, const uint32_t *bw, int K, const uint32_t *consts, int degree,
+            bool claim_mode = false);
+  // claim mode: round_sums returns the honest claim sum_x w(x) F(tables(x)) in out[0..D) (n >= 1)
+  bool claim_mode = false;
+  std::vector<uint32_t> eq0;  // the eq point's first coordinate, for the claim
+  int round_sums(uint32_t *out /* points * D */);
+  int fold(const uint32_t *r /* D */);
+  // finals: T * D; folded[t] (optional): K * D each
+  int finish(uint32_t *finals, uint32_t *const *folded);
+  // device pointers of the current (fully or partly folded) tables, after any pending fold
+  int flush();
+};
+
+}  // namespace exh

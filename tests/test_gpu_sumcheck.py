@@ -1,0 +1,202 @@
+"""GPU parity for the sumcheck path: the HIP library through its C ABI against the golden whole-proof
+vectors and against the CPU oracle on seeded inputs.  Integer work: every comparison is bit-exact."""
+import numpy as np
+import pytest
+
+import sable_amd as sa
+from oracle import binding as orc
+
+pytestmark = pytest.mark.gpu
+P = sa.P
+hx = bytes.fromhex
+
+
+def same(a, b):
+    return np.array_equal(np.asarray(a, np.uint64), np.asarray(b, np.uint64))
+
+
+def rand_ext(rng, shape, d):
+    return rng.integers(0, P, tuple(shape) + (d,), dtype=np.uint32)
+
+
+def both(form, tables, constants=()):
+    return sa.Statement(form, tables, constants), orc.Statement(form, tables, constants)
+
+
+def prove_both(label, d, n, form, names, host_tables, eq=None, constants=None, cnames=(), block_weights=None,
+               degree=None, sc_label="sc"):
+    st, ost = both(form, names, cnames)
+    dev = [sa.Table.upload(t) for t in host_tables]
+    tr, otr = sa.Transcript(label, d), orc.Transcript(label, d)
+    got = sa.prove(tr, n, st, dev, eq=eq, constants=constants, block_weights=block_weights, degree=degree,
+                   label=sc_label)
+    want = orc.prove(otr, n, ost, host_tables, eq=eq, constants=constants, block_weights=block_weights,
+                     degree=degree, label=sc_label)
+    for t in dev:
+        t.free()
+    assert tr.proof() == otr.proof(), f"proof bytes differ: {form} n={n} D={d}"
+    assert same(got[0], want[0]) and same(got[1], want[1])
+    for a, b in zip(got[2], want[2]):
+        assert same(a, b)
+    return st, ost, tr.proof(), got
+
+
+def test_golden_proofs_byte_for_byte(vectors):
+    """tests.lisp:277-282: the prover writes the same bytes as the original prover, after the magic."""
+    for v in vectors("sumcheck"):
+        d, n, nt = v["d"], v["n"], len(v["tables"])
+        names = [f"t{i}" for i in range(nt)]
+        st = sa.Statement("(* " + " ".join(names) + ")", names)
+        tables = [sa.Table.upload(np.array(t, np.uint32)) for t in v["tables"]]
+        eq = np.array(v["eq_r"], np.uint32) if v["eq_r"] else None
+        assert same(sa.hypercube_sum(st, n, tables, d, eq=eq), v["claim"])
+        tr = sa.Transcript("sc-vec", d)
+        rho, finals, _ = sa.prove(tr, n, st, tables, eq=eq)
+        assert same(rho, v["rho"]) and same(finals, v["finals"])
+        assert tr.proof() == b"EXACTPF1" + hx(v["proof"])[8:]
+        for t in tables:
+            t.free()
+
+
+@pytest.mark.parametrize("n", [1, 2, 5, 9, 12, 16])
+def test_config1_product_of_two_base_tables(n):
+    """(* eq t0 t1): two base tables, eq mode, F_p^4; n = 16 is the full configuration."""
+    rng = np.random.default_rng(1000 + n)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in range(2)]
+    eq = rand_ext(rng, (n,), 4)
+    st, ost, proof, _ = prove_both("config1", 4, n, "(* t0 t1)", ["t0", "t1"], tables, eq=eq)
+    assert st.has_generated_kernel(4)
+    assert len(proof) == 12 + n * (18 + 4 * 2 * 4)
+    # the oracle's verifier accepts the GPU proof
+    claim = orc.hypercube_sum(ost, n, tables, 4, eq=eq)
+    dev = [sa.Table.upload(t) for t in tables]
+    assert same(sa.hypercube_sum(st, n, dev, 4, eq=eq), claim)
+    vtr = orc.Transcript("config1", 4, proof=proof)
+    _, reduced = orc.verify(vtr, n, ost, claim, eq=eq)
+    finals = sa.prove(sa.Transcript("config1", 4), n, st, dev, eq=eq)[1]
+    assert orc.check_final(reduced, ost, finals) and vtr.finished()
+    for t in dev:
+        t.free()
+
+
+CONFIG2 = "(+ (* alpha t0 t1 t2) (* 3 t1))"
+CONFIG3 = "(* (+ c0 3) (- c1 c0) c2 c3)"
+
+
+@pytest.mark.parametrize("n", [1, 3, 8, 13])
+def test_config2_statement_with_a_constant(n):
+    rng = np.random.default_rng(2000 + n)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in range(3)]
+    eq, alpha = rand_ext(rng, (n,), 4), rand_ext(rng, (1,), 4)
+    st, ost, proof, _ = prove_both("config2", 4, n, CONFIG2, ["t0", "t1", "t2"], tables, eq=eq, constants=alpha,
+                                   cnames=["alpha"])
+    assert st.has_generated_kernel(4) and st.degree == 3
+    assert len(proof) == 12 + n * (18 + 4 * 3 * 4)
+    claim = orc.hypercube_sum(ost, n, tables, 4, eq=eq, constants=alpha)
+    vtr = sa.Transcript("config2", 4, proof=proof)
+    _, reduced = sa.verify(vtr, n, st, claim, eq=eq, constants=alpha)
+    dev = [sa.Table.upload(t) for t in tables]
+    assert same(sa.hypercube_sum(st, n, dev, 4, eq=eq, constants=alpha), claim)
+    for t in dev:
+        t.free()
+
+
+@pytest.mark.parametrize("n", [2, 7, 11])
+def test_config3_product_constraint_over_fp8(n):
+    rng = np.random.default_rng(3000 + n)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in range(4)]
+    eq = rand_ext(rng, (n,), 8)
+    st, ost, proof, _ = prove_both("config3", 8, n, CONFIG3, ["c0", "c1", "c2", "c3"], tables, eq=eq)
+    assert st.degree == 4 and len(proof) == 12 + n * (18 + 4 * 4 * 8)
+
+
+@pytest.mark.parametrize("form,names,cnames,d,base,with_eq", [
+    ("(* t0 t1 t2)", ["t0", "t1", "t2"], [], 4, True, True),
+    ("(* t0 t1 t2)", ["t0", "t1", "t2"], [], 8, False, False),
+    ("(+ (* t0 t1 t2) (* 7 t1) -1)", ["t0", "t1", "t2"], [], 4, True, True),
+    ("(+ (* t0 t1 t2) (* 7 t1) -1)", ["t0", "t1", "t2"], [], 8, True, False),
+    ("(- (* alpha (expt t0 2) t1) t1)", ["t0", "t1"], ["alpha"], 4, False, True),
+    ("t0", ["t0"], [], 4, True, True),
+    ("(- (expt t0 3) (* t0 t1))", ["t0", "t1"], [], 8, True, True),
+    ("(* t0 t1 t2 t3)", ["t0", "t1", "t2", "t3"], [], 4, False, True),
+    ("(+ (* alpha t0 t1) (* 3 t1) -2)", ["t0", "t1"], ["alpha"], 4, False, False),
+])
+def test_any_statement_on_the_interpreter_or_generated_kernels(form, names, cnames, d, base, with_eq):
+    """tests.lisp:311-395: statements that are not plain products, constants, base or extension tables."""
+    n = 6
+    rng = np.random.default_rng(len(form) + d)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) if base else rand_ext(rng, (1 << n,), d) for _ in names]
+    eq = rand_ext(rng, (n,), d) if with_eq else None
+    consts = rand_ext(rng, (len(cnames),), d) if cnames else None
+    prove_both("any", d, n, form, names, tables, eq=eq, constants=consts, cnames=cnames)
+
+
+def test_mixed_base_and_extension_tables():
+    n, d = 5, 4
+    rng = np.random.default_rng(77)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32), rand_ext(rng, (1 << n,), d)]
+    prove_both("mixed", d, n, "(* t0 t1)", ["t0", "t1"], tables, eq=rand_ext(rng, (n,), d))
+
+
+@pytest.mark.parametrize("K,n,d", [(3, 3, 4), (1, 4, 4), (5, 2, 8), (2, 0, 4)])
+def test_block_weights(K, n, d):
+    """prove with :block-weights (sumcheck.lisp:519-521, 549-550), as the GKR layers call it."""
+    rng = np.random.default_rng(K * 10 + n)
+    tables = [rand_ext(rng, (K << n,), d) for _ in range(2)]
+    bw = rand_ext(rng, (K,), d)
+    eq = rand_ext(rng, (n,), d) if n else None
+    prove_both("bw", d, n, "(* t0 t1)", ["t0", "t1"], tables, eq=eq, block_weights=bw, degree=2 if n else 0,
+               sc_label="gkr")
+
+
+def test_round_by_round_session_matches_the_oracle_rounds():
+    """The entry points an SBCL host binds: round sums and folds, one call each."""
+    n, d = 7, 4
+    rng = np.random.default_rng(5)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in range(3)]
+    eq, alpha = rand_ext(rng, (n,), d), rand_ext(rng, (1,), d)
+    st, ost = both(CONFIG2, ["t0", "t1", "t2"], ["alpha"])
+    dev = [sa.Table.upload(t) for t in tables]
+    s = sa.SumcheckSession(st, d, n, dev, eq=eq, constants=alpha)
+    cur = tables
+    for j in range(n):
+        frm, middle = j + 1, j + 1 + (n - j - 1) // 2
+        low, high = orc.eq_table(eq[frm:middle], d), orc.eq_table(eq[middle:], d)
+        assert same(s.round(), orc.round_sums(ost, d, 3, cur, low, high, alpha)), f"round {j}"
+        r = rand_ext(rng, (), d)
+        s.fold(r)
+        cur = [orc.fold_flat(t, r) for t in cur]
+    finals, folded = s.finish()
+    assert same(finals, [t[0] for t in cur])
+    with pytest.raises(sa.InvalidParameter):
+        sa.SumcheckSession(st, d, n, dev[:2], eq=eq, constants=alpha)
+    for t in dev:
+        t.free()
+
+
+def test_linearity_and_fold_consistency_at_scale():
+    """Size-independent properties at a size the oracle does not run: the config-2 statement's round
+    sums are alpha * sums(t0 t1 t2) + 3 * sums(t1), and g(0), g(2), g(3) with g(1) from the claim lie on
+    one cubic whose value at r is the next round's claim (the verifier's recurrence)."""
+    n, d = 20, 4
+    st = sa.Statement(CONFIG2, ["t0", "t1", "t2"], ["alpha"])
+    prod = sa.Statement("(* t0 t1 t2)", ["t0", "t1", "t2"])
+    lin = sa.Statement("(* 1 t1)", ["t0", "t1", "t2"])
+    rng = np.random.default_rng(9)
+    eq, alpha = rand_ext(rng, (n,), d), rand_ext(rng, (1,), d)
+    dev = [sa.Table.random(900 + k, 1 << n) for k in range(3)]
+    full = sa.SumcheckSession(st, d, n, dev, eq=eq, constants=alpha)
+    a = full.round()
+    b = sa.SumcheckSession(prod, d, n, dev, eq=eq).round()
+    c = sa.SumcheckSession(lin, d, n, dev, eq=eq, degree=3).round()
+    for k in range(3):
+        assert same(a[k], orc.ext_add(orc.ext_mul(alpha[0], b[k]), orc.ext_scale(c[k], 3)))
+    claim = sa.hypercube_sum(st, n, dev, d, eq=eq, constants=alpha)
+    tr = sa.Transcript("scale", d)
+    sa.prove(tr, n, st, dev, eq=eq, constants=alpha)
+    vtr = sa.Transcript("scale", d, proof=tr.proof())
+    _, reduced = sa.verify(vtr, n, st, claim, eq=eq, constants=alpha)
+    finals = sa.prove(sa.Transcript("scale", d), n, st, dev, eq=eq, constants=alpha)[1]
+    assert sa.check_final(reduced, st, finals, constants=alpha)
+    for t in dev:
+        t.free()
