@@ -4,10 +4,10 @@
 namespace exh {
 
 constexpr int MAXT = 16;    // tables per statement
-constexpr int MAXG = 12;    // table groups per statement
+constexpr int MAXG = 16;    // table groups per statement
 constexpr int MAXDEG = 6;   // tables per group
 constexpr int MAXEV = 6;    // evaluation points per group
-constexpr int MAXACC = 24;  // accumulators (group, point) per statement
+constexpr int MAXACC = 36;  // accumulators (group, point) per statement
 constexpr int MAXX = 7;     // largest evaluation point
 constexpr int BLOCK = 256;  // threads per workgroup
 

@@ -1,0 +1,138 @@
+"""GPU parity for the commitment path: Reed-Solomon encode and fold, BLAKE3 leaf digests and Merkle
+levels, pcs-commit and the BaseFold loop, through the C ABI against the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+
+import sable_amd as sa
+from oracle import binding as orc
+
+pytestmark = pytest.mark.gpu
+P = sa.P
+
+
+def same(a, b):
+    return np.array_equal(np.asarray(a, np.uint64), np.asarray(b, np.uint64))
+
+
+def test_rs_encode_golden_vectors(vectors):
+    for v in vectors("rs-encode"):
+        n = v["n"]
+        msg = sa.Table.upload(np.array(v["msg"], np.uint32))
+        cw = sa.encode(msg, 1, n - 1)
+        assert same(cw.download(), v["cw"])
+        msg.free(), cw.free()
+
+
+@pytest.mark.parametrize("c,ncols", [(0, 1), (1, 2), (4, 3), (11, 2), (12, 1), (13, 2), (16, 2), (19, 1)])
+def test_rs_encode_matches_the_oracle(c, ncols):
+    rng = np.random.default_rng(c)
+    msgs = rng.integers(0, P, (ncols, 1 << c), dtype=np.uint32)
+    t = sa.Table.upload(msgs.reshape(-1))
+    cw = sa.encode(t, ncols, c)
+    got = cw.download().reshape(ncols, -1)
+    for k in range(ncols):
+        assert same(got[k], orc.rs_encode(msgs[k], c + 1)), f"column {k}"
+    t.free(), cw.free()
+
+
+def test_rs_encode_is_evaluation_and_full_size_roundtrip():
+    """At the full size (2^23 coefficients -> 2^24 symbols) the oracle is too slow: check the codeword as
+    evaluations at a few positions (position t holds f(w^bitrev(t)), rs.lisp:4-6) and that folding the
+    codeword is the codeword of the folded message (rs.lisp:8-9)."""
+    c = 23
+    msg = sa.Table.random(5, 1 << c)
+    cw = sa.encode(msg, 1, c)
+    m = msg.download().astype(object)
+    w = orc.root_of_unity(c + 1)
+    for t in (0, 1, 2, 12345, (1 << 24) - 1):
+        x = pow(w, int(format(t, "024b")[::-1], 2), P)
+        # Horner in Python ints over 2^23 coefficients is slow; use numpy power sums in chunks
+        xs = np.array([pow(x, i, P) for i in range(1 << 10)], dtype=object)
+        step = pow(x, 1 << 10, P)
+        acc, xp = 0, 1
+        for i in range(0, 1 << c, 1 << 10):
+            acc = (acc + xp * int(np.dot(m[i:i + (1 << 10)], xs) % P)) % P
+            xp = xp * step % P
+        assert int(cw.download(t, 1)[0]) == acc
+    msg.free(), cw.free()
+
+
+@pytest.mark.parametrize("d,n", [(8, 6), (4, 9), (8, 13)])
+def test_rs_fold(d, n, vectors):
+    rng = np.random.default_rng(n)
+    cw = rng.integers(0, P, (1 << n, d), dtype=np.uint32)
+    r = rng.integers(0, P, d, dtype=np.uint32)
+    t = sa.Table.upload(cw)
+    for level in (0, 1):
+        m = (1 << n) >> (level + 1)
+        sub = sa.Table.upload(cw[:2 * m])
+        out = sa.rs_fold(sub, d, n, level, r)
+        assert same(out.download(), orc.rs_fold(cw[:2 * m], orc.twiddles(n)[level], r))
+        sub.free(), out.free()
+    t.free()
+    if d == 8 and n == 6:
+        for v in vectors("rs-fold"):
+            t = sa.Table.upload(np.array(v["cw"], np.uint32))
+            out = sa.rs_fold(t, 8, v["n"], 0, v["r"])
+            assert same(out.download(), v["res"])
+
+
+@pytest.mark.parametrize("c,ncols", [(1, 1), (5, 2), (9, 3), (10, 70), (14, 2)])
+def test_merkle_commit_matches_the_oracle(c, ncols):
+    rng = np.random.default_rng(c + ncols)
+    cols = [rng.integers(0, P, 1 << c, dtype=np.uint32) for _ in range(ncols)]
+    ocw, olevels, ocap = orc.commit_columns(cols, c)
+    tr, otr = sa.Transcript("commit", 4), orc.Transcript("commit", 4)
+    t = sa.Table.upload(np.concatenate(cols))
+    cw, levels = sa.pcs_commit(tr, t, ncols, c)
+    otr.send_bytes(ocap.tobytes())
+    assert tr.proof() == otr.proof()
+    assert same(cw.download().reshape(ncols, -1), ocw)
+    got = levels.download().reshape(-1, 8).astype("<u4").view(np.uint8).reshape(-1, 32)
+    assert same(got, np.concatenate(olevels))
+    for x in (t, cw, levels):
+        x.free()
+
+
+def test_commit_full_size_paths_open_to_the_cap():
+    """Config 5's commitment at full size: two 2^23-coefficient columns -> 2^22 leaves -> cap of 128; a few
+    leaves are recomputed on the host from the downloaded codeword symbols and opened against the cap."""
+    c, ncols = 23, 2
+    t = sa.Table.random(11, ncols << c)
+    tr = sa.Transcript("commit", 4)
+    cw, levels = sa.pcs_commit(tr, t, ncols, c)
+    cap = np.frombuffer(orc.decode_proof(tr.proof())[0], np.uint8).reshape(-1, 32)
+    nleaves = 1 << (c - 1)
+    lc = orc.cap_level(nleaves)
+    assert len(cap) == 128 and lc == 15
+    cwlen = 1 << (c + 1)
+    for leaf in (0, 1, 999999, nleaves - 1):
+        rows = [cw.download(k * cwlen + 4 * leaf, 4) for k in range(ncols)]
+        h = orc.leaf_digest(np.array(rows))
+        path, i, start, n = [], leaf, 0, nleaves
+        for _ in range(lc):
+            path.append(levels.download((start + (i ^ 1)) * 8, 8).reshape(-1).astype("<u4").view(np.uint8))
+            start += n
+            n //= 2
+            i >>= 1
+        assert orc.check_path(h, np.array(path), leaf, cap)
+    for x in (t, cw, levels):
+        x.free()
+
+
+@pytest.mark.parametrize("nv", [4, 9, 12])
+def test_basefold_matches_the_oracle(nv):
+    rng = np.random.default_rng(nv)
+    h = rng.integers(0, P, (1 << nv, 8), dtype=np.uint32)
+    rr = rng.integers(0, P, (nv, 8), dtype=np.uint32)
+    v = orc.mle_eval(h, rr, 8)
+    tr, otr = sa.Transcript("bf", 4), orc.Transcript("bf", 4)
+    t = sa.Table.upload(h)
+    got = sa.basefold_prove(tr, nv, rr, v, t)
+    want = orc.basefold_prove(otr, nv, rr, v, h)
+    assert tr.proof() == otr.proof()
+    assert got[0] == want[0] and same(got[1], want[1]) and same(got[2], want[2])
+    assert sa.basefold_verify(sa.Transcript("bf", 4, proof=tr.proof()), nv, rr, v) == got[0]
+    with pytest.raises(sa.VerificationFailure):
+        sa.basefold_verify(sa.Transcript("bf", 4, proof=tr.proof()), nv, rr, orc.ext_add(v, orc.base_to_ext(1, 8)))
+    t.free()
