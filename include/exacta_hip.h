@@ -42,8 +42,17 @@ typedef uint64_t exh_session; /* one sumcheck in progress */
 int exh_init(int device);
 void exh_shutdown(void);
 const char *exh_last_error(void);
+/* wait until everything the library has queued on the device is done */
+int exh_synchronize(void);
 /* 1 when a kernel generated for the statement is used, 0 when the interpreter kernel is */
 int exh_stmt_has_generated_kernel(exh_stmt stmt, int degree_d);
+
+/* ---- measurement (no counterpart in the reference): with profiling on, every data-parallel kernel
+   launch is bracketed by HIP events on the library's stream; entries report the kernel, the round it
+   served, its duration and the bytes it had to move (tables read + tables written) */
+int exh_profile_enable(int on);
+int exh_profile_count(void);
+int exh_profile_entry(int index, char *name, int name_cap, int *round, float *ms, uint64_t *alg_bytes);
 
 /* ---- tables: MAKE-TABLE and the read-back at the end of PROVE (src/sumcheck.lisp:61-70, 564-571) */
 int exh_table_upload(const uint32_t *host, uint64_t n_u32, int stride, exh_table *out);

@@ -83,6 +83,43 @@ void exh_shutdown(void) {
   ctx_shutdown();
 }
 const char *exh_last_error(void) { return last_error(); }
+int exh_synchronize(void) {
+  int status = ctx().require();
+  if (status) return status;
+  EXH_HIP(hipDeviceSynchronize());
+  return OK;
+}
+
+int exh_profile_enable(int on) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  (void)hipStreamSynchronize(c.stream);
+  c.prof_clear();
+  c.profiling = on != 0;
+  return OK;
+}
+int exh_profile_count(void) { return (int)ctx().profile.size(); }
+int exh_profile_entry(int index, char *name, int name_cap, int *round, float *ms, uint64_t *alg_bytes) {
+  Context &c = ctx();
+  if (index < 0 || index >= (int)c.profile.size()) {
+    set_error("invalid-parameter: profile index");
+    return E_PARAM;
+  }
+  ProfileEntry &e = c.profile[index];
+  if (e.ms < 0) {
+    EXH_HIP(hipEventSynchronize(e.stop));
+    EXH_HIP(hipEventElapsedTime(&e.ms, e.start, e.stop));
+  }
+  if (name && name_cap > 0) {
+    strncpy(name, e.name.c_str(), name_cap - 1);
+    name[name_cap - 1] = 0;
+  }
+  if (round) *round = e.round;
+  if (ms) *ms = e.ms;
+  if (alg_bytes) *alg_bytes = e.alg_bytes;
+  return OK;
+}
 
 // ------------------------------------------------------------------ tables
 int exh_table_alloc(uint64_t n_u32, int stride, exh_table *out) {

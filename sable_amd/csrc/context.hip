@@ -42,6 +42,26 @@ int Context::require() {
   return OK;
 }
 
+void Context::prof_begin(const char *name, int round, uint64_t alg_bytes) {
+  if (!profiling) return;
+  ProfileEntry e;
+  e.name = name, e.round = round, e.alg_bytes = alg_bytes;
+  if (hipEventCreate(&e.start) != hipSuccess || hipEventCreate(&e.stop) != hipSuccess) return;
+  (void)hipEventRecord(e.start, stream);
+  profile.push_back(e);
+}
+void Context::prof_end() {
+  if (!profiling || profile.empty()) return;
+  (void)hipEventRecord(profile.back().stop, stream);
+}
+void Context::prof_clear() {
+  for (ProfileEntry &e : profile) {
+    if (e.start) (void)hipEventDestroy(e.start);
+    if (e.stop) (void)hipEventDestroy(e.stop);
+  }
+  profile.clear();
+}
+
 int ctx_init(int device) {
   Context &c = g_ctx;
   if (c.ready) return OK;
@@ -74,6 +94,7 @@ void ctx_shutdown() {
   Context &c = g_ctx;
   if (!c.ready) return;
   (void)hipStreamSynchronize(c.stream);
+  c.prof_clear();
   for (auto &kv : c.tables)
     if (kv.second.owned && kv.second.ptr) (void)hipFree(kv.second.ptr);
   c.tables.clear();

@@ -36,8 +36,24 @@ struct Arena {
   void release();
 };
 
+// One timed kernel launch (HIP events on the library's stream), kept while profiling is on.
+struct ProfileEntry {
+  std::string name;
+  int round = 0;
+  uint64_t alg_bytes = 0;  // bytes the launch must move: tables read + tables written
+  hipEvent_t start = nullptr, stop = nullptr;
+  float ms = -1.0f;
+};
+
 struct Context {
   bool ready = false;
+  bool profiling = false;
+  std::vector<ProfileEntry> profile;
+  // bracket a launch: prof_begin records the start event, prof_end the stop event (no-ops unless
+  // profiling is on)
+  void prof_begin(const char *name, int round, uint64_t alg_bytes);
+  void prof_end();
+  void prof_clear();
   int device = -1;
   hipStream_t stream = nullptr;
   std::map<uint64_t, DeviceTable> tables;

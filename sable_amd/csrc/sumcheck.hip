@@ -345,10 +345,17 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   if (fold)
     for (int k = 0; k < D; k++) a.r_mont[k] = to_mont(s.pending_r[k]);
   uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
+  {
+    // bytes this launch must move: every table read once, the folded tables written once
+    uint64_t in_words = (fold ? 4 : 2) * n_pairs * (s.cur_base ? 1 : D), out_words = fold ? 2 * n_pairs * D : 0;
+    const char *name = fold ? (s.cur_base ? "round_fold_base" : "round_fold_ext") : (s.cur_base ? "round_base" : "round_ext");
+    c.prof_begin(name, j, (uint64_t)T * 4 * (in_words + out_words));
+  }
   if (s.generated)
     s.kernels->launch(&a, s.cur_base, fold, grid, c.stream);
   else
     launch_interp<D>(a, s.desc, s.cur_base, fold, grid, c.stream);
+  c.prof_end();
   if (do_sums) {
     uint32_t width = (uint32_t)s.st.nacc * D;
     hipLaunchKernelGGL(reduce_partials_kernel, dim3(width), dim3(BLOCK), 0, c.stream, s.d_partials, grid, width,
