@@ -1,7 +1,10 @@
 // prover.cpp -- see prover.hpp.
 #include "prover.hpp"
 
+#include <stdlib.h>
 #include <string.h>
+
+#include <vector>
 
 #include "hostfield.hpp"
 
@@ -26,6 +29,31 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
   int status = s.begin(st, D, n, d_tables, strides, eq, bw, K, consts, degree);
   if (status) return status;
   absorb_header(tr, label, n, degree, bw ? K : 1);
+  const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS");
+  if (n > 0 && s.device_capable() && !(host_rounds && host_rounds[0] == '1')) {
+    // the rounds run back to back on the device, transcript included; the messages are then replayed
+    // into this transcript, which must draw the same challenges
+    DevB3S state;
+    memcpy(state.cv, tr.state.cv, 32);
+    for (int i = 0; i < 16; i++)
+      state.block[i] = (uint32_t)tr.state.block[4 * i] | (uint32_t)tr.state.block[4 * i + 1] << 8 |
+                       (uint32_t)tr.state.block[4 * i + 2] << 16 | (uint32_t)tr.state.block[4 * i + 3] << 24;
+    state.used = tr.state.used;
+    state.counter_lo = (uint32_t)tr.state.counter, state.counter_hi = (uint32_t)(tr.state.counter >> 32);
+    std::vector<uint32_t> messages((size_t)n * points * D), challenges((size_t)n * D);
+    if ((status = s.run_device(state, messages.data(), challenges.data()))) return status;
+    for (int j = 0; j < n; j++) {
+      uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
+      if ((status = tr.send(&messages[(size_t)j * points * D], 2, dims, nullptr))) return status;
+      uint32_t *r = out_chal + (size_t)j * D;
+      tr.challenge(D, r);
+      if (memcmp(r, &challenges[(size_t)j * D], 4 * D) != 0) {
+        set_error("device-error: the device transcript drew a different challenge in round " + std::to_string(j));
+        return E_DEVICE;
+      }
+    }
+    return s.finish(out_finals, out_folded);
+  }
   uint32_t sums[16 * 8];
   for (int j = 0; j < n; j++) {
     if ((status = s.round_sums(sums))) return status;

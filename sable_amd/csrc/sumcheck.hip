@@ -75,10 +75,10 @@ __global__ __launch_bounds__(BLOCK) void fold_kernel(const uint32_t *in, uint32_
 
 // sums[o] = sum over the workgroups' partials: one workgroup per output word
 __global__ __launch_bounds__(BLOCK) void reduce_partials_kernel(const uint32_t *partials, uint32_t nblocks,
-                                                                uint32_t width, uint32_t *sums) {
+                                                                uint32_t stride, uint32_t *sums) {
   __shared__ uint32_t lds[BLOCK / 64];
   uint32_t o = blockIdx.x, v = 0;
-  for (uint32_t b = threadIdx.x; b < nblocks; b += BLOCK) v = fadd(v, partials[(uint64_t)b * width + o]);
+  for (uint32_t b = threadIdx.x; b < nblocks; b += BLOCK) v = fadd(v, partials[(uint64_t)b * stride + o]);
   v = wave_sum(v);
   if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
   __syncthreads();
@@ -100,6 +100,11 @@ static void launch_interp(const RoundArgs<D> &a, const StmtDesc &d, bool in_base
     hipLaunchKernelGGL((round_kernel_interp<D, false, true>), dim3(grid), dim3(BLOCK), 0, s, a, d);
   else
     hipLaunchKernelGGL((round_kernel_interp<D, false, false>), dim3(grid), dim3(BLOCK), 0, s, a, d);
+}
+
+template <int D>
+static void launch_tail_interp(const TailArgs<D> &a, const StmtDesc &d, hipStream_t s) {
+  hipLaunchKernelGGL((tail_kernel_interp<D>), dim3(1), dim3(BLOCK), 0, s, a, d);
 }
 
 // ------------------------------------------------------------------ registry of generated kernels
@@ -239,9 +244,15 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   }
   uint64_t pairs0 = size / 2;
   max_grid = pairs0 ? (pairs0 + BLOCK - 1) / BLOCK : 1;
-  if (max_grid > 8192) max_grid = 8192;
+  if (max_grid > 1024) max_grid = 1024;
+  pstride = next_pow2((uint64_t)std::max(st.nacc, 1) * D);
   uint64_t partial_off = pos * D;  // from here in words
-  uint64_t words = partial_off + (max_grid + 1) * (uint64_t)std::max(st.nacc, 1) * D + 64;
+  uint64_t words = partial_off + (max_grid + 1) * (uint64_t)pstride + 64;
+  // the device-driven loop's constants: control block | message map | constant-group terms
+  uint64_t ctrl_off = (words + 63) & ~(uint64_t)63;
+  uint64_t mt_off = ctrl_off + (sizeof(Ctrl) + 3) / 4;
+  uint64_t c0_off = mt_off + (uint64_t)points * std::max(st.nacc, 1) * D;
+  words = c0_off + (uint64_t)std::max(n, 1) * points * D + 64;
   // mixed base / extension inputs: lift the base ones
   bool any_base = false, all_base = true;
   for (int t = 0; t < T; t++) {
@@ -262,7 +273,10 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   uint32_t *base = (uint32_t *)c.misc.ptr;
   d_weights = base;
   d_partials = base + partial_off;
-  d_sums = d_partials + max_grid * (uint64_t)std::max(st.nacc, 1) * D;
+  d_sums = d_partials + max_grid * (uint64_t)pstride;
+  d_ctrl = reinterpret_cast<Ctrl *>(base + ctrl_off);
+  d_mtilde = base + mt_off;
+  d_c0 = base + c0_off;
 
   cur.assign(T, nullptr);
   cur_base = all_base;
@@ -342,7 +356,9 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   a.pairs_per_thread = ppt;
   a.deferred = do_sums && ((uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits)) ? 1 : 0;
   a.partials = s.d_partials;
-  if (fold)
+  a.pstride = s.pstride;
+  if (s.device_loop) a.ctrl = s.d_ctrl;
+  if (fold && !s.device_loop)
     for (int k = 0; k < D; k++) a.r_mont[k] = to_mont(s.pending_r[k]);
   uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
   {
@@ -356,13 +372,36 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   else
     launch_interp<D>(a, s.desc, s.cur_base, fold, grid, c.stream);
   c.prof_end();
-  if (do_sums) {
+  if (do_sums && s.device_loop) {
+    EpilogueArgs e;
+    e.partials = s.d_partials, e.nblocks = grid, e.pstride = s.pstride, e.nacc = (uint32_t)s.st.nacc;
+    e.points = (uint32_t)s.points, e.mtilde = s.d_mtilde, e.c0 = s.d_c0 + (size_t)j * s.points * D, e.ctrl = s.d_ctrl;
+    c.prof_begin("epilogue", j, 0);
+    if (D == 4)
+      hipLaunchKernelGGL(epilogue_kernel<4>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
+    else
+      hipLaunchKernelGGL(epilogue_kernel<8>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
+    c.prof_end();
+  }
+  if (do_sums && !s.device_loop) {
     uint32_t width = (uint32_t)s.st.nacc * D;
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3(width), dim3(BLOCK), 0, c.stream, s.d_partials, grid, width,
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3(width), dim3(BLOCK), 0, c.stream, s.d_partials, grid, s.pstride,
                        s.d_sums);
   }
   EXH_HIP(hipGetLastError());
   return OK;
+}
+
+// the total weight of round j's pairs, sum_h HIGH[h] sum_l LOW[l]: what a constant term is multiplied by
+static hf::E weight_sum(const SumcheckSession &s, int j) {
+  hf::E wsum = hf::lift(1, s.D);
+  uint64_t nl = (uint64_t)1 << s.low_bits[j];
+  if (!s.has_eq) wsum = hf::lift((uint32_t)(nl % P), s.D);
+  if (s.has_bw)
+    wsum = hf::mul(wsum, s.bw_sum);
+  else if (!s.has_eq)
+    wsum = hf::scale(wsum, (uint32_t)(s.n_high[j] % P));
+  return wsum;
 }
 
 int SumcheckSession::round_sums(uint32_t *out) {
@@ -403,15 +442,7 @@ int SumcheckSession::round_sums(uint32_t *out) {
 
   // ---- the message rows from the groups' sums
   // total weight of the pairs, for the constant group
-  hf::E wsum = hf::lift(1, D);
-  {
-    uint64_t nl = (uint64_t)1 << low_bits[j];
-    if (!has_eq) wsum = hf::lift((uint32_t)(nl % P), D);
-    if (has_bw)
-      wsum = hf::mul(wsum, bw_sum);
-    else if (!has_eq)
-      wsum = hf::scale(wsum, (uint32_t)(n_high[j] % P));
-  }
+  hf::E wsum = weight_sum(*this, j);
   if (claim_mode) {  // sum_g coef_g ((1 - r_0) G(0) + r_0 G(1)), or G(0) + G(1) without eq
     hf::E total = hf::zero(D), one = hf::lift(1, D);
     for (size_t g = 0; g < st.groups.size(); g++) {
@@ -523,6 +554,183 @@ int SumcheckSession::finish(uint32_t *finals, uint32_t *const *folded) {
       if (folded && folded[t]) memcpy(folded[t] + x * D, e, 4 * D);
     }
   }
+  return OK;
+}
+
+// ------------------------------------------------------------------ the device-driven loop
+constexpr uint64_t TAIL_PAIRS = 256;  // rounds with at most this many pairs run in the one-workgroup tail
+
+int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges) {
+  Context &c = ctx();
+  if (round != 0 || pending_fold || claim_mode || !device_capable()) {
+    set_error("invalid-parameter: the device loop starts a fresh session of at most 7 wire points");
+    return E_PARAM;
+  }
+  if (n == 0) return OK;
+  const int T = st.T(), nacc = st.nacc;
+  // ---- constants: control block, message map (times R), per-round constant terms
+  std::vector<uint32_t> up(((sizeof(Ctrl) + 3) / 4) + (size_t)points * std::max(nacc, 1) * D + (size_t)n * points * D, 0);
+  Ctrl *hc = reinterpret_cast<Ctrl *>(up.data());
+  hc->tr = state;
+  uint32_t *mt = up.data() + (sizeof(Ctrl) + 3) / 4, *c0 = mt + (size_t)points * std::max(nacc, 1) * D;
+  std::vector<int> wire(points);
+  for (int k = 0; k < points; k++) wire[k] = k == 0 ? 0 : k + 1;
+  for (size_t g = 0; g < st.groups.size(); g++) {
+    const Group &grp = st.groups[g];
+    hf::E coef(group_coef.begin() + g * D, group_coef.begin() + (g + 1) * D);
+    if (grp.tabs.empty()) {
+      for (int j = 0; j < n; j++) {
+        hf::E v = hf::mul(coef, weight_sum(*this, j));
+        for (int k = 0; k < points; k++)
+          for (int cc = 0; cc < D; cc++)
+            c0[((size_t)j * points + k) * D + cc] = fadd(c0[((size_t)j * points + k) * D + cc], v[cc]);
+      }
+      continue;
+    }
+    uint32_t fix = fpow(R1, grp.tabs.size());  // the sums carry R^-degree
+    bool direct = (int)grp.tabs.size() >= points;
+    for (size_t e = 0; e < grp.evalx.size(); e++) {
+      for (int k = 0; k < points; k++) {
+        uint32_t lag;  // the Lagrange basis of node e over the group's nodes, at wire point k
+        if (direct)
+          lag = (int)e == k ? 1u : 0u;
+        else {
+          uint32_t num = 1, den = 1;
+          for (size_t o = 0; o < grp.evalx.size(); o++) {
+            if (o == e) continue;
+            int64_t a = wire[k] - grp.evalx[o], b = grp.evalx[e] - grp.evalx[o];
+            num = fmul(num, (uint32_t)(((a % (int64_t)P) + P) % P));
+            den = fmul(den, (uint32_t)(((b % (int64_t)P) + P) % P));
+          }
+          lag = fmul(num, finv(den));
+        }
+        hf::E m = hf::scale(coef, fmul(lag, fix));
+        uint32_t *dst = mt + ((size_t)k * nacc + grp.acc_base + e) * D;
+        for (int cc = 0; cc < D; cc++) dst[cc] = to_mont(m[cc]);
+      }
+    }
+  }
+  EXH_HIP(hipMemcpyAsync(d_ctrl, up.data(), up.size() * 4, hipMemcpyHostToDevice, c.stream));
+  EXH_HIP(hipStreamSynchronize(c.stream));  // `up` is pageable host memory
+
+  device_loop = true;
+  bool tail_done = false;
+  int status = OK, j = 0;
+  for (; j < n && status == OK; j++) {
+    uint64_t n_pairs = (size / (j == 0 ? 1 : 2)) / 2;  // pairs summed in round j (after the pending fold)
+    if (n_pairs <= TAIL_PAIRS && n - j <= MAXTAIL && (!cur_base || j == 0)) break;
+    round = j;
+    if (j == 0) {
+      status = D == 4 ? launch_round<4>(*this, false, true, out_buf, n_pairs, j)
+                      : launch_round<8>(*this, false, true, out_buf, n_pairs, j);
+    } else {
+      uint64_t out_size = size / 2;
+      Arena &dst = (generation % 2 == 0) ? c.fold_a : c.fold_b;
+      out_buf.assign(T, nullptr);
+      for (int t = 0; t < T; t++) out_buf[t] = (uint32_t *)dst.ptr + (uint64_t)t * out_size * D;
+      status = D == 4 ? launch_round<4>(*this, true, true, out_buf, n_pairs, j)
+                      : launch_round<8>(*this, true, true, out_buf, n_pairs, j);
+      for (int t = 0; t < T; t++) cur[t] = out_buf[t];
+      cur_base = false;
+      size = out_size;
+      generation++;
+    }
+  }
+  if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
+    status = launch_tail(j);
+    tail_done = status == OK;
+  }
+  device_loop = false;
+  if (status) return status;
+  // ---- read the logs back: one copy, one wait
+  std::vector<uint32_t> logs((sizeof(Ctrl) + 3) / 4);
+  EXH_HIP(hipMemcpyAsync(logs.data(), d_ctrl, sizeof(Ctrl), hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  const Ctrl *rc = reinterpret_cast<const Ctrl *>(logs.data());
+  if ((int)rc->round != n) {
+    set_error("device-error: the device loop completed " + std::to_string(rc->round) + " of " + std::to_string(n) +
+              " rounds");
+    return E_DEVICE;
+  }
+  for (int r = 0; r < n; r++) {
+    memcpy(messages + (size_t)r * points * D, rc->msg[r], (size_t)points * D * 4);
+    memcpy(challenges + (size_t)r * D, rc->chal[r], (size_t)D * 4);
+  }
+  round = n;
+  pending_fold = !tail_done;  // without a tail the last challenge's fold is still to do
+  if (pending_fold) memcpy(pending_r, rc->chal[n - 1], (size_t)D * 4);
+  return OK;
+}
+
+int SumcheckSession::launch_tail(int j) {
+  Context &c = ctx();
+  const int T = st.T();
+  const bool first_fold = j > 0;
+  if (cur_base) {  // the tail reads extension tables: lift base inputs (a tiny sumcheck)
+    if (first_fold) {
+      set_error("device-error: base tables with a pending fold at the tail");
+      return E_DEVICE;
+    }
+    int status = c.fold_b.reserve((size_t)T * size * D * 4 * 2);
+    if (status) return status;
+    uint32_t *dst = (uint32_t *)c.fold_b.ptr + (uint64_t)T * size * D;  // above the generations' area
+    for (int t = 0; t < T; t++) {
+      uint32_t grid = (uint32_t)((size + BLOCK - 1) / BLOCK);
+      if (D == 4)
+        hipLaunchKernelGGL(lift_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], dst, size);
+      else
+        hipLaunchKernelGGL(lift_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], dst, size);
+      cur[t] = dst;
+      dst += size * D;
+    }
+    cur_base = false;
+  }
+  auto fill = [&](auto &a) {
+    memset(&a, 0, sizeof(a));
+    for (int t = 0; t < T; t++) a.in[t] = cur[t];
+    a.buf[0] = (uint32_t *)c.fold_a.ptr;
+    a.buf[1] = (uint32_t *)c.fold_b.ptr;
+    a.weights = d_weights;
+    a.entries = size;
+    a.first_fold = first_fold ? 1 : 0;
+    a.rounds = (uint32_t)(n - j);
+    a.generation = (uint32_t)generation;
+    a.points = (uint32_t)points;
+    a.ctrl = d_ctrl;
+    a.mtilde = d_mtilde;
+    a.c0 = d_c0 + (size_t)j * points * D;
+    for (int jj = 0; jj < n - j; jj++) {
+      a.low_off[jj] = low_off[j + jj];
+      a.high_off[jj] = high_off[j + jj];
+      a.low_bits[jj] = (uint32_t)low_bits[j + jj];
+    }
+  };
+  c.prof_begin("tail", j, 0);
+  if (D == 4) {
+    TailArgs<4> a;
+    fill(a);
+    if (generated)
+      kernels->launch_tail(&a, c.stream);
+    else
+      launch_tail_interp<4>(a, desc, c.stream);
+  } else {
+    TailArgs<8> a;
+    fill(a);
+    if (generated)
+      kernels->launch_tail(&a, c.stream);
+    else
+      launch_tail_interp<8>(a, desc, c.stream);
+  }
+  c.prof_end();
+  EXH_HIP(hipGetLastError());
+  // where the tail leaves the tables: it folds (first_fold ? 1 : 0) + (n - j) times, alternating arenas
+  int folds = (first_fold ? 1 : 0) + (n - j);
+  uint64_t final_size = size >> folds;
+  int last_gen = generation + folds - 1;
+  Arena &dst = (last_gen % 2 == 0) ? c.fold_a : c.fold_b;
+  for (int t = 0; t < T; t++) cur[t] = (uint32_t *)dst.ptr + (uint64_t)t * final_size * D;
+  size = final_size;
+  generation += folds;
   return OK;
 }
 

@@ -14,6 +14,7 @@ namespace exh {
 
 struct KernelSet {  // the launchers generated for one statement and one degree D
   void (*launch)(const void *args, bool in_base, bool fold, uint32_t grid, hipStream_t stream);
+  void (*launch_tail)(const void *args, hipStream_t stream);
 };
 void register_kernels(const std::string &key, int D, KernelSet set);
 const KernelSet *find_kernels(const std::string &key, int D);
@@ -39,6 +40,10 @@ struct SumcheckSession {
   std::vector<uint64_t> n_high;
   uint32_t *d_partials = nullptr, *d_sums = nullptr, *d_lifted = nullptr;
   uint64_t max_grid = 0;
+  uint32_t pstride = 0;  // words per workgroup partial
+  bool device_loop = false;
+  Ctrl *d_ctrl = nullptr;
+  uint32_t *d_mtilde = nullptr, *d_c0 = nullptr;
   bool pending_fold = false;
   uint32_t pending_r[8];
   int generation = 0;
@@ -53,6 +58,12 @@ struct SumcheckSession {
   bool claim_mode = false;
   std::vector<uint32_t> eq0;  // the eq point's first coordinate, for the claim
   int round_sums(uint32_t *out /* points * D */);
+  // All rounds on the device without a host round trip: the transcript runs on the device from the
+  // given B3S state; afterwards messages[j] (points * D words) and challenges[j] (D words) hold what
+  // was sent and drawn, and the session is ready for finish().  Needs points <= MAXPTS.
+  int run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges);
+  int launch_tail(int first_round);
+  bool device_capable() const { return points <= MAXPTS && n <= MAXROUNDS; }
   int fold(const uint32_t *r /* D */);
   // finals: T * D; folded[t] (optional): K * D each
   int finish(uint32_t *finals, uint32_t *const *folded);

@@ -18,12 +18,27 @@
 
 #include <type_traits>
 
+#include "dev_transcript.cuh"
 #include "field.cuh"
 #include "stmtdesc.hpp"
 
 namespace exh {
 
 // StmtDesc and the limits MAXT, MAXG, ... come from stmtdesc.hpp
+constexpr int MAXROUNDS = 48;  // rounds of one device-driven sumcheck
+constexpr int MAXPTS = 7;      // wire points of a device-driven round message
+constexpr int MAXTAIL = 16;    // rounds the tail kernel can take
+
+// The control block of a device-driven sumcheck, in device memory: the transcript state, the current
+// fold challenge, the launch's completion counter and the logs the host reads back at the end.
+struct Ctrl {
+  DevB3S tr;
+  uint32_t r_mont[8];
+  uint32_t round;  // rounds completed
+  uint32_t pad[3];
+  uint32_t msg[MAXROUNDS][MAXPTS * 8];
+  uint32_t chal[MAXROUNDS][8];
+};
 template <int D>
 struct RoundArgs {
   const uint32_t *in[MAXT];  // the tables read: 4 entries per pair when folding, else 2
@@ -36,7 +51,27 @@ struct RoundArgs {
   uint32_t pairs_per_thread;
   uint32_t deferred;         // every workgroup's pairs share one h: HIGH[h] applied once per workgroup
   uint32_t do_sums;
-  uint32_t r_mont[D];        // the fold challenge, times R
+  uint32_t r_mont[D];        // the fold challenge, times R (host-driven rounds)
+  Ctrl *ctrl;                // device-driven rounds: the fold challenge is read from here (else null)
+  uint32_t pstride;          // words per workgroup partial (a power of two >= nacc * D)
+};
+
+// the rounds at the end of a sumcheck, all in one workgroup (tables of at most a few thousand entries)
+template <int D>
+struct TailArgs {
+  const uint32_t *in[MAXT];  // extension tables of `entries` entries each
+  uint32_t *buf[2];          // the two generations' arenas; table t of a generation of E entries is at t * E * D
+  const uint32_t *weights;   // base of the weight tables
+  uint64_t low_off[MAXTAIL], high_off[MAXTAIL];  // in EXTs, per tail round
+  uint32_t low_bits[MAXTAIL];
+  uint64_t entries;
+  uint32_t first_fold;       // fold by ctrl's challenge before the first tail round
+  uint32_t rounds;           // rounds summed here; one more fold follows the last
+  uint32_t generation;       // parity of the arena the next fold writes
+  uint32_t points;
+  Ctrl *ctrl;
+  const uint32_t *mtilde;
+  const uint32_t *c0;        // [rounds][points][D]
 };
 
 template <int D>
@@ -133,11 +168,122 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
   }
 }
 
-// cross-lane sum of a canonical value over the 64 lanes of a wavefront
+// cross-lane sum of a canonical value over the 64 lanes of a wavefront: four DPP butterfly steps inside
+// each row of 16 lanes (no LDS traffic), then the four row sums through read-lane
+#define EXH_DPP(v, ctrl) ((uint32_t)__builtin_amdgcn_update_dpp(0, (int)(v), (ctrl), 0xf, 0xf, false))
 __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+  v = fadd(v, EXH_DPP(v, 0xB1));   // quad_perm [1,0,3,2]
+  v = fadd(v, EXH_DPP(v, 0x4E));   // quad_perm [2,3,0,1]
+  v = fadd(v, EXH_DPP(v, 0x141));  // row_half_mirror
+  v = fadd(v, EXH_DPP(v, 0x140));  // row_mirror
+  uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+  uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+  return fadd(fadd(a, b), fadd(c, d));
+}
+
+// the pair (lo, hi) of every table at pair index i, folding first when FOLD
+template <int D, bool IN_BASE, bool FOLD, class V, class Desc>
+__device__ __forceinline__ void load_pair(const Desc &d, const uint32_t *const *in, uint32_t *const *out, uint64_t i,
+                                          const Ext<D> &r, V *lo, V *hi) {
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fadd(v, (uint32_t)__shfl_xor((int)v, off, 64));
-  return v;
+  for (int t = 0; t < MAXT; t++) {
+    if (t < d.T) {
+      if constexpr (FOLD && IN_BASE) {
+        uint4 e = *reinterpret_cast<const uint4 *>(in[t] + 4 * i);
+        lo[t] = fold_base<D>(e.x, e.y, r);
+        hi[t] = fold_base<D>(e.z, e.w, r);
+      } else if constexpr (FOLD) {
+        const uint32_t *p = in[t] + 4 * i * D;
+        lo[t] = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
+        hi[t] = fold_ext<D>(load_ext<D>(p + 2 * D), load_ext<D>(p + 3 * D), r);
+      } else if constexpr (IN_BASE) {
+        uint2 e = *reinterpret_cast<const uint2 *>(in[t] + 2 * i);
+        lo[t] = e.x;
+        hi[t] = e.y;
+      } else {
+        const uint32_t *p = in[t] + 2 * i * D;
+        lo[t] = load_ext<D>(p);
+        hi[t] = load_ext<D>(p + D);
+      }
+      if constexpr (FOLD) {
+        store_ext<D>(out[t] + 2 * i * D, lo[t]);
+        store_ext<D>(out[t] + (2 * i + 1) * D, hi[t]);
+      }
+    }
+  }
+}
+
+// the workgroup's sums of every accumulator, reduced mod p, into sums[nacc * D] (LDS); all threads call
+template <int D, class Desc>
+__device__ __forceinline__ void block_sums(const Desc &d, Acc96 (*acc)[D], uint32_t (*lds)[MAXACC * D],
+                                           uint32_t *sums) {
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+  for (int a = 0; a < MAXACC; a++) {
+    if (a < d.nacc) {
+#pragma unroll
+      for (int c = 0; c < D; c++) {
+        uint32_t v = wave_sum(acc_reduce(acc[a][c]));
+        if (lane == 0) lds[wave][a * D + c] = v;
+      }
+    }
+  }
+  __syncthreads();
+  for (uint32_t o = tid; o < (uint32_t)d.nacc * D; o += BLOCK) {
+    uint32_t v = lds[0][o];
+#pragma unroll
+    for (int wv = 1; wv < BLOCK / 64; wv++) v = fadd(v, lds[wv][o]);
+    sums[o] = v;
+  }
+  __syncthreads();
+}
+
+// From the round's accumulator sums (LDS, nacc * D words, scaled as the kernels leave them) to the round
+// message, through the transcript, to the next challenge: rows = mtilde * sums + c0
+// (ROUND-MESSAGE, src/sumcheck.lisp:313-317), send = absorb the rows (src/transcript.lisp:116-128),
+// r = challenge (src/transcript.lisp:174-176).  All threads of the workgroup call; scratch is LDS.
+struct EpilogueLds {
+  uint32_t prod[MAXPTS * MAXACC * 8];
+  uint32_t msg[MAXPTS * 8];
+  uint32_t chal[8];
+  uint32_t r_mont[8];
+  uint32_t ring[32];
+};
+
+template <int D>
+__device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums, uint32_t nacc, uint32_t points,
+                                               const uint32_t *mtilde, const uint32_t *c0, EpilogueLds *e) {
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
+  for (uint32_t u = tid; u < points * nacc; u += nthreads) {
+    uint32_t a = u % nacc;
+    Ext<D> m = load_ext<D>(mtilde + (size_t)u * D), sv;
+#pragma unroll
+    for (int c = 0; c < D; c++) sv.c[c] = sums[a * D + c];
+    Ext<D> pr = ext_mul_mont<D>(m, sv);
+#pragma unroll
+    for (int c = 0; c < D; c++) e->prod[u * D + c] = pr.c[c];
+  }
+  __syncthreads();
+  for (uint32_t o = tid; o < points * D; o += nthreads) {
+    uint32_t k = o / D, c = o % D, v = c0[o];
+    for (uint32_t a = 0; a < nacc; a++) v = fadd(v, e->prod[(k * nacc + a) * D + c]);
+    e->msg[o] = v;
+  }
+  __syncthreads();
+  if (tid < 64) {  // the first wavefront runs the transcript, every lane the same steps
+    const uint32_t round = ctrl->round;
+    RunB3S tr;
+    rb3s_load(tr, e->ring, &ctrl->tr);
+    dev_absorb_words(tr, e->msg, points * D);
+    dev_challenge(tr, D, e->chal);
+    rb3s_store(tr, &ctrl->tr);
+    for (uint32_t o = tid; o < points * D; o += 64) ctrl->msg[round][o] = e->msg[o];
+    if (tid < (uint32_t)D) {
+      ctrl->chal[round][tid] = e->chal[tid];
+      ctrl->r_mont[tid] = e->r_mont[tid] = to_mont(e->chal[tid]);
+    }
+    if (tid == 0) ctrl->round = round + 1;
+  }
 }
 
 template <int D, bool IN_BASE, bool FOLD, class Desc>
@@ -155,42 +301,18 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
 #pragma unroll
     for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
 
-  Ext<D> r;
+  Ext<D> r = ext_zero<D>();
   if constexpr (FOLD) {
+    const uint32_t *rp = args.ctrl ? args.ctrl->r_mont : args.r_mont;
 #pragma unroll
-    for (int c = 0; c < D; c++) r.c[c] = args.r_mont[c];
+    for (int c = 0; c < D; c++) r.c[c] = rp[c];
   }
 
   for (uint32_t k = 0; k < args.pairs_per_thread; k++) {
     const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
     if (i >= args.n_pairs) break;
     V lo[MAXT], hi[MAXT];
-#pragma unroll
-    for (int t = 0; t < MAXT; t++) {
-      if (t < d.T) {
-        if constexpr (FOLD && IN_BASE) {
-          uint4 e = *reinterpret_cast<const uint4 *>(args.in[t] + 4 * i);
-          lo[t] = fold_base<D>(e.x, e.y, r);
-          hi[t] = fold_base<D>(e.z, e.w, r);
-        } else if constexpr (FOLD) {
-          const uint32_t *p = args.in[t] + 4 * i * D;
-          lo[t] = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
-          hi[t] = fold_ext<D>(load_ext<D>(p + 2 * D), load_ext<D>(p + 3 * D), r);
-        } else if constexpr (IN_BASE) {
-          uint2 e = *reinterpret_cast<const uint2 *>(args.in[t] + 2 * i);
-          lo[t] = e.x;
-          hi[t] = e.y;
-        } else {
-          const uint32_t *p = args.in[t] + 2 * i * D;
-          lo[t] = load_ext<D>(p);
-          hi[t] = load_ext<D>(p + D);
-        }
-        if constexpr (FOLD) {
-          store_ext<D>(args.out[t] + 2 * i * D, lo[t]);
-          store_ext<D>(args.out[t] + (2 * i + 1) * D, hi[t]);
-        }
-      }
-    }
+    load_pair<D, IN_BASE, FOLD, V>(d, args.in, args.out, i, r, lo, hi);
     if (args.do_sums) {
       Ext<D> w = load_ext<D>(args.low + (i & low_mask) * D);
       if (!args.deferred) w = ext_mul_mont<D>(w, load_ext<D>(args.high + (i >> args.low_bits) * D));
@@ -199,31 +321,120 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
   }
   if (!args.do_sums) return;
 
-  // reduce: thread -> wavefront -> workgroup
   __shared__ uint32_t lds[BLOCK / 64][MAXACC * D];
-  const uint32_t lane = tid & 63, wave = tid >> 6;
-#pragma unroll
-  for (int a = 0; a < MAXACC; a++) {
-    if (a < d.nacc) {
-#pragma unroll
-      for (int c = 0; c < D; c++) {
-        uint32_t v = wave_sum(acc_reduce(acc[a][c]));
-        if (lane == 0) lds[wave][a * D + c] = v;
-      }
-    }
-  }
-  __syncthreads();
+  __shared__ uint32_t sums[MAXACC * D];
+  block_sums<D>(d, acc, lds, sums);
   if (tid < (uint32_t)d.nacc) {
     Ext<D> s;
 #pragma unroll
-    for (int c = 0; c < D; c++) {
-      uint32_t v = lds[0][tid * D + c];
-#pragma unroll
-      for (int wv = 1; wv < BLOCK / 64; wv++) v = fadd(v, lds[wv][tid * D + c]);
-      s.c[c] = v;
-    }
+    for (int c = 0; c < D; c++) s.c[c] = sums[tid * D + c];
     if (args.deferred) s = ext_mul_mont<D>(s, load_ext<D>(args.high + (tile_start >> args.low_bits) * D));
-    store_ext<D>(args.partials + ((uint64_t)blockIdx.x * d.nacc + tid) * D, s);
+    store_ext<D>(args.partials + (uint64_t)blockIdx.x * args.pstride + tid * D, s);
+  }
+}
+
+// The round's second launch when the device drives the loop: one workgroup adds the partials, forms the
+// message, runs the transcript and leaves the next challenge in ctrl.  (A last-workgroup-done scheme
+// inside the round kernel needs a device-scope fence per workgroup, which on this part writes back the
+// XCD's whole L2 and costs more than a launch.)
+struct EpilogueArgs {
+  const uint32_t *partials;
+  uint32_t nblocks, pstride, nacc, points;
+  const uint32_t *mtilde, *c0;
+  Ctrl *ctrl;
+};
+
+constexpr int EPI_BLOCK = 1024;
+
+template <int D>
+__global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) {
+  __shared__ uint32_t scratch[EPI_BLOCK];
+  __shared__ uint32_t sums[MAXACC * D];
+  __shared__ EpilogueLds epi;
+  const uint32_t tid = threadIdx.x, width = args.nacc * D, ps = args.pstride;
+  // sums[o] = sum over workgroups of partial[o]: thread t takes column t % pstride of the rows
+  // t / pstride, t / pstride + rstep, ...; four loads in flight per thread
+  for (uint32_t col0 = 0; col0 < ps; col0 += EPI_BLOCK) {
+    const uint32_t col = col0 + (ps < EPI_BLOCK ? tid % ps : tid);
+    const uint32_t row0 = ps < EPI_BLOCK ? tid / ps : 0, rstep = ps < EPI_BLOCK ? EPI_BLOCK / ps : 1;
+    uint32_t v0 = 0, v1 = 0, v2 = 0, v3 = 0;
+    if (col < width) {
+      const uint32_t *p = args.partials + col;
+      uint32_t b = row0;
+      for (; b + 3 * rstep < args.nblocks; b += 4 * rstep) {
+        uint32_t x0 = p[(uint64_t)b * ps], x1 = p[(uint64_t)(b + rstep) * ps], x2 = p[(uint64_t)(b + 2 * rstep) * ps],
+                 x3 = p[(uint64_t)(b + 3 * rstep) * ps];
+        v0 = fadd(v0, x0), v1 = fadd(v1, x1), v2 = fadd(v2, x2), v3 = fadd(v3, x3);
+      }
+      for (; b < args.nblocks; b += rstep) v0 = fadd(v0, p[(uint64_t)b * ps]);
+    }
+    __syncthreads();
+    scratch[tid] = fadd(fadd(v0, v1), fadd(v2, v3));
+    __syncthreads();
+    if (tid < (ps < EPI_BLOCK ? ps : EPI_BLOCK) && col0 + tid < width) {
+      uint32_t total = scratch[tid];
+      for (uint32_t g = 1; g < rstep; g++) total = fadd(total, scratch[g * ps + tid]);
+      sums[col0 + tid] = total;
+    }
+  }
+  __syncthreads();
+  round_epilogue<D>(args.ctrl, sums, args.nacc, args.points, args.mtilde, args.c0, &epi);
+}
+
+// The last rounds in one workgroup: [fold], then per round sums -> message -> challenge -> fold.
+template <int D, class Desc>
+__device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args) {
+  const uint32_t tid = threadIdx.x;
+  __shared__ uint32_t lds[BLOCK / 64][MAXACC * D];
+  __shared__ uint32_t sums[MAXACC * D];
+  __shared__ EpilogueLds epi;
+  const uint32_t *cur[MAXT];
+#pragma unroll
+  for (int t = 0; t < MAXT; t++) cur[t] = t < d.T ? args.in[t] : nullptr;
+  uint64_t entries = args.entries;
+  uint32_t gen = args.generation;
+  // one fold of every table by ctrl's challenge, into the next generation
+  auto fold_all = [&](const uint32_t *r_mont) {
+    Ext<D> r;
+#pragma unroll
+    for (int c = 0; c < D; c++) r.c[c] = r_mont[c];
+    const uint64_t out_entries = entries / 2;
+    uint32_t *dst = args.buf[gen & 1];
+#pragma unroll
+    for (int t = 0; t < MAXT; t++) {
+      if (t < d.T) {
+        uint32_t *o = dst + (uint64_t)t * out_entries * D;
+        for (uint64_t x = tid; x < out_entries; x += BLOCK)
+          store_ext<D>(o + x * D, fold_ext<D>(load_ext<D>(cur[t] + 2 * x * D), load_ext<D>(cur[t] + (2 * x + 1) * D), r));
+        cur[t] = o;
+      }
+    }
+    entries = out_entries;
+    gen++;
+    __threadfence();  // the folded entries are read back by other lanes of this workgroup
+    __syncthreads();
+    __threadfence();
+  };
+  if (args.first_fold) fold_all(args.ctrl->r_mont);
+  for (uint32_t jj = 0; jj < args.rounds; jj++) {
+    Acc96 acc[MAXACC][D];
+#pragma unroll
+    for (int a = 0; a < MAXACC; a++)
+#pragma unroll
+      for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
+    const uint64_t n_pairs = entries / 2, low_mask = ((uint64_t)1 << args.low_bits[jj]) - 1;
+    const uint32_t *low = args.weights + args.low_off[jj] * D, *high = args.weights + args.high_off[jj] * D;
+    for (uint64_t i = tid; i < n_pairs; i += BLOCK) {
+      Ext<D> lo[MAXT], hi[MAXT], r0 = ext_zero<D>();
+      load_pair<D, false, false, Ext<D>>(d, cur, nullptr, i, r0, lo, hi);
+      Ext<D> w = ext_mul_mont<D>(load_ext<D>(low + (i & low_mask) * D), load_ext<D>(high + (i >> args.low_bits[jj]) * D));
+      accumulate_pair<D, Ext<D>>(d, lo, hi, w, acc);
+    }
+    block_sums<D>(d, acc, lds, sums);
+    round_epilogue<D>(args.ctrl, sums, (uint32_t)d.nacc, args.points, args.mtilde,
+                      args.c0 + (size_t)jj * args.points * D, &epi);
+    __syncthreads();
+    fold_all(epi.r_mont);
   }
 }
 
@@ -232,13 +443,19 @@ template <int D, bool IN_BASE, bool FOLD, class S>
 __global__ __launch_bounds__(BLOCK) void round_kernel(RoundArgs<D> args) {
   round_body<D, IN_BASE, FOLD>(S::d, args);
 }
+template <int D, class S>
+__global__ __launch_bounds__(BLOCK) void tail_kernel(TailArgs<D> args) {
+  tail_body<D>(S::d, args);
+}
 
-// the interpreter: the same body over a run-time descriptor
+// the interpreter: the same bodies over a run-time descriptor
 template <int D, bool IN_BASE, bool FOLD>
 __global__ __launch_bounds__(BLOCK) void round_kernel_interp(RoundArgs<D> args, StmtDesc d) {
   round_body<D, IN_BASE, FOLD>(d, args);
 }
-
-typedef void (*RoundLauncher)(const void *args, int D, bool in_base, bool fold, uint32_t grid, hipStream_t stream);
+template <int D>
+__global__ __launch_bounds__(BLOCK) void tail_kernel_interp(TailArgs<D> args, StmtDesc d) {
+  tail_body<D>(d, args);
+}
 
 }  // namespace exh
