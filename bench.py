@@ -69,8 +69,182 @@ def cpu_baseline(n_sample, d, seed):
                       f"{dt:.1f} s); the reference's Lisp prover cannot run here (no SBCL)"}
 
 
+def run_sumcheck_config(sa, name, form, tables, consts, n, d, seed, steps, warmup, cpu_n):
+    """A sumcheck workload other than the headline one: same timing rules, one JSON line."""
+    st = sa.Statement(form, tables, consts)
+    T = len(tables)
+    dev = [sa.Table.random(seed * 1000 + k, 1 << n) for k in range(T)]
+    eq = splitmix_field(seed + 900, n * d).reshape(n, d)
+    cv = splitmix_field(seed + 901, d * max(len(consts), 1)).reshape(-1, d) if consts else None
+
+    def step():
+        tr = sa.Transcript(name, d)
+        sa.prove(tr, n, st, dev, eq=eq, constants=cv)
+        return tr
+
+    for _ in range(warmup):
+        step()
+    sa.check(sa.load().exh_synchronize())
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tr = step()
+    sa.check(sa.load().exh_synchronize())
+    dt = (time.perf_counter() - t0) / steps
+    sa.check(sa.load().exh_profile_enable(1))
+    for _ in range(steps):
+        step()
+    by_kernel = {}
+    for kname, rnd, ms, nbytes in profile_entries(sa):
+        k = by_kernel.setdefault((kname, rnd), [0.0, 0, nbytes])
+        k[0] += ms
+        k[1] += 1
+    sa.check(sa.load().exh_profile_enable(0))
+    (kname, kround), (ktotal, kcalls, kbytes) = max(by_kernel.items(), key=lambda kv: kv[1][0])
+    avg_ms = ktotal / kcalls
+    achieved = kbytes / (avg_ms * 1e-3) / 1e9
+    points = max(st.degree, 1)
+    out = {"metric": f"sumcheck table entries/s ({name})", "value": T * (1 << n) / dt, "unit": "table entries/s",
+           "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": 1e3 * dt, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": f"u32 (Montgomery KoalaBear, F_p^{d} tower)",
+           "data": "synthetic (SplitMix64-seeded uniform field elements)",
+           "config": {"workload": f"sumcheck prove of {form}, eq mode, n={n}, {T} base tables, F_p^{d}",
+                      "generated_kernel": st.has_generated_kernel(d), "proof_bytes": len(tr.proof()),
+                      "proof_sha256": hashlib.sha256(tr.proof()).hexdigest()},
+           "loop_hbm_fraction": T * (1 << n) * (8 + 8 * d) / dt / (HBM_PEAK_GBS * 1e9),
+           "roofline": {"bound": "hbm", "kernel": f"{kname} (round {kround})", "achieved": achieved,
+                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                        "avg_launch_ms": avg_ms, "alg_bytes_per_launch": kbytes, "traffic": None}}
+    assert len(tr.proof()) == 12 + n * (18 + 4 * points * d)
+    if cpu_n > 0:
+        from oracle import binding as orc
+        ost = orc.Statement(form, tables, consts)
+        ht = [splitmix_field(seed * 1000 + k, 1 << cpu_n) for k in range(T)]
+        heq = splitmix_field(seed + 900, cpu_n * d).reshape(cpu_n, d)
+        t0 = time.perf_counter()
+        orc.prove(orc.Transcript(name, d), cpu_n, ost, ht, eq=heq, constants=cv)
+        cdt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": T * (1 << cpu_n) / cdt, "unit": "table entries/s", "cores": 1, "kind": "port",
+                               "sample": f"same statement at n={cpu_n} ({cdt:.1f} s)"}
+    for t in dev:
+        t.free()
+    return out
+
+
+def run_gkr(sa, steps, warmup, cpu_n):
+    """Config 4: LogUp-GKR of 2^22 int8-range lookups into a 2^16-entry range table.  The witness tree has
+    leaves (1, Z - v_i), n = 22; the table tree leaves (m_j, Z - t_j), n = 16, t_j = j - 32768, m_j the exact
+    multiplicities; both roots are equal as fractions.  A step = prove-upper of both trees (fraction trees +
+    every layer's sumcheck)."""
+    d, nw, nt, seed = 4, 22, 16, 4
+    rng = np.random.default_rng(seed)
+    values = rng.integers(-128, 128, 1 << nw)
+    table = np.arange(1 << nt) - 32768
+    mult = np.bincount(values + 32768, minlength=1 << nt)
+    z = sa.Transcript("config4-z", d).challenge()
+
+    def leaves(num, val):
+        P = sa.P
+        p = np.zeros((len(num), d), np.uint32)
+        p[:, 0] = np.asarray(num, np.int64) % P
+        q = np.tile(z.astype(np.int64), (len(val), 1))
+        q[:, 0] = (q[:, 0] - np.asarray(val, np.int64)) % P
+        return p, q.astype(np.uint32)
+
+    wit = [sa.Table.upload(a) for a in leaves(np.ones(1 << nw, np.int64), values)]
+    tab = [sa.Table.upload(a) for a in leaves(mult, table)]
+
+    def step():
+        tw, tt = sa.Transcript("config4-w", d), sa.Transcript("config4-t", d)
+        sa.prove_upper(tw, nw, 1, [tuple(wit)])
+        sa.prove_upper(tt, nt, 1, [tuple(tab)])
+        return tw, tt
+
+    for _ in range(warmup):
+        step()
+    sa.check(sa.load().exh_synchronize())
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tw, tt = step()
+    sa.check(sa.load().exh_synchronize())
+    dt = (time.perf_counter() - t0) / steps
+    from oracle import binding as orc
+    rw, rt = orc.decode_proof(tw.proof())[0], orc.decode_proof(tt.proof())[0]
+    same_fraction = np.array_equal(orc.ext_mul(rw[0], rt[1]), orc.ext_mul(rt[0], rw[1]))
+    # algorithmic bytes of prove-upper per tree (16 B entries): tree build 3 * 2 * 2^n * 16 - ..., layer sumchecks
+    def alg(n):
+        build = sum(2 * (2 << m) * 16 + 2 * (1 << m) * 16 for m in range(n))
+        layers = sum(4 * (4 * (1 << l) * 16) for l in range(n - 1))
+        return build + layers
+    nbytes = alg(nw) + alg(nt)
+    out = {"metric": "LogUp-GKR prove-upper lookups/s (config 4)", "value": (1 << nw) / dt, "unit": "lookups/s",
+           "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": 1e3 * dt, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "u32 (Montgomery KoalaBear, F_p^4 tower)",
+           "data": "synthetic (seeded uniform int8 lookups, exact multiplicities)",
+           "config": {"workload": "LogUp-GKR: 2^22 int8-range lookups into a 2^16-entry table, witness tree n=22 + "
+                                  "table tree n=16, F_p^4, prove-upper of both", "roots_equal_as_fractions": bool(same_fraction),
+                      "proof_bytes": len(tw.proof()) + len(tt.proof())},
+           "roofline": {"bound": "hbm", "kernel": "prove-upper (whole: tree build + 36 layer sumchecks)",
+                        "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "alg_bytes": nbytes, "traffic": None}}
+    if cpu_n > 0:
+        rng = np.random.default_rng(1)
+        p = rng.integers(0, sa.P, (1 << cpu_n, d), dtype=np.uint32)
+        q = rng.integers(1, sa.P, (1 << cpu_n, d), dtype=np.uint32)
+        t0 = time.perf_counter()
+        orc.gkr_prove_upper(orc.Transcript("config4-w", d), cpu_n, 1, [(p, q)])
+        cdt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": (1 << cpu_n) / cdt, "unit": "lookups/s", "cores": 1, "kind": "port",
+                               "sample": f"prove-upper of one tree of 2^{cpu_n} leaves ({cdt:.1f} s)"}
+    return out
+
+
+def run_commit(sa, steps, warmup, cpu_c):
+    """Config 5 as the reference runs it: 2^24 coefficients = two columns of 2^23 (the code's domain is capped
+    at 2^24 points), rate-1/2 encode to two codewords of 2^24, 2^22 BLAKE3 leaves, Merkle levels, cap of 128."""
+    c, ncols = 23, 2
+    cols = sa.Table.random(5005, ncols << c)
+
+    def step():
+        tr = sa.Transcript("config5", 4)
+        cw, levels = sa.pcs_commit(tr, cols, ncols, c)
+        cw.free(), levels.free()
+        return tr
+
+    for _ in range(warmup):
+        step()
+    sa.check(sa.load().exh_synchronize())
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tr = step()
+    sa.check(sa.load().exh_synchronize())
+    dt = (time.perf_counter() - t0) / steps
+    nleaves = 1 << (c - 1)
+    nbytes = ncols * (4 << c) + ncols * (4 << (c + 1)) + ncols * (4 << (c + 1)) + 32 * nleaves + 64 * (nleaves - 1) + 32 * (nleaves - 1)
+    out = {"metric": "BaseFold commit ms (config 5)", "value": 1e3 * dt, "unit": "ms", "n_gpus": 1, "steps": steps,
+           "warmup": warmup, "ms_per_step": 1e3 * dt, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+           "dtype": "u32 (Montgomery KoalaBear) + BLAKE3", "data": "synthetic (SplitMix64-seeded uniform field elements)",
+           "config": {"workload": "pcs-commit: 2 columns of 2^23 coefficients -> 2 codewords of 2^24, 2^22 leaves, "
+                                  "Merkle levels, cap of 128 digests", "cap_sha256": hashlib.sha256(tr.proof()).hexdigest(),
+                      "leaf_hashes_per_s": nleaves / dt, "butterflies_per_s": ncols * 23 * (1 << 23) / dt},
+           "roofline": {"bound": "hbm", "kernel": "encode + leaves + Merkle (whole commit)", "achieved": nbytes / dt / 1e9,
+                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS,
+                        "alg_bytes": nbytes, "traffic": None}}
+    if cpu_c > 0:
+        from oracle import binding as orc
+        hc = [splitmix_field(77 + k, 1 << cpu_c) for k in range(ncols)]
+        t0 = time.perf_counter()
+        orc.commit_columns(hc, cpu_c)
+        cdt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": 1e3 * cdt * (1 << (c - cpu_c)), "unit": "ms", "cores": 1, "kind": "port",
+                               "sample": f"commit of 2 columns of 2^{cpu_c} ({cdt:.1f} s), scaled linearly by 2^{c - cpu_c} "
+                                         "(ignores the log factor of the encoder, so it flatters the CPU)"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5"],
+                    help="config2 (default) is the headline; the others are the remaining configured workloads")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -83,6 +257,21 @@ def main():
 
     import sable_amd as sa
     sa.init(0)
+    if args.workload == "config1":
+        print(json.dumps(run_sumcheck_config(sa, "config1", "(* t0 t1)", ["t0", "t1"], [], 16, 4, 1, args.steps,
+                                             args.warmup, 16 if args.cpu_n else 0)))
+        return
+    if args.workload == "config3":
+        print(json.dumps(run_sumcheck_config(sa, "config3", "(* (+ c0 3) (- c1 c0) c2 c3)", ["c0", "c1", "c2", "c3"], [],
+                                             26 if args.n == 24 else args.n, 8, 3, args.steps, args.warmup,
+                                             18 if args.cpu_n else 0)))
+        return
+    if args.workload == "config4":
+        print(json.dumps(run_gkr(sa, args.steps, args.warmup, 18 if args.cpu_n else 0)))
+        return
+    if args.workload == "config5":
+        print(json.dumps(run_commit(sa, args.steps, args.warmup, 18 if args.cpu_n else 0)))
+        return
     n, d, seed = args.n, 4, 2
     st = sa.Statement(FORM, TABLES, CONSTS)
     tables = [sa.Table.random(seed * 1000 + k, 1 << n) for k in range(3)]

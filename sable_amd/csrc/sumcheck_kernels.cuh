@@ -102,7 +102,8 @@ __device__ __forceinline__ Ext<D> fold_base(uint32_t lo, uint32_t hi, const Ext<
 }
 template <int D>
 __device__ __forceinline__ Ext<D> fold_ext(const Ext<D> &lo, const Ext<D> &hi, const Ext<D> &r_mont) {
-  return ext_add<D>(lo, ext_mul_mont<D>(r_mont, ext_sub<D>(hi, lo)));
+  // r is the second operand: its tripled wrap coefficients are the same for every entry of the launch
+  return ext_add<D>(lo, ext_mul_mont<D>(ext_sub<D>(hi, lo), r_mont));
 }
 
 // ---- the per-pair work: all groups at all their points.  V is uint32_t (base mode) or Ext<D>.
@@ -243,16 +244,22 @@ __device__ __forceinline__ void block_sums(const Desc &d, Acc96 (*acc)[D], uint3
 // (ROUND-MESSAGE, src/sumcheck.lisp:313-317), send = absorb the rows (src/transcript.lisp:116-128),
 // r = challenge (src/transcript.lisp:174-176).  All threads of the workgroup call; scratch is LDS.
 struct EpilogueLds {
-  uint32_t prod[MAXPTS * MAXACC * 8];
+  alignas(16) uint32_t prod[MAXPTS * MAXACC * 8];
   uint32_t msg[MAXPTS * 8];
   uint32_t chal[8];
   uint32_t r_mont[8];
   uint32_t ring[32];
+  // staged copies (filled by the caller when it passes staged = true)
+  uint32_t state[sizeof(DevB3S) / 4];
+  uint32_t round;
+  alignas(16) uint32_t mtilde[MAXPTS * MAXACC * 8];
+  alignas(16) uint32_t c0[MAXPTS * 8];
 };
 
 template <int D>
 __device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums, uint32_t nacc, uint32_t points,
-                                               const uint32_t *mtilde, const uint32_t *c0, EpilogueLds *e) {
+                                               const uint32_t *mtilde, const uint32_t *c0, EpilogueLds *e,
+                                               bool staged = false) {
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   for (uint32_t u = tid; u < points * nacc; u += nthreads) {
     uint32_t a = u % nacc;
@@ -271,9 +278,9 @@ __device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums,
   }
   __syncthreads();
   if (tid < 64) {  // the first wavefront runs the transcript, every lane the same steps
-    const uint32_t round = ctrl->round;
+    const uint32_t round = staged ? e->round : ctrl->round;
     RunB3S tr;
-    rb3s_load(tr, e->ring, &ctrl->tr);
+    rb3s_load(tr, e->ring, staged ? reinterpret_cast<const DevB3S *>(e->state) : &ctrl->tr);
     dev_absorb_words(tr, e->msg, points * D);
     dev_challenge(tr, D, e->chal);
     rb3s_store(tr, &ctrl->tr);
@@ -352,6 +359,12 @@ __global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) 
   __shared__ uint32_t sums[MAXACC * D];
   __shared__ EpilogueLds epi;
   const uint32_t tid = threadIdx.x, width = args.nacc * D, ps = args.pstride;
+  // everything the serial part needs from global memory is requested first, so that its latency
+  // overlaps the partial sums: the transcript state, the message map and the constant terms
+  if (tid < sizeof(DevB3S) / 4) epi.state[tid] = reinterpret_cast<const uint32_t *>(&args.ctrl->tr)[tid];
+  if (tid == 64) epi.round = args.ctrl->round;
+  for (uint32_t u = tid; u < args.points * width; u += EPI_BLOCK) epi.mtilde[u] = args.mtilde[u];
+  for (uint32_t u = tid; u < args.points * D; u += EPI_BLOCK) epi.c0[u] = args.c0[u];
   // sums[o] = sum over workgroups of partial[o]: thread t takes column t % pstride of the rows
   // t / pstride, t / pstride + rstep, ...; four loads in flight per thread
   for (uint32_t col0 = 0; col0 < ps; col0 += EPI_BLOCK) {
@@ -378,7 +391,7 @@ __global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) 
     }
   }
   __syncthreads();
-  round_epilogue<D>(args.ctrl, sums, args.nacc, args.points, args.mtilde, args.c0, &epi);
+  round_epilogue<D>(args.ctrl, sums, args.nacc, args.points, epi.mtilde, epi.c0, &epi, true);
 }
 
 // The last rounds in one workgroup: [fold], then per round sums -> message -> challenge -> fold.
