@@ -1,6 +1,8 @@
 // forms.cpp -- see forms.hpp.
 #include "forms.hpp"
 
+#include <string.h>
+
 #include <algorithm>
 #include <map>
 #include <memory>
@@ -170,6 +172,198 @@ bool expand_node(const Node &n, Poly *out) {
   return false;
 }
 
+
+// ---- the written shape of a form: a sum of products whose factors are integers, constants, tables
+// or linear forms in the tables.  Returns false when the form has another shape.
+struct Product {
+  uint32_t coeff = 1;
+  std::vector<int> consts;
+  std::vector<Linear> factors;  // a plain table is the linear form 1 * table + 0
+  bool zero = false;
+};
+
+struct Shape {
+  const std::vector<std::string> *tables, *constants;
+  int find(const std::vector<std::string> &names, const std::string &v) const {
+    auto it = std::find(names.begin(), names.end(), v);
+    return it == names.end() ? -1 : (int)(it - names.begin());
+  }
+  // a form that expands to integer multiples of tables plus an integer
+  bool linear(const Node &n, Linear *out) const {
+    Poly p;
+    if (!expand_node(n, &p)) return false;
+    std::map<int, uint32_t> by_table;
+    out->constant = 0;
+    for (auto &t : p) {
+      if (t.first.size() > 1) return false;
+      if (t.first.empty()) {
+        out->constant = t.second;
+        continue;
+      }
+      int ti = find(*tables, t.first[0]);
+      if (ti < 0) return false;
+      if (t.second) by_table[ti] = t.second;
+    }
+    out->terms.assign(by_table.begin(), by_table.end());
+    return true;
+  }
+  bool factor(const Node &n, Product *out) const {
+    if (n.kind == Node::INT) {
+      out->coeff = fmul(out->coeff, (uint32_t)n.value);
+      return true;
+    }
+    if (n.kind == Node::VAR) {
+      int ci = find(*constants, n.name);
+      if (ci >= 0 && find(*tables, n.name) < 0) {
+        out->consts.push_back(ci);
+        return true;
+      }
+    }
+    if (n.kind == Node::OP && n.name == "*") {
+      for (auto &a : n.args)
+        if (!factor(*a, out)) return false;
+      return true;
+    }
+    if (n.kind == Node::OP && n.name == "EXPT" && n.args.size() == 2 && n.args[1]->kind == Node::INT &&
+        n.args[1]->value <= MAXDEG) {
+      for (long long i = 0; i < n.args[1]->value; i++)
+        if (!factor(*n.args[0], out)) return false;
+      return true;
+    }
+    Linear lin;
+    if (!linear(n, &lin)) return false;
+    if (lin.terms.empty()) {  // an integer after all
+      out->coeff = fmul(out->coeff, lin.constant);
+      return true;
+    }
+    out->factors.push_back(lin);
+    return true;
+  }
+  bool sum(const Node &n, bool negate, std::vector<Product> *out) const {
+    if (n.kind == Node::OP && n.name == "+") {
+      for (auto &a : n.args)
+        if (!sum(*a, negate, out)) return false;
+      return true;
+    }
+    if (n.kind == Node::OP && n.name == "-" && !n.args.empty()) {
+      for (size_t i = 0; i < n.args.size(); i++)
+        if (!sum(*n.args[i], negate != (n.args.size() == 1 || i > 0), out)) return false;
+      return true;
+    }
+    Product prod;
+    if (!factor(n, &prod)) return false;
+    if (negate) prod.coeff = fneg(prod.coeff);
+    out->push_back(prod);
+    return true;
+  }
+};
+
+bool is_table(const Linear &l) { return l.terms.size() == 1 && l.terms[0].second == 1 && l.constant == 0; }
+
+void sort_groups(std::vector<Group> *groups) {
+  // constant group first, then by degree, then by factors: a fixed order for the kernels' accumulators
+  std::stable_sort(groups->begin(), groups->end(), [](const Group &a, const Group &b) {
+    if (a.tabs.size() != b.tabs.size()) return a.tabs.size() < b.tabs.size();
+    return a.tabs < b.tabs;
+  });
+}
+
+// the factored groups multiplied out again, as a polynomial in table and constant names
+Poly multiply_out(const Statement &st, const std::vector<Group> &groups, const std::vector<Linear> &linear) {
+  Poly total;
+  for (const Group &g : groups) {
+    Poly prod;
+    add_term(prod, {}, 1);
+    for (int f : g.tabs) {
+      Poly lin;
+      if (f < st.T())
+        add_term(lin, {st.tables[f]}, 1);
+      else {
+        const Linear &l = linear[f - st.T()];
+        for (auto &t : l.terms) add_term(lin, {st.tables[t.first]}, t.second);
+        if (l.constant) add_term(lin, {}, l.constant);
+      }
+      prod = multiply(prod, lin);
+    }
+    Poly coef;
+    for (const Group::Part &part : g.parts) {
+      std::vector<std::string> m;
+      for (int k : part.consts) m.push_back(st.constants[k]);
+      std::sort(m.begin(), m.end());
+      add_term(coef, m, part.coeff);
+    }
+    Poly term = multiply(prod, coef);
+    for (auto &t : term) add_term(total, t.first, t.second);
+  }
+  for (auto it = total.begin(); it != total.end();) it = it->second ? std::next(it) : total.erase(it);
+  return total;
+}
+
+void factor_statement(const Node &root, Statement *st) {
+  st->factored_groups.clear();
+  st->factored_linear.clear();
+  Shape shape{&st->tables, &st->constants};
+  std::vector<Product> products;
+  if (!shape.sum(root, false, &products)) return;
+  std::map<Linear, int> ids;
+  std::map<std::vector<int>, Group> groups;
+  for (const Product &prod : products) {
+    if (prod.coeff == 0) continue;
+    std::vector<int> factors;
+    for (const Linear &l : prod.factors) {
+      if (is_table(l)) {
+        factors.push_back(l.terms[0].first);
+        continue;
+      }
+      auto it = ids.find(l);
+      if (it == ids.end()) {
+        it = ids.emplace(l, st->T() + (int)st->factored_linear.size()).first;
+        st->factored_linear.push_back(l);
+      }
+      factors.push_back(it->second);
+    }
+    std::sort(factors.begin(), factors.end());
+    Group &g = groups[factors];
+    g.tabs = factors;
+    std::vector<int> consts(prod.consts);
+    std::sort(consts.begin(), consts.end());
+    g.parts.push_back(Group::Part{prod.coeff, consts});
+  }
+  for (auto &kv : groups) st->factored_groups.push_back(kv.second);
+  sort_groups(&st->factored_groups);
+  // accept the written shape only if it multiplies out to the canonical expansion
+  Poly expanded;
+  for (const Term &t : st->terms) add_term(expanded, t.vars, t.coeff);
+  if (multiply_out(*st, st->factored_groups, st->factored_linear) != expanded) {
+    st->factored_groups.clear();
+    st->factored_linear.clear();
+  }
+}
+
+// products per pair and round of a shape planned for POINTS wire points: every evaluation of a group
+// costs its degree (degree - 1 for the factors, 1 for the weight)
+long plan_groups(std::vector<Group> *groups, int points, int *nacc) {
+  long cost = 0;
+  *nacc = 0;
+  for (Group &g : *groups) {
+    g.evalx.clear();
+    g.acc_base = *nacc;
+    int d = (int)g.tabs.size();
+    if (d == 0) continue;  // its sum is the sum of the weights: no device work
+    if (points < 0)
+      g.evalx = {0, 1};  // the honest claim
+    else if (d >= points) {  // the wire points 0, 2, 3, ..., points
+      g.evalx.push_back(0);
+      for (int x = 2; x <= points; x++) g.evalx.push_back(x);
+    } else {  // degree d: d + 1 cheap points, extrapolated on the host
+      for (int x = 0; x <= d; x++) g.evalx.push_back(x);
+    }
+    *nacc += (int)g.evalx.size();
+    cost += (long)g.evalx.size() * d;
+  }
+  return cost;
+}
+
 }  // namespace
 
 int expand_form(const std::string &text, std::vector<Term> *out) {
@@ -223,50 +417,53 @@ int compile_statement(const std::string &text, const std::vector<std::string> &t
     g.tabs = tabs;
     g.parts.push_back(Group::Part{term.coeff, consts});
   }
-  st->groups.clear();
-  for (auto &kv : groups) st->groups.push_back(kv.second);
-  // constant group first, then by degree, then by tables: a fixed order for the kernels' accumulators
-  std::stable_sort(st->groups.begin(), st->groups.end(), [](const Group &a, const Group &b) {
-    if (a.tabs.size() != b.tabs.size()) return a.tabs.size() < b.tabs.size();
-    return a.tabs < b.tabs;
-  });
+  st->expanded_groups.clear();
+  for (auto &kv : groups) st->expanded_groups.push_back(kv.second);
+  sort_groups(&st->expanded_groups);
+  Parser parser(text);
+  auto root = parser.parse();
+  factor_statement(*root, st);
+  st->groups = st->expanded_groups;
+  st->linear.clear();
   st->planned_points = -1;
   return OK;
+}
+
+// both shapes are planned; the factored one is taken only when it needs fewer products
+static void choose_shape(Statement *st, int points) {
+  int nacc_e = 0, nacc_f = 0;
+  long cost_e = plan_groups(&st->expanded_groups, points, &nacc_e);
+  bool factored = false;
+  if (!st->factored_groups.empty() && (int)st->factored_linear.size() <= MAXV &&
+      st->T() + (int)st->factored_linear.size() <= MAXT) {
+    bool fits = true;
+    for (const Linear &l : st->factored_linear) fits = fits && (int)l.terms.size() <= MAXVT;
+    long cost_f = plan_groups(&st->factored_groups, points, &nacc_f);
+    factored = fits && cost_f < cost_e;
+  }
+  st->groups = factored ? st->factored_groups : st->expanded_groups;
+  st->linear = factored ? st->factored_linear : std::vector<Linear>();
+  st->nacc = factored ? nacc_f : nacc_e;
 }
 
 void Statement::plan(int points) {
   if (planned_points == points) return;
   planned_points = points;
-  nacc = 0;
-  for (Group &g : groups) {
-    g.evalx.clear();
-    g.acc_base = nacc;
-    int d = (int)g.tabs.size();
-    if (d == 0) continue;  // its sum is the sum of the weights: no device work
-    if (d >= points) {     // the wire points 0, 2, 3, ..., points
-      g.evalx.push_back(0);
-      for (int x = 2; x <= points; x++) g.evalx.push_back(x);
-    } else {  // degree d: d + 1 cheap points, extrapolated on the host
-      for (int x = 0; x <= d; x++) g.evalx.push_back(x);
-    }
-    nacc += (int)g.evalx.size();
-  }
+  choose_shape(this, points);
 }
 
 void Statement::plan_claim() {
   planned_points = -2;
-  nacc = 0;
-  for (Group &g : groups) {
-    g.evalx.clear();
-    g.acc_base = nacc;
-    if (g.tabs.empty()) continue;
-    g.evalx = {0, 1};
-    nacc += 2;
-  }
+  choose_shape(this, -1);
 }
 
 std::string Statement::key() const {
   std::string k = "T" + std::to_string(T()) + ":";
+  for (const Linear &l : linear) {
+    k += "(";
+    for (auto &t : l.terms) k += std::to_string(t.second) + "*" + std::to_string(t.first) + "+";
+    k += std::to_string(l.constant) + ")";
+  }
   for (const Group &g : groups) {
     if (g.tabs.empty()) continue;
     k += "[";
@@ -282,7 +479,16 @@ void evaluate_statement(const Statement &st, int D, const uint32_t *tv, const ui
   hf::E acc = hf::zero(D);
   for (const Group &g : st.groups) {
     hf::E prod = hf::lift(1, D);
-    for (int t : g.tabs) prod = hf::mul(prod, hf::from(tv + (size_t)t * D, D));
+    for (int f : g.tabs) {
+      if (f < st.T()) {
+        prod = hf::mul(prod, hf::from(tv + (size_t)f * D, D));
+        continue;
+      }
+      const Linear &l = st.linear[f - st.T()];
+      hf::E v = hf::lift(l.constant, D);
+      for (auto &t : l.terms) v = hf::add(v, hf::mul(hf::lift(t.second, D), hf::from(tv + (size_t)t.first * D, D)));
+      prod = hf::mul(prod, v);
+    }
     hf::E coef = hf::zero(D);
     for (const Group::Part &part : g.parts) {
       hf::E c = hf::lift(part.coeff, D);
@@ -292,6 +498,42 @@ void evaluate_statement(const Statement &st, int D, const uint32_t *tv, const ui
     acc = hf::add(acc, hf::mul(coef, prod));
   }
   memcpy(out, acc.data(), 4 * D);
+}
+
+bool make_desc(const Statement &st, StmtDesc *out) {
+  StmtDesc d;
+  memset(&d, 0, sizeof(d));
+  d.T = st.T();
+  d.NV = (int)st.linear.size();
+  if (d.T < 1 || d.NV > MAXV || d.T + d.NV > MAXT || st.nacc > MAXACC) return false;
+  for (int v = 0; v < d.NV; v++) {
+    const Linear &l = st.linear[v];
+    if ((int)l.terms.size() > MAXVT) return false;
+    d.vn[v] = (int)l.terms.size();
+    for (size_t k = 0; k < l.terms.size(); k++) {
+      d.vtab[v][k] = l.terms[k].first;
+      d.vcoef[v][k] = l.terms[k].second;
+      d.vcoefm[v][k] = to_mont(l.terms[k].second);
+    }
+    d.vconst[v] = l.constant;
+  }
+  int g = 0, maxx = 0;
+  for (const Group &grp : st.groups) {
+    if (grp.tabs.empty()) continue;
+    if (g >= MAXG || (int)grp.tabs.size() > MAXDEG || (int)grp.evalx.size() > MAXEV || grp.evalx.back() > MAXX)
+      return false;
+    d.deg[g] = (int)grp.tabs.size();
+    for (size_t j = 0; j < grp.tabs.size(); j++) d.tab[g][j] = grp.tabs[j];
+    d.nev[g] = (int)grp.evalx.size();
+    for (size_t k = 0; k < grp.evalx.size(); k++) {
+      d.ev[g][k] = grp.evalx[k];
+      if (grp.evalx[k] > maxx) maxx = grp.evalx[k];
+    }
+    g++;
+  }
+  d.G = g, d.nacc = st.nacc, d.maxx = maxx;
+  *out = d;
+  return true;
 }
 
 void group_coefficients(const Statement &st, int D, const uint32_t *cv, uint32_t *out) {

@@ -8,6 +8,8 @@
 #include <utility>
 #include <vector>
 
+#include "stmtdesc.hpp"
+
 namespace exh {
 
 struct Term {  // coefficient * product of variables (names upper-cased, sorted)
@@ -22,7 +24,9 @@ int expand_form(const std::string &text, std::vector<Term> *out);
 // One group of a compiled statement: a multiset of tables with the constant-side of every term
 // over it, so that  statement = sum_g coefficient_g(constants) * prod_{t in g} table_t.
 struct Group {
-  std::vector<int> tabs;  // table indices, sorted; empty: the constant group
+  // factor indices, sorted; empty: the constant group.  An index below T is a table, T + v is the
+  // statement's linear form v
+  std::vector<int> tabs;
   struct Part {
     uint32_t coeff;
     std::vector<int> consts;  // constant indices (with repetition)
@@ -34,6 +38,15 @@ struct Group {
   int acc_base = 0;  // index of its first accumulator
 };
 
+// A factor that is not a single table: sum of integer multiples of tables plus an integer, as in
+// (+ c0 3) or (- c1 c0).  Kept as a factor instead of being multiplied out, a product of such forms
+// needs one accumulator per evaluation point instead of one per monomial.
+struct Linear {
+  std::vector<std::pair<int, uint32_t>> terms;  // (table, coefficient mod p), by table
+  uint32_t constant = 0;
+  bool operator<(const Linear &o) const { return terms != o.terms ? terms < o.terms : constant < o.constant; }
+};
+
 struct Statement {
   std::string text;
   std::vector<std::string> tables, constants;
@@ -41,8 +54,14 @@ struct Statement {
   int degree = 0;  // in the tables (src/sumcheck.lisp:33-35)
   int T() const { return (int)tables.size(); }
   int C() const { return (int)constants.size(); }
-  std::vector<Group> groups;  // constant group (if any) included
-  int nacc = 0;               // accumulators per round over all groups
+  // the statement as sum_g coefficient_g * prod(factors of g), in two equivalent shapes: one group per
+  // table monomial of the expanded form, and (when the form is a sum of products of linear forms) one
+  // group per written product.  plan() points `groups` at the cheaper one.
+  std::vector<Group> expanded_groups, factored_groups;
+  std::vector<Linear> factored_linear;
+  std::vector<Group> groups;   // the planned shape; constant group (if any) included
+  std::vector<Linear> linear;  // its linear forms
+  int nacc = 0;                // accumulators per round over all groups
   // the device evaluation points are chosen for POINTS = max(header degree, 1) wire points
   void plan(int points);
   // every group at X = 0 and X = 1 only: what the honest claim (HYPERCUBE-SUM) needs
@@ -57,6 +76,8 @@ int compile_statement(const std::string &text, const std::vector<std::string> &t
 // the statement over F_p^D at the given table and constant values (exact, host side)
 void evaluate_statement(const Statement &st, int D, const uint32_t *table_vals, const uint32_t *const_vals,
                         uint32_t *out);
+// the descriptor of the planned statement for the kernels; false when it exceeds their limits
+bool make_desc(const Statement &st, StmtDesc *out);
 // the groups' coefficients at the constants: out[g*D .. g*D+D)
 void group_coefficients(const Statement &st, int D, const uint32_t *const_vals, uint32_t *out);
 

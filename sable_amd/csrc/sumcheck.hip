@@ -118,28 +118,6 @@ const KernelSet *find_kernels(const std::string &key, int D) {
   return it == registry().end() ? nullptr : &it->second;
 }
 
-StmtDesc make_desc(const Statement &st) {
-  StmtDesc d;
-  memset(&d, 0, sizeof(d));
-  d.T = st.T();
-  int g = 0, maxx = 0;
-  for (const Group &grp : st.groups) {
-    if (grp.tabs.empty()) continue;
-    d.deg[g] = (int)grp.tabs.size();
-    for (size_t j = 0; j < grp.tabs.size(); j++) d.tab[g][j] = grp.tabs[j];
-    d.nev[g] = (int)grp.evalx.size();
-    for (size_t k = 0; k < grp.evalx.size(); k++) {
-      d.ev[g][k] = grp.evalx[k];
-      if (grp.evalx[k] > maxx) maxx = grp.evalx[k];
-    }
-    g++;
-  }
-  d.G = g;
-  d.nacc = st.nacc;
-  d.maxx = maxx;
-  return d;
-}
-
 // ------------------------------------------------------------------ the session
 static inline uint32_t next_pow2(uint64_t v) {
   uint32_t p = 1;
@@ -168,20 +146,11 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
     st.plan(points);
   eq0.clear();
   if (eq && n > 0) eq0.assign(eq, eq + D);
-  int T = st.T(), real_groups = 0;
-  for (const Group &g : st.groups) {
-    if (g.tabs.empty()) continue;
-    real_groups++;
-    if ((int)g.tabs.size() > MAXDEG || (int)g.evalx.size() > MAXEV || g.evalx.back() > MAXX) {
-      set_error("invalid-parameter: statement degree beyond the kernels' limit");
-      return E_PARAM;
-    }
-  }
-  if (T < 1 || T > MAXT || real_groups > MAXG || st.nacc > MAXACC || points > 16) {
+  int T = st.T();
+  if (T > MAXT || points > 16 || !make_desc(st, &desc)) {
     set_error("invalid-parameter: statement beyond the kernels' limits");
     return E_PARAM;
   }
-  desc = make_desc(st);
   kernels = find_kernels(st.key(), D);
   generated = kernels != nullptr;
   has_eq = eq != nullptr;

@@ -18,7 +18,6 @@ struct KernelSet {  // the launchers generated for one statement and one degree 
 };
 void register_kernels(const std::string &key, int D, KernelSet set);
 const KernelSet *find_kernels(const std::string &key, int D);
-StmtDesc make_desc(const Statement &st);
 
 struct SumcheckSession {
   int D = 4, n = 0, K = 1, points = 1;

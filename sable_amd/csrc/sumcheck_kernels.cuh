@@ -124,6 +124,26 @@ __device__ __forceinline__ void v_weigh(Acc96 *acc, const Ext<D> &w, uint32_t v)
 template <int D>
 __device__ __forceinline__ void v_weigh(Acc96 *acc, const Ext<D> &w, const Ext<D> &v) { ext_mul_acc<D>(acc, w, v); }
 
+// integer multiples and integer offsets, for the linear forms
+template <int D>
+__device__ __forceinline__ uint32_t v_scale(uint32_t a, uint32_t c, uint32_t c_mont) {
+  return c == 1 ? a : c == P - 1 ? fneg(a) : mont_mul(a, c_mont);
+}
+template <int D>
+__device__ __forceinline__ Ext<D> v_scale(const Ext<D> &a, uint32_t c, uint32_t c_mont) {
+  Ext<D> o;
+#pragma unroll
+  for (int k = 0; k < D; k++) o.c[k] = v_scale<D>(a.c[k], c, c_mont);
+  return o;
+}
+template <int D>
+__device__ __forceinline__ uint32_t v_offset(uint32_t a, uint32_t k) { return fadd(a, k); }
+template <int D>
+__device__ __forceinline__ Ext<D> v_offset(Ext<D> a, uint32_t k) {
+  a.c[0] = fadd(a.c[0], k);
+  return a;
+}
+
 template <int D, class V, class Desc>
 __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, const V *hi, const Ext<D> &w,
                                                 Acc96 (*acc)[D]) {
@@ -134,17 +154,33 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
       cur[t] = lo[t];
       slope[t] = v_sub<D>(hi[t], lo[t]);
     }
+  // the linear forms are lines too: value at 0 from the tables' values at 0 plus the offset, slope
+  // from the tables' slopes
+#pragma unroll
+  for (int v = 0; v < MAXV; v++)
+    if (v < d.NV) {
+      V c0 = v_scale<D>(cur[d.vtab[v][0]], d.vcoef[v][0], d.vcoefm[v][0]);
+      V s0 = v_scale<D>(slope[d.vtab[v][0]], d.vcoef[v][0], d.vcoefm[v][0]);
+#pragma unroll
+      for (int k = 1; k < MAXVT; k++)
+        if (k < d.vn[v]) {
+          c0 = v_add<D>(c0, v_scale<D>(cur[d.vtab[v][k]], d.vcoef[v][k], d.vcoefm[v][k]));
+          s0 = v_add<D>(s0, v_scale<D>(slope[d.vtab[v][k]], d.vcoef[v][k], d.vcoefm[v][k]));
+        }
+      cur[d.T + v] = v_offset<D>(c0, d.vconst[v]);
+      slope[d.T + v] = s0;
+    }
 #pragma unroll
   for (int x = 0; x <= MAXX; x++) {
     if (x <= d.maxx) {
-      if (x == 1) {
+      if (x >= 1) {
 #pragma unroll
-        for (int t = 0; t < MAXT; t++)
-          if (t < d.T) cur[t] = hi[t];
-      } else if (x >= 2) {
-#pragma unroll
-        for (int t = 0; t < MAXT; t++)
-          if (t < d.T) cur[t] = v_add<D>(cur[t], slope[t]);
+        for (int t = 0; t < MAXT; t++) {
+          if (x == 1 && t < d.T)
+            cur[t] = hi[t];
+          else if (t < d.T + d.NV)
+            cur[t] = v_add<D>(cur[t], slope[t]);
+        }
       }
       int a = 0;
 #pragma unroll

@@ -120,6 +120,12 @@ def test_config3_product_constraint_over_fp8(n):
     ("(- (expt t0 3) (* t0 t1))", ["t0", "t1"], [], 8, True, True),
     ("(* t0 t1 t2 t3)", ["t0", "t1", "t2", "t3"], [], 4, False, True),
     ("(+ (* alpha t0 t1) (* 3 t1) -2)", ["t0", "t1"], ["alpha"], 4, False, False),
+    # products of linear forms: kept as factors on the device, identical field elements
+    ("(* (+ (* 2 t0) t1 5) (- t0 7) t2)", ["t0", "t1", "t2"], [], 4, True, True),
+    ("(* (+ (* 2 t0) t1 5) (- t0 7) t2)", ["t0", "t1", "t2"], [], 8, False, True),
+    ("(+ (* alpha (+ t0 1) (- t1 t0) t2) (* 3 t0) 9)", ["t0", "t1", "t2"], ["alpha"], 4, False, True),
+    ("(- (* (expt (- t0 1) 2) (+ t1 t0)) (* beta (- t1 4) t0))", ["t0", "t1"], ["beta"], 4, True, False),
+    ("(* (- t0) (+ t1 -3) (+ t0 t1 t2 t3 1) t3)", ["t0", "t1", "t2", "t3"], [], 8, True, True),
 ])
 def test_any_statement_on_the_interpreter_or_generated_kernels(form, names, cnames, d, base, with_eq):
     """tests.lisp:311-395: statements that are not plain products, constants, base or extension tables."""

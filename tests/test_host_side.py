@@ -156,3 +156,15 @@ def test_statement_compile_matches_expand():
     tv = rng.integers(0, sa.P, (3, d), dtype=np.uint32)
     cv = rng.integers(0, sa.P, (1, d), dtype=np.uint32)
     assert sa.check_final(ost.evaluate(tv, cv, d), st, tv, constants=cv)
+    # a product of linear forms keeps its written shape for the kernels (the generated kernel of the F_p^8
+    # configuration is registered under that shape) and evaluates to the same field element
+    form = "(* (+ c0 3) (- c1 c0) c2 c3)"
+    names = ["c0", "c1", "c2", "c3"]
+    st, ost = sa.Statement(form, names), orc.Statement(form, names)
+    assert st.has_generated_kernel(8) and not st.has_generated_kernel(4)
+    for form, names, cnames in [(form, names, []),
+                                ("(- (* (expt (- t0 1) 2) (+ t1 t0)) (* beta (- t1 4) t0))", ["t0", "t1"], ["beta"])]:
+        st, ost = sa.Statement(form, names, cnames), orc.Statement(form, names, cnames)
+        tv = rng.integers(0, sa.P, (len(names), 8), dtype=np.uint32)
+        cv = rng.integers(0, sa.P, (max(len(cnames), 1), 8), dtype=np.uint32)
+        assert sa.check_final(ost.evaluate(tv, cv, 8), st, tv, constants=cv if cnames else None)
