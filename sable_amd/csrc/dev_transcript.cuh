@@ -70,7 +70,9 @@ __device__ __forceinline__ void b3_quad_cv(uint32_t w0, uint32_t w1, uint32_t ou
 }
 
 // The running state: chaining value and counters in registers, the pending block as a 128-byte ring in
-// LDS (`ring`, 32 words) whose two halves are used alternately.
+// LDS (`ring`, the first 32 of RING_WORDS words) whose two halves are used alternately; the other 16
+// words stage a squeeze's output.  Input is appended by all lanes at once, lane k storing byte k.
+constexpr int RING_WORDS = 48;
 struct RunB3S {
   uint32_t cv[8];
   uint32_t *ring;
@@ -96,77 +98,70 @@ __device__ inline void rb3s_store(const RunB3S &s, DevB3S *g) {
   g->counter_lo = (uint32_t)s.counter, g->counter_hi = (uint32_t)(s.counter >> 32);
 }
 
-// the pending block is full and more input arrives: compress it, move to the other half
-__device__ inline void rb3s_flush(RunB3S &s) {
-  uint32_t w0, w1, w2, w3;
-  b3_compress_quad(s.cv, s.ring + 16 * s.half, s.counter, 64, 0, w0, w1, w2, w3);
-  b3_quad_cv(w0, w1, s.cv);
-  s.counter++;
-  s.half ^= 1;
-#pragma unroll
-  for (int i = 0; i < 16; i++) s.ring[16 * s.half + i] = 0;
-  s.used = 0;
-}
-
-// append the low NBYTES (1..4) bytes of W
-__device__ inline void rb3s_append(RunB3S &s, uint32_t w, uint32_t nbytes) {
-  uint8_t *bytes = reinterpret_cast<uint8_t *>(s.ring) + 64 * s.half;
-  if (s.used + nbytes <= 64) {  // the common case: one store, aligned or not
-    if (nbytes == 4)
-      __builtin_memcpy(bytes + s.used, &w, 4);
-    else
-      for (uint32_t b = 0; b < nbytes; b++) bytes[s.used + b] = (uint8_t)(w >> (8 * b));
-    s.used += nbytes;
-    return;
+// Append LEN <= 64 bytes, byte k of them held by lane k.  Bytes that do not fit the pending block go
+// to the ring's other half (cleared first); the pending block is then full with more input behind it,
+// so it is compressed and the halves change roles.  (A wavefront's LDS operations complete in order.)
+__device__ inline void rb3s_append_bytes(RunB3S &s, uint32_t byte, uint32_t len) {
+  const uint32_t lane = threadIdx.x & 63;
+  uint8_t *bytes = reinterpret_cast<uint8_t *>(s.ring);
+  if (lane < 16) s.ring[16 * (s.half ^ 1) + lane] = 0;
+  __builtin_amdgcn_wave_barrier();
+  if (lane < len) {
+    const uint32_t o = s.used + lane;
+    bytes[o < 64 ? 64 * s.half + o : 64 * (s.half ^ 1) + (o - 64)] = (uint8_t)byte;
   }
-  for (uint32_t b = 0; b < nbytes; b++) {  // the word straddles two blocks
-    if (s.used == 64) {
-      rb3s_flush(s);
-      bytes = reinterpret_cast<uint8_t *>(s.ring) + 64 * s.half;
-    }
-    bytes[s.used++] = (uint8_t)(w >> (8 * b));
+  __builtin_amdgcn_wave_barrier();
+  if (s.used + len > 64) {
+    uint32_t w0, w1, w2, w3;
+    b3_compress_quad(s.cv, s.ring + 16 * s.half, s.counter, 64, 0, w0, w1, w2, w3);
+    b3_quad_cv(w0, w1, s.cv);
+    s.counter++;
+    s.half ^= 1;
+    s.used = s.used + len - 64;
+  } else {
+    s.used += len;
   }
 }
 
-// 48 bytes of output for everything absorbed so far (state unchanged)
-__device__ inline void rb3s_digest48(const RunB3S &s, uint32_t out[12]) {
-  uint32_t w0, w1, w2, w3;
-  b3_compress_quad(s.cv, s.ring + 16 * s.half, 0, s.used, B3_CHUNK_END | B3_ROOT, w0, w1, w2, w3);
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    out[i] = (uint32_t)__builtin_amdgcn_readlane((int)w0, i);
-    out[4 + i] = (uint32_t)__builtin_amdgcn_readlane((int)w1, i);
-    out[8 + i] = (uint32_t)__builtin_amdgcn_readlane((int)w2, i);
-  }
-}
-
-// absorb(data) for NWORDS little-endian words: the length as u64 LE, then the bytes
+// absorb(data) for NWORDS little-endian words in LDS: the length as u64 LE, then the bytes
 // (src/transcript.lisp:95-100)
 __device__ inline void dev_absorb_words(RunB3S &s, const uint32_t *words, uint32_t nwords) {
-  rb3s_append(s, 4 * nwords, 4);
-  rb3s_append(s, 0, 4);
-  for (uint32_t i = 0; i < nwords; i++) rb3s_append(s, words[i], 4);
+  const uint32_t lane = threadIdx.x & 63, total = 8 + 4 * nwords;
+  for (uint32_t base = 0; base < total; base += 64) {
+    const uint32_t g = base + lane;  // this lane's byte of the stream
+    uint32_t word = g < 4 ? 4 * nwords : (g < 8 || g >= total) ? 0 : words[(g - 8) >> 2];
+    rb3s_append_bytes(s, (word >> (8 * (g & 3))) & 0xff, total - base < 64 ? total - base : 64);
+  }
 }
 
 // K <= 8 base-field challenges (CHALLENGE-BASE, src/transcript.lisp:159-172): squeeze 4 (missing + 4)
 // bytes, keep the 31-bit words below p, repeat until K are kept; each squeeze then absorbs "squeeze" and
-// the first min(32, n) bytes of its output (src/transcript.lisp:152-157).
+// the first min(32, n) bytes of its output (src/transcript.lisp:152-157).  OUT is in LDS.
 __device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out) {
+  const uint32_t lane = threadIdx.x & 63;
+  uint32_t *stage = s.ring + 32;
   int have = 0;
   while (have < k) {
-    uint32_t n = 4u * (uint32_t)(k - have + 4);  // at most 48 bytes: one output block
-    uint32_t o[12];
-    rb3s_digest48(s, o);
-    rb3s_append(s, 0x65757173u, 4);  // "sque"
-    rb3s_append(s, 0x00657a65u, 3);  // "eze"
-#pragma unroll
-    for (uint32_t i = 0; i < 8; i++)
-      if (4 * i < n) rb3s_append(s, o[i], 4);
-#pragma unroll
-    for (uint32_t i = 0; i < 12; i++) {
-      uint32_t w = o[i] & 0x7fffffffu;
-      if (4 * i < n && have < k && w < P) out[have++] = w;
-    }
+    const uint32_t n = 4u * (uint32_t)(k - have + 4);  // at most 48 bytes: one output block
+    uint32_t w0, w1, w2, w3;
+    b3_compress_quad(s.cv, s.ring + 16 * s.half, 0, s.used, B3_CHUNK_END | B3_ROOT, w0, w1, w2, w3);
+    if (lane < 4) stage[lane] = w0, stage[4 + lane] = w1, stage[8 + lane] = w2;
+    __builtin_amdgcn_wave_barrier();
+    // "squeeze", then the first min(32, n) bytes of the output
+    const uint32_t fed = n < 32 ? n : 32;
+    uint32_t byte = 0;
+    if (lane < 7)
+      byte = (lane < 4 ? 0x65757173u >> (8 * lane) : 0x00657a65u >> (8 * (lane - 4))) & 0xff;
+    else if (lane < 7 + fed)
+      byte = (stage[(lane - 7) >> 2] >> (8 * ((lane - 7) & 3))) & 0xff;
+    const uint32_t cand = lane < n / 4 ? stage[lane] & 0x7fffffffu : P;
+    rb3s_append_bytes(s, byte, 7 + fed);
+    // the candidates below p, in order, as far as needed
+    const uint64_t ok = __ballot(cand < P);
+    const int rank = __popcll(ok & (((uint64_t)1 << lane) - 1));
+    if (cand < P && have + rank < k) out[have + rank] = cand;
+    have += __popcll(ok);
+    __builtin_amdgcn_wave_barrier();
   }
 }
 

@@ -104,7 +104,7 @@ static void launch_interp(const RoundArgs<D> &a, const StmtDesc &d, bool in_base
 
 template <int D>
 static void launch_tail_interp(const TailArgs<D> &a, const StmtDesc &d, hipStream_t s) {
-  hipLaunchKernelGGL((tail_kernel_interp<D>), dim3(1), dim3(BLOCK), 0, s, a, d);
+  hipLaunchKernelGGL((tail_kernel_interp<D>), dim3(1), dim3(BLOCK), a.lds_bytes, s, a, d);
 }
 
 // ------------------------------------------------------------------ registry of generated kernels
@@ -527,7 +527,13 @@ int SumcheckSession::finish(uint32_t *finals, uint32_t *const *folded) {
 }
 
 // ------------------------------------------------------------------ the device-driven loop
-constexpr uint64_t TAIL_PAIRS = 256;  // rounds with at most this many pairs run in the one-workgroup tail
+// rounds with at most this many pairs run in the one-workgroup tail: one pair per thread, and the
+// tables (two entries per pair) must fit the tail's LDS
+static uint64_t tail_pairs(int T, int D) {
+  uint64_t p = BLOCK;
+  while (p > 1 && (uint64_t)T * 2 * p * D * 4 > TAIL_LDS_BYTES) p /= 2;
+  return p;
+}
 
 int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges) {
   Context &c = ctx();
@@ -587,7 +593,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   int status = OK, j = 0;
   for (; j < n && status == OK; j++) {
     uint64_t n_pairs = (size / (j == 0 ? 1 : 2)) / 2;  // pairs summed in round j (after the pending fold)
-    if (n_pairs <= TAIL_PAIRS && n - j <= MAXTAIL && (!cur_base || j == 0)) break;
+    if (n_pairs <= tail_pairs(T, D) && n - j <= MAXTAIL) break;
     round = j;
     if (j == 0) {
       status = D == 4 ? launch_round<4>(*this, false, true, out_buf, n_pairs, j)
@@ -635,35 +641,25 @@ int SumcheckSession::launch_tail(int j) {
   Context &c = ctx();
   const int T = st.T();
   const bool first_fold = j > 0;
-  if (cur_base) {  // the tail reads extension tables: lift base inputs (a tiny sumcheck)
-    if (first_fold) {
-      set_error("device-error: base tables with a pending fold at the tail");
-      return E_DEVICE;
-    }
-    int status = c.fold_b.reserve((size_t)T * size * D * 4 * 2);
-    if (status) return status;
-    uint32_t *dst = (uint32_t *)c.fold_b.ptr + (uint64_t)T * size * D;  // above the generations' area
-    for (int t = 0; t < T; t++) {
-      uint32_t grid = (uint32_t)((size + BLOCK - 1) / BLOCK);
-      if (D == 4)
-        hipLaunchKernelGGL(lift_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], dst, size);
-      else
-        hipLaunchKernelGGL(lift_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, cur[t], dst, size);
-      cur[t] = dst;
-      dst += size * D;
-    }
-    cur_base = false;
-  }
+  // it folds (first_fold ? 1 : 0) + (n - j) times; the result goes where alternating arenas would put it
+  int folds = (first_fold ? 1 : 0) + (n - j);
+  uint64_t final_size = size >> folds;
+  int last_gen = generation + folds - 1;
+  Arena &dst = (last_gen % 2 == 0) ? c.fold_a : c.fold_b;
+  int status = dst.reserve((size_t)T * final_size * D * 4);
+  if (status) return status;
   auto fill = [&](auto &a) {
     memset(&a, 0, sizeof(a));
     for (int t = 0; t < T; t++) a.in[t] = cur[t];
-    a.buf[0] = (uint32_t *)c.fold_a.ptr;
-    a.buf[1] = (uint32_t *)c.fold_b.ptr;
+    a.out = (uint32_t *)dst.ptr;
     a.weights = d_weights;
-    a.entries = size;
+    a.entries = (uint32_t)size;
+    a.in_base = cur_base ? 1 : 0;
     a.first_fold = first_fold ? 1 : 0;
     a.rounds = (uint32_t)(n - j);
-    a.generation = (uint32_t)generation;
+    a.first_round = (uint32_t)j;
+    a.capacity = (uint32_t)(2 * tail_pairs(T, D));
+    a.lds_bytes = (uint32_t)(T * a.capacity * D * 4);
     a.points = (uint32_t)points;
     a.ctrl = d_ctrl;
     a.mtilde = d_mtilde;
@@ -692,11 +688,7 @@ int SumcheckSession::launch_tail(int j) {
   }
   c.prof_end();
   EXH_HIP(hipGetLastError());
-  // where the tail leaves the tables: it folds (first_fold ? 1 : 0) + (n - j) times, alternating arenas
-  int folds = (first_fold ? 1 : 0) + (n - j);
-  uint64_t final_size = size >> folds;
-  int last_gen = generation + folds - 1;
-  Arena &dst = (last_gen % 2 == 0) ? c.fold_a : c.fold_b;
+  cur_base = false;
   for (int t = 0; t < T; t++) cur[t] = (uint32_t *)dst.ptr + (uint64_t)t * final_size * D;
   size = final_size;
   generation += folds;

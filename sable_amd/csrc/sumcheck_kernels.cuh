@@ -56,18 +56,23 @@ struct RoundArgs {
   uint32_t pstride;          // words per workgroup partial (a power of two >= nacc * D)
 };
 
-// the rounds at the end of a sumcheck, all in one workgroup (tables of at most a few thousand entries)
+// The rounds at the end of a sumcheck, all in one workgroup with the tables resident in LDS: no global
+// memory round trip separates a round's sums, its transcript step and its fold.
+constexpr uint32_t TAIL_LDS_BYTES = 32768;  // LDS given to the tables
 template <int D>
 struct TailArgs {
-  const uint32_t *in[MAXT];  // extension tables of `entries` entries each
-  uint32_t *buf[2];          // the two generations' arenas; table t of a generation of E entries is at t * E * D
+  const uint32_t *in[MAXT];  // tables of `entries` entries each; base (stride 1) when in_base
+  uint32_t *out;             // where the folded tables go: table t at t * final_entries * D
   const uint32_t *weights;   // base of the weight tables
   uint64_t low_off[MAXTAIL], high_off[MAXTAIL];  // in EXTs, per tail round
   uint32_t low_bits[MAXTAIL];
-  uint64_t entries;
-  uint32_t first_fold;       // fold by ctrl's challenge before the first tail round
-  uint32_t rounds;           // rounds summed here; one more fold follows the last
-  uint32_t generation;       // parity of the arena the next fold writes
+  uint32_t entries;
+  uint32_t in_base;
+  uint32_t first_fold;       // fold by ctrl's challenge while loading
+  uint32_t rounds;           // rounds summed here; a fold follows each
+  uint32_t first_round;      // index of the first of them
+  uint32_t capacity;         // entries per table in LDS
+  uint32_t lds_bytes;        // T * capacity * D * 4
   uint32_t points;
   Ctrl *ctrl;
   const uint32_t *mtilde;
@@ -284,7 +289,7 @@ struct EpilogueLds {
   uint32_t msg[MAXPTS * 8];
   uint32_t chal[8];
   uint32_t r_mont[8];
-  uint32_t ring[32];
+  uint32_t ring[RING_WORDS];
   // staged copies (filled by the caller when it passes staged = true)
   uint32_t state[sizeof(DevB3S) / 4];
   uint32_t round;
@@ -293,9 +298,8 @@ struct EpilogueLds {
 };
 
 template <int D>
-__device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums, uint32_t nacc, uint32_t points,
-                                               const uint32_t *mtilde, const uint32_t *c0, EpilogueLds *e,
-                                               bool staged = false) {
+__device__ __forceinline__ void round_message(const uint32_t *sums, uint32_t nacc, uint32_t points,
+                                              const uint32_t *mtilde, const uint32_t *c0, EpilogueLds *e) {
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   for (uint32_t u = tid; u < points * nacc; u += nthreads) {
     uint32_t a = u % nacc;
@@ -313,18 +317,34 @@ __device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums,
     e->msg[o] = v;
   }
   __syncthreads();
-  if (tid < 64) {  // the first wavefront runs the transcript, every lane the same steps
+}
+
+// the first wavefront's part: send the message, draw the challenge, log both (every lane the same steps)
+template <int D>
+__device__ __forceinline__ void transcript_step(RunB3S &tr, Ctrl *ctrl, uint32_t round, uint32_t points,
+                                                EpilogueLds *e) {
+  const uint32_t tid = threadIdx.x;
+  dev_absorb_words(tr, e->msg, points * D);
+  dev_challenge(tr, D, e->chal);
+  for (uint32_t o = tid; o < points * D; o += 64) ctrl->msg[round][o] = e->msg[o];
+  if (tid < (uint32_t)D) {
+    ctrl->chal[round][tid] = e->chal[tid];
+    ctrl->r_mont[tid] = e->r_mont[tid] = to_mont(e->chal[tid]);
+  }
+}
+
+template <int D>
+__device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums, uint32_t nacc, uint32_t points,
+                                               const uint32_t *mtilde, const uint32_t *c0, EpilogueLds *e,
+                                               bool staged = false) {
+  const uint32_t tid = threadIdx.x;
+  round_message<D>(sums, nacc, points, mtilde, c0, e);
+  if (tid < 64) {
     const uint32_t round = staged ? e->round : ctrl->round;
     RunB3S tr;
     rb3s_load(tr, e->ring, staged ? reinterpret_cast<const DevB3S *>(e->state) : &ctrl->tr);
-    dev_absorb_words(tr, e->msg, points * D);
-    dev_challenge(tr, D, e->chal);
+    transcript_step<D>(tr, ctrl, round, points, e);
     rb3s_store(tr, &ctrl->tr);
-    for (uint32_t o = tid; o < points * D; o += 64) ctrl->msg[round][o] = e->msg[o];
-    if (tid < (uint32_t)D) {
-      ctrl->chal[round][tid] = e->chal[tid];
-      ctrl->r_mont[tid] = e->r_mont[tid] = to_mont(e->chal[tid]);
-    }
     if (tid == 0) ctrl->round = round + 1;
   }
 }
@@ -430,60 +450,112 @@ __global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) 
   round_epilogue<D>(args.ctrl, sums, args.nacc, args.points, epi.mtilde, epi.c0, &epi, true);
 }
 
-// The last rounds in one workgroup: [fold], then per round sums -> message -> challenge -> fold.
+// The last rounds in one workgroup: load (folding or lifting on the way in) into LDS, then per round
+// sums -> message -> challenge -> fold without leaving the compute unit.  Thread i owns pair i.
 template <int D, class Desc>
 __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args) {
-  const uint32_t tid = threadIdx.x;
+  extern __shared__ __align__(16) uint32_t tail_tables[];  // [T][capacity][D]
   __shared__ uint32_t lds[BLOCK / 64][MAXACC * D];
   __shared__ uint32_t sums[MAXACC * D];
   __shared__ EpilogueLds epi;
-  const uint32_t *cur[MAXT];
+  __shared__ uint32_t c0s[MAXTAIL * MAXPTS * D];
+  const uint32_t tid = threadIdx.x, cap = args.capacity;
+  RunB3S tr;
+  if (tid < 64) rb3s_load(tr, epi.ring, &args.ctrl->tr);
+  uint32_t entries = args.first_fold ? args.entries / 2 : args.entries;
+  {
+    Ext<D> r = ext_zero<D>();
+    if (args.first_fold) {
 #pragma unroll
-  for (int t = 0; t < MAXT; t++) cur[t] = t < d.T ? args.in[t] : nullptr;
-  uint64_t entries = args.entries;
-  uint32_t gen = args.generation;
-  // one fold of every table by ctrl's challenge, into the next generation
-  auto fold_all = [&](const uint32_t *r_mont) {
-    Ext<D> r;
-#pragma unroll
-    for (int c = 0; c < D; c++) r.c[c] = r_mont[c];
-    const uint64_t out_entries = entries / 2;
-    uint32_t *dst = args.buf[gen & 1];
+      for (int c = 0; c < D; c++) r.c[c] = args.ctrl->r_mont[c];
+    }
 #pragma unroll
     for (int t = 0; t < MAXT; t++) {
       if (t < d.T) {
-        uint32_t *o = dst + (uint64_t)t * out_entries * D;
-        for (uint64_t x = tid; x < out_entries; x += BLOCK)
-          store_ext<D>(o + x * D, fold_ext<D>(load_ext<D>(cur[t] + 2 * x * D), load_ext<D>(cur[t] + (2 * x + 1) * D), r));
-        cur[t] = o;
+        const uint32_t *in = args.in[t];
+        for (uint32_t x = tid; x < entries; x += BLOCK) {
+          Ext<D> v;
+          if (args.in_base) {
+            if (args.first_fold) {
+              uint2 e = *reinterpret_cast<const uint2 *>(in + 2 * x);
+              v = fold_base<D>(e.x, e.y, r);
+            } else {
+              v = ext_zero<D>();
+              v.c[0] = in[x];
+            }
+          } else if (args.first_fold) {
+            v = fold_ext<D>(load_ext<D>(in + (size_t)2 * x * D), load_ext<D>(in + (size_t)(2 * x + 1) * D), r);
+          } else {
+            v = load_ext<D>(in + (size_t)x * D);
+          }
+          store_ext<D>(tail_tables + ((size_t)t * cap + x) * D, v);
+        }
       }
     }
-    entries = out_entries;
-    gen++;
-    __threadfence();  // the folded entries are read back by other lanes of this workgroup
-    __syncthreads();
-    __threadfence();
+    for (uint32_t u = tid; u < args.points * (uint32_t)d.nacc * D; u += BLOCK) epi.mtilde[u] = args.mtilde[u];
+    for (uint32_t u = tid; u < args.rounds * args.points * D; u += BLOCK) c0s[u] = args.c0[u];
+  }
+  // the weight of this thread's pair, fetched one round ahead
+  Ext<D> wl = ext_zero<D>(), wh = ext_zero<D>();
+  auto fetch_weight = [&](uint32_t jj, uint32_t pairs) {
+    if (tid < pairs) {
+      wl = load_ext<D>(args.weights + (args.low_off[jj] + (tid & ((1u << args.low_bits[jj]) - 1))) * D);
+      wh = load_ext<D>(args.weights + (args.high_off[jj] + (tid >> args.low_bits[jj])) * D);
+    }
   };
-  if (args.first_fold) fold_all(args.ctrl->r_mont);
+  fetch_weight(0, entries / 2);
+  __syncthreads();
   for (uint32_t jj = 0; jj < args.rounds; jj++) {
+    const uint32_t pairs = entries / 2;
     Acc96 acc[MAXACC][D];
 #pragma unroll
     for (int a = 0; a < MAXACC; a++)
 #pragma unroll
       for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
-    const uint64_t n_pairs = entries / 2, low_mask = ((uint64_t)1 << args.low_bits[jj]) - 1;
-    const uint32_t *low = args.weights + args.low_off[jj] * D, *high = args.weights + args.high_off[jj] * D;
-    for (uint64_t i = tid; i < n_pairs; i += BLOCK) {
-      Ext<D> lo[MAXT], hi[MAXT], r0 = ext_zero<D>();
-      load_pair<D, false, false, Ext<D>>(d, cur, nullptr, i, r0, lo, hi);
-      Ext<D> w = ext_mul_mont<D>(load_ext<D>(low + (i & low_mask) * D), load_ext<D>(high + (i >> args.low_bits[jj]) * D));
-      accumulate_pair<D, Ext<D>>(d, lo, hi, w, acc);
+    if (tid < pairs) {
+      Ext<D> lo[MAXT], hi[MAXT];
+#pragma unroll
+      for (int t = 0; t < MAXT; t++)
+        if (t < d.T) {
+          const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * tid) * D;
+          lo[t] = load_ext<D>(p);
+          hi[t] = load_ext<D>(p + D);
+        }
+      accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
     }
+    if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
     block_sums<D>(d, acc, lds, sums);
-    round_epilogue<D>(args.ctrl, sums, (uint32_t)d.nacc, args.points, args.mtilde,
-                      args.c0 + (size_t)jj * args.points * D, &epi);
+    round_message<D>(sums, (uint32_t)d.nacc, args.points, epi.mtilde, c0s + (size_t)jj * args.points * D, &epi);
+    if (tid < 64) transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi);
     __syncthreads();
-    fold_all(epi.r_mont);
+    Ext<D> r, folded[MAXT];
+#pragma unroll
+    for (int c = 0; c < D; c++) r.c[c] = epi.r_mont[c];
+    if (tid < pairs) {
+#pragma unroll
+      for (int t = 0; t < MAXT; t++)
+        if (t < d.T) {
+          const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * tid) * D;
+          folded[t] = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
+        }
+    }
+    __syncthreads();
+    if (tid < pairs) {
+#pragma unroll
+      for (int t = 0; t < MAXT; t++)
+        if (t < d.T) store_ext<D>(tail_tables + ((size_t)t * cap + tid) * D, folded[t]);
+    }
+    __syncthreads();
+    entries = pairs;
+  }
+#pragma unroll
+  for (int t = 0; t < MAXT; t++)
+    if (t < d.T)
+      for (uint32_t x = tid; x < entries; x += BLOCK)
+        store_ext<D>(args.out + ((size_t)t * entries + x) * D, load_ext<D>(tail_tables + ((size_t)t * cap + x) * D));
+  if (tid < 64) {
+    rb3s_store(tr, &args.ctrl->tr);
+    if (tid == 0) args.ctrl->round = args.first_round + args.rounds;
   }
 }
 
