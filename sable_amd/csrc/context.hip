@@ -101,6 +101,7 @@ void ctx_shutdown() {
   c.fold_a.release();
   c.fold_b.release();
   c.misc.release();
+  c.tree.release();
   if (c.host_pinned) (void)hipHostFree(c.host_pinned);
   c.host_pinned = nullptr;
   (void)hipStreamDestroy(c.stream);

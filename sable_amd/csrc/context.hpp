@@ -60,6 +60,7 @@ struct Context {
   uint64_t next_handle = 1;
   Arena fold_a, fold_b;  // the two generations of folded tables
   Arena misc;            // weights, partial sums, small results
+  Arena tree;            // the layers of a fraction tree above its leaves, for the length of one proof
   uint32_t *host_pinned = nullptr;  // small pinned buffer for per-round results
   size_t host_pinned_words = 0;
   int require();  // OK, or E_DEVICE with the reason when the library is not initialised

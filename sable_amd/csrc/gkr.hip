@@ -180,14 +180,14 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
   // FRACTION-TREES: every in-block layer, bottom up, kept on the device
   std::vector<std::vector<const uint32_t *>> layers(n + 1, std::vector<const uint32_t *>(2 * L));
   for (int i = 0; i < 2 * L; i++) layers[n][i] = leaves[i];
+  // one allocation holds every layer above the leaves: 2 L K (2^n - 1) entries
+  if ((status = c.tree.reserve(((((uint64_t)K << n) - K) * 2 * L * D + 64) * 4))) return status;
+  uint32_t *next = (uint32_t *)c.tree.ptr;
   for (int m = n - 1; m >= 0; m--)
     for (int l = 0; l < L; l++) {
       uint64_t words = ((uint64_t)K << m) * D;
-      uint32_t *pp = bufs.alloc(words), *qq = bufs.alloc(words);
-      if (!pp || !qq) {
-        set_error("device-out-of-memory: GKR layers");
-        return E_NOMEM;
-      }
+      uint32_t *pp = next, *qq = next + words;
+      next += 2 * words;
       if ((status = gkr_reduce_layer(D, K, m, layers[m + 1][2 * l], layers[m + 1][2 * l + 1], pp, qq))) return status;
       layers[m][2 * l] = pp;
       layers[m][2 * l + 1] = qq;

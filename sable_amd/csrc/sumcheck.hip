@@ -119,6 +119,11 @@ const KernelSet *find_kernels(const std::string &key, int D) {
 }
 
 // ------------------------------------------------------------------ the session
+// regions of the context's pinned host buffer (in words): per-round results | the session's eq point
+// and block weights | the device loop's constants | the device loop's logs and final tables
+constexpr size_t PIN_BEGIN = 16384, PIN_BEGIN_WORDS = 4096;
+constexpr size_t PIN_LOOP = PIN_BEGIN + PIN_BEGIN_WORDS, PIN_LOOP_WORDS = 12288;
+constexpr size_t PIN_DOWN = PIN_LOOP + PIN_LOOP_WORDS, PIN_DOWN_WORDS = 32768;
 static inline uint32_t next_pow2(uint64_t v) {
   uint32_t p = 1;
   while (p < v) p <<= 1;
@@ -218,10 +223,11 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   uint64_t partial_off = pos * D;  // from here in words
   uint64_t words = partial_off + (max_grid + 1) * (uint64_t)pstride + 64;
   // the device-driven loop's constants: control block | message map | constant-group terms
-  uint64_t ctrl_off = (words + 63) & ~(uint64_t)63;
-  uint64_t mt_off = ctrl_off + (sizeof(Ctrl) + 3) / 4;
+  // (message map | constant terms | control block: one upload covers the first two and the block's head)
+  uint64_t mt_off = (words + 63) & ~(uint64_t)63;
   uint64_t c0_off = mt_off + (uint64_t)points * std::max(st.nacc, 1) * D;
-  words = c0_off + (uint64_t)std::max(n, 1) * points * D + 64;
+  uint64_t ctrl_off = c0_off + (uint64_t)std::max(n, 1) * points * D;
+  words = ctrl_off + (sizeof(Ctrl) + 3) / 4 + 64;
   // mixed base / extension inputs: lift the base ones
   bool any_base = false, all_base = true;
   for (int t = 0; t < T; t++) {
@@ -265,7 +271,13 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   }
 
   // ---- upload the eq factors and block weights, build the weight tables
-  std::vector<uint32_t> host((size_t)(2 * n + (has_bw ? K : 0)) * D, 0);
+  // staged in pinned memory when it fits (no wait: the region is not written again before this
+  // session's next wait), else in a vector that must outlive the copy
+  const size_t host_words = (size_t)(2 * n + (has_bw ? K : 0)) * D;
+  const bool staged = host_words <= PIN_BEGIN_WORDS;
+  std::vector<uint32_t> spill(staged ? 0 : host_words, 0);
+  uint32_t *host = staged ? c.host_pinned + PIN_BEGIN : spill.data();
+  if (staged) memset(host, 0, host_words * 4);
   if (has_eq)
     for (int v = 0; v < n; v++)
       for (int k = 0; k < D; k++) {
@@ -275,8 +287,8 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
       }
   if (has_bw)
     for (size_t i = 0; i < (size_t)K * D; i++) host[(size_t)2 * n * D + i] = bw[i] % P;
-  if (!host.empty()) EXH_HIP(hipMemcpyAsync(base, host.data(), host.size() * 4, hipMemcpyHostToDevice, c.stream));
-  EXH_HIP(hipStreamSynchronize(c.stream));  // host vector goes out of scope
+  if (host_words) EXH_HIP(hipMemcpyAsync(base, host, host_words * 4, hipMemcpyHostToDevice, c.stream));
+  if (!staged) EXH_HIP(hipStreamSynchronize(c.stream));
   if (has_eq && total_eq) {
     uint32_t grid = (uint32_t)((total_eq + BLOCK - 1) / BLOCK);
     // tables are laid out in launch order, so thread gid maps to table k by running sums; the
@@ -507,12 +519,16 @@ int SumcheckSession::finish(uint32_t *finals, uint32_t *const *folded) {
   if (status) return status;
   int T = st.T();
   // each table's current entries (K of them after n rounds), lifted if still base
-  std::vector<uint32_t> tmp;
-  for (int t = 0; t < T; t++) {
-    uint64_t words = size * (cur_base ? 1 : D);
-    tmp.resize(words);
-    EXH_HIP(hipMemcpyAsync(tmp.data(), cur[t], words * 4, hipMemcpyDeviceToHost, c.stream));
+  const uint64_t words = size * (cur_base ? 1 : D);
+  const bool cached = !cur_base && final_cache.size() == (size_t)T * words;
+  std::vector<uint32_t> all(cached ? 0 : (size_t)T * words);
+  if (!cached) {
+    for (int t = 0; t < T; t++)
+      EXH_HIP(hipMemcpyAsync(all.data() + (size_t)t * words, cur[t], words * 4, hipMemcpyDeviceToHost, c.stream));
     EXH_HIP(hipStreamSynchronize(c.stream));
+  }
+  for (int t = 0; t < T; t++) {
+    const uint32_t *tmp = (cached ? final_cache.data() : all.data()) + (size_t)t * words;
     for (uint64_t x = 0; x < size; x++) {
       uint32_t e[8] = {0};
       if (cur_base)
@@ -544,10 +560,18 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   if (n == 0) return OK;
   const int T = st.T(), nacc = st.nacc;
   // ---- constants: control block, message map (times R), per-round constant terms
-  std::vector<uint32_t> up(((sizeof(Ctrl) + 3) / 4) + (size_t)points * std::max(nacc, 1) * D + (size_t)n * points * D, 0);
-  Ctrl *hc = reinterpret_cast<Ctrl *>(up.data());
+  // (staged in pinned memory: message map | constant terms | head of the control block)
+  const size_t mt_words = (size_t)points * std::max(nacc, 1) * D, c0_words = (size_t)n * points * D;
+  const size_t head_words = offsetof(Ctrl, msg) / 4, up_words = mt_words + c0_words + head_words;
+  if (up_words > PIN_LOOP_WORDS) {
+    set_error("invalid-parameter: statement beyond the device loop's staging buffer");
+    return E_PARAM;
+  }
+  uint32_t *up = c.host_pinned + PIN_LOOP;
+  memset(up, 0, up_words * 4);
+  uint32_t *mt = up, *c0 = mt + mt_words;
+  Ctrl *hc = reinterpret_cast<Ctrl *>(c0 + c0_words);  // only its head is staged
   hc->tr = state;
-  uint32_t *mt = up.data() + (sizeof(Ctrl) + 3) / 4, *c0 = mt + (size_t)points * std::max(nacc, 1) * D;
   std::vector<int> wire(points);
   for (int k = 0; k < points; k++) wire[k] = k == 0 ? 0 : k + 1;
   for (size_t g = 0; g < st.groups.size(); g++) {
@@ -585,8 +609,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       }
     }
   }
-  EXH_HIP(hipMemcpyAsync(d_ctrl, up.data(), up.size() * 4, hipMemcpyHostToDevice, c.stream));
-  EXH_HIP(hipStreamSynchronize(c.stream));  // `up` is pageable host memory
+  EXH_HIP(hipMemcpyAsync(d_mtilde, up, up_words * 4, hipMemcpyHostToDevice, c.stream));
 
   device_loop = true;
   bool tail_done = false;
@@ -617,11 +640,17 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   }
   device_loop = false;
   if (status) return status;
-  // ---- read the logs back: one copy, one wait
-  std::vector<uint32_t> logs((sizeof(Ctrl) + 3) / 4);
-  EXH_HIP(hipMemcpyAsync(logs.data(), d_ctrl, sizeof(Ctrl), hipMemcpyDeviceToHost, c.stream));
+  // ---- read the logs back, and with them what the tail left of the tables: one wait for both
+  uint32_t *down = c.host_pinned + PIN_DOWN;
+  const size_t ctrl_words = (sizeof(Ctrl) + 3) / 4, final_words = (size_t)T * size * D;
+  EXH_HIP(hipMemcpyAsync(down, d_ctrl, sizeof(Ctrl), hipMemcpyDeviceToHost, c.stream));
+  final_cache.clear();
+  const bool with_finals = tail_done && ctrl_words + final_words <= PIN_DOWN_WORDS;
+  if (with_finals)  // the tail wrote table t at t * size * D of one arena
+    EXH_HIP(hipMemcpyAsync(down + ctrl_words, cur[0], final_words * 4, hipMemcpyDeviceToHost, c.stream));
   EXH_HIP(hipStreamSynchronize(c.stream));
-  const Ctrl *rc = reinterpret_cast<const Ctrl *>(logs.data());
+  if (with_finals) final_cache.assign(down + ctrl_words, down + ctrl_words + final_words);
+  const Ctrl *rc = reinterpret_cast<const Ctrl *>(down);
   if ((int)rc->round != n) {
     set_error("device-error: the device loop completed " + std::to_string(rc->round) + " of " + std::to_string(n) +
               " rounds");

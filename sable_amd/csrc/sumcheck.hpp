@@ -42,6 +42,7 @@ struct SumcheckSession {
   uint32_t pstride = 0;  // words per workgroup partial
   bool device_loop = false;
   Ctrl *d_ctrl = nullptr;
+  std::vector<uint32_t> final_cache;  // the tables as the device loop's tail left them, when read back with its logs
   uint32_t *d_mtilde = nullptr, *d_c0 = nullptr;
   bool pending_fold = false;
   uint32_t pending_r[8];
