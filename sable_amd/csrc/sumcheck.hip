@@ -699,7 +699,7 @@ int SumcheckSession::launch_tail(int j) {
       a.low_bits[jj] = (uint32_t)low_bits[j + jj];
     }
   };
-  c.prof_begin("tail", j, 0);
+  c.prof_begin("tail", j, (uint64_t)T * size * (cur_base ? 1 : D) * 4 + (uint64_t)T * final_size * D * 4);
   if (D == 4) {
     TailArgs<4> a;
     fill(a);
