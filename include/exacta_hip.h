@@ -86,6 +86,15 @@ int exh_sumcheck_begin(exh_stmt stmt, int degree_d, int n, const exh_table *tabl
 int exh_sumcheck_round(exh_session session, uint32_t *out_sums);
 /* FOLD-FLAT-TABLE of every table by the round's challenge, src/sumcheck.lisp:562, 84-104 */
 int exh_sumcheck_fold(exh_session session, const uint32_t *r);
+/* Every round of a fresh session back to back on the device, the Fiat-Shamir transcript included: the loop
+   body of PROVE (src/sumcheck.lisp:546-563) with SEND and CHALLENGE (src/transcript.lisp:116-128, 174-176)
+   run by the device on the sequential BLAKE3 state (src/blake3.lisp:125-155) the host's transcript holds after
+   absorbing the header (src/sumcheck.lisp:534): cv (8 words), the pending block (64 bytes, zero beyond
+   `used`), used, counter.  out_messages: n * max(degree,1) * D words; out_challenges: n * D words.  The host
+   sends the messages through its own transcript afterwards and must draw the same challenges.  Statements
+   of more than 7 wire points are rejected (use the round-by-round calls). */
+int exh_sumcheck_run(exh_session session, const uint32_t *cv, const uint8_t *block, uint32_t used, uint64_t counter,
+                     uint32_t *out_messages, uint32_t *out_challenges);
 /* finals: n_tables * D words (entry 0 of each folded table); folded: NULL, or n_tables pointers to
    K * D words (src/sumcheck.lisp:564-571).  Ends the session. */
 int exh_sumcheck_finish(exh_session session, uint32_t *finals, uint32_t *const *folded);

@@ -38,6 +38,9 @@ int exh_transcript_challenge_bits(exh_transcript tr, int nbits, int k, uint64_t 
 int exh_transcript_grind(exh_transcript tr, int bits, uint64_t *nonce);                          /* :196-201 */
 int exh_transcript_verify_grind(exh_transcript tr, int bits, uint64_t *nonce);                   /* :203-209 */
 int exh_transcript_digest(exh_transcript tr, uint8_t out[32]);
+/* the sequential-mode hash state behind the transcript (src/blake3.lisp:125-134): chaining value,
+   pending block (zero beyond *used), bytes pending, blocks compressed -- what exh_sumcheck_run takes */
+int exh_transcript_state(exh_transcript tr, uint32_t cv[8], uint8_t block[64], uint32_t *used, uint64_t *counter);
 int exh_transcript_finished(exh_transcript tr);
 int exh_transcript_message_count(exh_transcript tr, uint64_t *count);
 /* ENCODE-PROOF of the messages so far (src/proofio.lisp:45-49): size in *out_len; bytes written when

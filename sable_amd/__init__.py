@@ -296,6 +296,16 @@ class SumcheckSession:
         r = _u32(r)
         check(load().exh_sumcheck_fold(C.c_uint64(self.handle), _p(r)))
 
+    def run(self, tr, n):
+        """All n rounds on the device from the transcript's present hash state: (messages, challenges).  The
+        caller's transcript is not advanced; it replays the messages itself."""
+        cv, block = np.zeros(8, np.uint32), (C.c_uint8 * 64)()
+        used, counter = C.c_uint32(), C.c_uint64()
+        check(load().exh_transcript_state(tr.h, _p(cv), block, C.byref(used), C.byref(counter)))
+        msgs, chal = np.zeros((n, self.points, self.d), np.uint32), np.zeros((n, self.d), np.uint32)
+        check(load().exh_sumcheck_run(C.c_uint64(self.handle), _p(cv), block, used, counter, _p(msgs), _p(chal)))
+        return msgs, chal
+
     def finish(self):
         finals = np.zeros((self.T, self.d), np.uint32)
         folded = [np.zeros((self.K, self.d), np.uint32) for _ in range(self.T)]

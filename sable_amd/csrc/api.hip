@@ -272,6 +272,22 @@ int exh_sumcheck_fold(exh_session session, const uint32_t *r) {
   SumcheckSession *s = session_of(session);
   return s ? s->fold(r) : E_PARAM;
 }
+int exh_sumcheck_run(exh_session session, const uint32_t *cv, const uint8_t *block, uint32_t used, uint64_t counter,
+                     uint32_t *out_messages, uint32_t *out_challenges) {
+  SumcheckSession *s = session_of(session);
+  if (!s || !cv || !block || used > 64 || !out_messages || !out_challenges) {
+    set_error("invalid-parameter: exh_sumcheck_run arguments");
+    return E_PARAM;
+  }
+  DevB3S state;
+  memcpy(state.cv, cv, 32);
+  for (int i = 0; i < 16; i++)
+    state.block[i] = (uint32_t)block[4 * i] | (uint32_t)block[4 * i + 1] << 8 | (uint32_t)block[4 * i + 2] << 16 |
+                     (uint32_t)block[4 * i + 3] << 24;
+  state.used = used;
+  state.counter_lo = (uint32_t)counter, state.counter_hi = (uint32_t)(counter >> 32);
+  return s->run_device(state, out_messages, out_challenges);
+}
 int exh_sumcheck_finish(exh_session session, uint32_t *finals, uint32_t *const *folded) {
   SumcheckSession *s = session_of(session);
   if (!s) return E_PARAM;
@@ -392,6 +408,16 @@ int exh_transcript_digest(exh_transcript h, uint8_t out[32]) {
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   tr->state.digest(out, 32);
+  return OK;
+}
+int exh_transcript_state(exh_transcript h, uint32_t cv[8], uint8_t block[64], uint32_t *used, uint64_t *counter) {
+  Transcript *tr = tr_of(h);
+  if (!tr || !cv || !block || !used || !counter) return E_PARAM;
+  memcpy(cv, tr->state.cv, 32);
+  memset(block, 0, 64);
+  memcpy(block, tr->state.block, tr->state.used);
+  *used = tr->state.used;
+  *counter = tr->state.counter;
   return OK;
 }
 int exh_transcript_finished(exh_transcript h) {

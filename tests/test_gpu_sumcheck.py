@@ -206,3 +206,29 @@ def test_linearity_and_fold_consistency_at_scale():
     assert sa.check_final(reduced, st, finals, constants=alpha)
     for t in dev:
         t.free()
+
+
+def test_device_loop_entry_point_from_a_host_transcript_state():
+    """exh_sumcheck_run: the host absorbs the header, hands over its hash state, and replays the messages."""
+    n, d = 11, 4
+    rng = np.random.default_rng(6)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in range(3)]
+    eq, alpha = rand_ext(rng, (n,), d), rand_ext(rng, (1,), d)
+    st, ost = both(CONFIG2, ["t0", "t1", "t2"], ["alpha"])
+    otr = orc.Transcript("run", d)
+    rho, finals, _ = orc.prove(otr, n, ost, tables, eq=eq, constants=alpha)
+    want = orc.decode_proof(otr.proof())
+    dev = [sa.Table.upload(t) for t in tables]
+    tr = sa.Transcript("run", d)
+    tr.absorb(b"sc|" + n.to_bytes(2, "little") + (3).to_bytes(2, "little") + (1).to_bytes(4, "little"))
+    s = sa.SumcheckSession(st, d, n, dev, eq=eq, constants=alpha)
+    msgs, chal = s.run(tr, n)
+    assert same(chal, rho)
+    for j in range(n):
+        assert same(msgs[j], want[j])
+        tr.send(msgs[j])
+        assert same(tr.challenge(), chal[j])
+    got_finals, _ = s.finish()
+    assert same(got_finals, finals) and tr.proof() == otr.proof()
+    for t in dev:
+        t.free()
