@@ -129,10 +129,9 @@ int exh_table_alloc(uint64_t n_u32, int stride, exh_table *out) {
     set_error("invalid-parameter: table stride");
     return E_PARAM;
   }
-  void *ptr = nullptr;
-  hipError_t e = hipMalloc(&ptr, n_u32 ? n_u32 * 4 : 4);
-  if (e != hipSuccess) {
-    set_error(std::string("device-out-of-memory: ") + hipGetErrorString(e));
+  void *ptr = ctx().pool.alloc(n_u32 * 4);
+  if (!ptr) {
+    set_error("device-out-of-memory: table of " + std::to_string(n_u32 * 4) + " bytes");
     return E_NOMEM;
   }
   *out = add_table((uint32_t *)ptr, n_u32, stride, true);
@@ -178,8 +177,7 @@ int exh_table_download(exh_table table, uint64_t offset_u32, uint32_t *host, uin
 int exh_table_free(exh_table table) {
   DeviceTable *dt = table_of(table);
   if (!dt) return E_PARAM;
-  (void)hipStreamSynchronize(ctx().stream);
-  if (dt->owned && dt->ptr) EXH_HIP(hipFree(dt->ptr));
+  if (dt->owned && dt->ptr) ctx().pool.release(dt->ptr);  // stream-ordered reuse: no wait
   ctx().tables.erase(table);
   return OK;
 }

@@ -102,12 +102,62 @@ static int get_domain(int n, Domain **out) {
 // all 2^S mids and C consecutive lows (C = tile / 2^S), so its loads are segments of C words and
 // every butterfly of these stages stays inside the tile.  With `first` the input is the message
 // m, read as m || m (src/rs.lisp:81).
+//
+// Inside the tile the stages run four at a time in registers: a thread gathers the 16 elements that
+// differ in the four stage bits, does the 32 butterflies, and scatters them back, so LDS and the
+// workgroup barrier are touched once per four stages.  LDS words are padded by one per 32 so that
+// the strided gathers fall on distinct banks.
+// A tile is 2^12 words, 16 per thread: a domain of 2^24 takes three passes (6 + 5 + 12 stages) with
+// global segments of at least 64 words.  The passes are bound by the butterflies' modular multiplies
+// (three quarter-rate integer multiplies each), not by their bytes: tiles of 2^14 words, which need
+// two passes only, measured slower (338 us against 295 us for both columns of 2^24).
 constexpr int NTT_TILE_BITS = 12;
+constexpr int NTT_BLOCK = 256;
+constexpr int NTT_MAX_UPPER_STAGES = 7;  // per pass above the last: segments of 2^(12-7) words at least
+__device__ __forceinline__ uint32_t ntt_pad(uint32_t e) { return e + (e >> 5); }
 
-__global__ __launch_bounds__(BLOCK) void ntt_pass_kernel(const uint32_t *in, uint32_t *out, int n, int b_hi, int b_lo,
-                                                         int tile_bits, const uint32_t *tw, LevelOffsets lv,
-                                                         int first, uint64_t in_stride, uint64_t out_stride) {
-  __shared__ uint32_t lds[1 << NTT_TILE_BITS];
+// R stages d_lo .. d_lo + R - 1 of the pass (stage d pairs tile indices differing in bit cbits + d)
+template <int R>
+__device__ __forceinline__ void ntt_round(uint32_t *lds, uint32_t tile, int cbits, int d_lo, int b_lo, int b_hi,
+                                          uint64_t top, const uint32_t *tw, const LevelOffsets &lv) {
+  const int p = cbits + d_lo;
+  for (uint32_t g = threadIdx.x; g < (tile >> R); g += NTT_BLOCK) {
+    const uint32_t upper = g >> p, e_base = (upper << (p + R)) | (g & ((1u << p) - 1));
+    uint32_t v[1 << R], t[(1 << R) - 1];
+    // the twiddles of stage d_lo + s: 2^(R-1-s) of them, index (top | mid above the stage bit)
+#pragma unroll
+    for (int s = R - 1; s >= 0; s--) {
+      const int b = b_lo + d_lo + s;
+      const uint32_t *level = tw + lv.off[b] + ((top << (b_hi - b)) | ((uint64_t)upper << (R - 1 - s)));
+#pragma unroll
+      for (int jh = 0; jh < (1 << (R - 1 - s)); jh++) t[(1 << (R - 1 - s)) - 1 + jh] = level[jh];
+    }
+#pragma unroll
+    for (int j = 0; j < (1 << R); j++) v[j] = lds[ntt_pad(e_base | ((uint32_t)j << p))];
+#pragma unroll
+    for (int s = R - 1; s >= 0; s--) {
+#pragma unroll
+      for (int jh = 0; jh < (1 << (R - 1 - s)); jh++) {
+        const uint32_t x = t[(1 << (R - 1 - s)) - 1 + jh];
+#pragma unroll
+        for (int jl = 0; jl < (1 << s); jl++) {
+          const int j = (jh << (s + 1)) | jl;
+          uint32_t a = v[j], tc = mont_mul(x, v[j + (1 << s)]);
+          v[j] = fadd(a, tc);
+          v[j + (1 << s)] = fsub(a, tc);
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < (1 << R); j++) lds[ntt_pad(e_base | ((uint32_t)j << p))] = v[j];
+  }
+}
+
+__global__ __launch_bounds__(NTT_BLOCK) void ntt_pass_kernel(const uint32_t *in, uint32_t *out, int n, int b_hi,
+                                                             int b_lo, int tile_bits, const uint32_t *tw,
+                                                             LevelOffsets lv, int first, uint64_t in_stride,
+                                                             uint64_t out_stride) {
+  extern __shared__ uint32_t lds[];  // 2^tile_bits words plus one per 32
   const int S = b_hi - b_lo + 1, cbits = tile_bits - S;
   const uint32_t tile = 1u << tile_bits, C = 1u << cbits;
   in += (uint64_t)blockIdx.y * in_stride;
@@ -116,28 +166,27 @@ __global__ __launch_bounds__(BLOCK) void ntt_pass_kernel(const uint32_t *in, uin
   const uint64_t top = blockIdx.x / chunks_per_top, chunk = blockIdx.x % chunks_per_top;
   const uint64_t base = (top << (b_hi + 1)) | (chunk << cbits);
   const uint64_t msg_mask = ((uint64_t)1 << (n - 1)) - 1;
-  for (uint32_t e = threadIdx.x; e < tile; e += BLOCK) {
+  for (uint32_t e = threadIdx.x; e < tile; e += NTT_BLOCK) {
     uint64_t g = base | ((uint64_t)(e >> cbits) << b_lo) | (e & (C - 1));
-    lds[e] = first ? in[g & msg_mask] : in[g];
+    lds[ntt_pad(e)] = first ? in[g & msg_mask] : in[g];
   }
   __syncthreads();
-  for (int b = b_hi; b >= b_lo; b--) {
-    const int d = b - b_lo;
-    const uint32_t *level = tw + lv.off[b];
-    for (uint32_t u = threadIdx.x; u < tile / 2; u += BLOCK) {
-      uint32_t cc = u & (C - 1), mm = u >> cbits;
-      uint32_t mid_lo = mm & ((1u << d) - 1), mid_hi = mm >> d;
-      uint32_t ia = ((((mid_hi << (d + 1)) | mid_lo)) << cbits) | cc, ib = ia + (1u << (d + cbits));
-      uint64_t k = (top << (b_hi - b)) | mid_hi;
-      uint32_t a = lds[ia], tc = mont_mul(level[k], lds[ib]);
-      lds[ia] = fadd(a, tc);
-      lds[ib] = fsub(a, tc);
-    }
+  for (int d_hi = S - 1; d_hi >= 0;) {
+    const int R = d_hi + 1 < 4 ? d_hi + 1 : 4, d_lo = d_hi - R + 1;
+    if (R == 4)
+      ntt_round<4>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
+    else if (R == 3)
+      ntt_round<3>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
+    else if (R == 2)
+      ntt_round<2>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
+    else
+      ntt_round<1>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
     __syncthreads();
+    d_hi = d_lo - 1;
   }
-  for (uint32_t e = threadIdx.x; e < tile; e += BLOCK) {
+  for (uint32_t e = threadIdx.x; e < tile; e += NTT_BLOCK) {
     uint64_t g = base | ((uint64_t)(e >> cbits) << b_lo) | (e & (C - 1));
-    out[g] = lds[e];
+    out[g] = lds[ntt_pad(e)];
   }
 }
 
@@ -165,7 +214,14 @@ int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_
   lv.levels = n - 1, lv.n = n;
   for (int l = 0; l < n - 1; l++) lv.off[l] = dom->off[l];
   int tile_bits = n - 1 < NTT_TILE_BITS ? n - 1 : NTT_TILE_BITS;  // a tile never spans two tops
-  // stages n-2 .. 0: the last pass takes the low tile_bits stages, earlier passes up to 7 each
+  const uint32_t lds_bytes = (((uint32_t)1 << tile_bits) + ((uint32_t)1 << tile_bits >> 5) + 1) * 4;
+  static bool lds_enabled = false;
+  if (!lds_enabled) {  // more than the default 64 KiB of dynamic LDS
+    EXH_HIP(hipFuncSetAttribute((const void *)ntt_pass_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                ((1 << NTT_TILE_BITS) + (1 << (NTT_TILE_BITS - 5)) + 1) * 4));
+    lds_enabled = true;
+  }
+  // stages n-2 .. 0: the last pass takes the low tile_bits stages, earlier passes share the rest
   int b = n - 2;
   bool first = true;
   while (b >= 0) {
@@ -174,11 +230,13 @@ int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_
       b_lo = 0;
     else {
       int remaining = b - tile_bits + 1;  // stages above the last pass
-      int take = remaining > 7 ? (remaining > 14 ? 7 : (remaining + 1) / 2) : remaining;
+      int take = remaining > NTT_MAX_UPPER_STAGES
+                     ? (remaining > 2 * NTT_MAX_UPPER_STAGES ? NTT_MAX_UPPER_STAGES : (remaining + 1) / 2)
+                     : remaining;
       b_lo = b - take + 1;
     }
     uint32_t grid = (uint32_t)(len >> tile_bits);
-    hipLaunchKernelGGL(ntt_pass_kernel, dim3(grid, ncols), dim3(BLOCK), 0, cx.stream,
+    hipLaunchKernelGGL(ntt_pass_kernel, dim3(grid, ncols), dim3(NTT_BLOCK), lds_bytes, cx.stream,
                        first ? d_messages : d_codewords, d_codewords, n, b, b_lo, tile_bits, dom->tw, lv, first ? 1 : 0,
                        first ? len / 2 : len, len);
     first = false;
@@ -233,12 +291,10 @@ int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d
 
 // ------------------------------------------------------------------ Merkle trees
 // LEAF-DIGEST (src/pcs.lisp:44-52) of leaf l of ncols codewords: one row of 4 symbols per column,
-// rows hashed 64 at a time and chained h = BLAKE3(h || d).  A thread per leaf.
-__global__ __launch_bounds__(BLOCK) void leaf_kernel(const uint32_t *cw, int ncols, uint64_t cw_len, uint64_t nleaves,
-                                                     uint32_t *digests) {
-  uint64_t l = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
-  if (l >= nleaves) return;
-  uint32_t h[8], d[8], m[16];
+// rows hashed 64 at a time and chained h = BLAKE3(h || d).
+__device__ __forceinline__ void column_leaf_digest(const uint32_t *cw, int ncols, uint64_t cw_len, uint64_t l,
+                                                   uint32_t h[8]) {
+  uint32_t d[8], m[16];
   bool have = false;
   for (int start = 0; start < ncols; start += 64) {
     int rows = ncols - start < 64 ? ncols - start : 64;
@@ -263,16 +319,11 @@ __global__ __launch_bounds__(BLOCK) void leaf_kernel(const uint32_t *cw, int nco
       have = true;
     }
   }
-  uint4 *o = reinterpret_cast<uint4 *>(digests + l * 8);
-  o[0] = make_uint4(h[0], h[1], h[2], h[3]);
-  o[1] = make_uint4(h[4], h[5], h[6], h[7]);
 }
 
 // leaf l of an oracle codeword of EXT8s: one row per coordinate, symbols 4l..4l+3
 // (ORACLE-ROWS, src/pcs.lisp:577-579): 128 bytes, two blocks
-__global__ __launch_bounds__(BLOCK) void oracle_leaf_kernel(const uint32_t *cw, uint64_t nleaves, uint32_t *digests) {
-  uint64_t l = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
-  if (l >= nleaves) return;
+__device__ __forceinline__ void oracle_leaf_digest(const uint32_t *cw, uint64_t l, uint32_t h[8]) {
   uint32_t sym[4][8];
 #pragma unroll
   for (int s = 0; s < 4; s++) {
@@ -280,7 +331,7 @@ __global__ __launch_bounds__(BLOCK) void oracle_leaf_kernel(const uint32_t *cw, 
 #pragma unroll
     for (int d = 0; d < 8; d++) sym[s][d] = e.c[d];
   }
-  uint32_t h[8], m[16];
+  uint32_t m[16];
   b3_iv(h);
 #pragma unroll
   for (int b = 0; b < 2; b++) {
@@ -291,22 +342,84 @@ __global__ __launch_bounds__(BLOCK) void oracle_leaf_kernel(const uint32_t *cw, 
     uint32_t flags = b == 0 ? B3_CHUNK_START : (B3_CHUNK_END | B3_ROOT);
     b3_compress(h, m, 0, 64, flags, h, 0);
   }
-  uint4 *o = reinterpret_cast<uint4 *>(digests + l * 8);
+}
+
+__device__ __forceinline__ void store_digest(uint32_t *p, const uint32_t h[8]) {
+  uint4 *o = reinterpret_cast<uint4 *>(p);
   o[0] = make_uint4(h[0], h[1], h[2], h[3]);
   o[1] = make_uint4(h[4], h[5], h[6], h[7]);
 }
+__device__ __forceinline__ void load_digest(const uint32_t *p, uint32_t h[8]) {
+  const uint4 *i = reinterpret_cast<const uint4 *>(p);
+  uint4 a = i[0], b = i[1];
+  h[0] = a.x, h[1] = a.y, h[2] = a.z, h[3] = a.w, h[4] = b.x, h[5] = b.y, h[6] = b.z, h[7] = b.w;
+}
 
-// one level of nodes: node = BLAKE3(left || right) (src/pcs.lisp:54-55, 64-77)
-__global__ __launch_bounds__(BLOCK) void node_kernel(const uint32_t *level, uint32_t *next, uint64_t n_next) {
-  uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
-  if (i >= n_next) return;
-  const uint4 *p = reinterpret_cast<const uint4 *>(level + 16 * i);
-  uint4 a = p[0], b = p[1], c = p[2], d = p[3];
-  uint32_t left[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w}, right[8] = {c.x, c.y, c.z, c.w, d.x, d.y, d.z, d.w}, h[8];
-  b3_node(left, right, h);
-  uint4 *o = reinterpret_cast<uint4 *>(next + 8 * i);
-  o[0] = make_uint4(h[0], h[1], h[2], h[3]);
-  o[1] = make_uint4(h[4], h[5], h[6], h[7]);
+// Up to `height` levels of nodes above 2 * BLOCK consecutive nodes of `level` (n of them), node =
+// BLAKE3(left || right) (src/pcs.lisp:54-55, 64-77), every level written behind the one below
+// (level k + 1 starts 8 * n_k words after level k) and carried to the next step through LDS.
+// LEAVES 0: `level` holds digests; 1: the bottom nodes are the leaf digests of ncols codewords
+// (written too); 2: of an oracle codeword.
+template <int LEAVES>
+__global__ __launch_bounds__(BLOCK) void subtree_kernel(uint32_t *level, uint64_t n, int height, const uint32_t *cw,
+                                                        int ncols, uint64_t cw_len) {
+  __shared__ uint32_t lds[BLOCK][9];  // a digest per row, padded against bank conflicts
+  const uint32_t t = threadIdx.x;
+  uint64_t first = (uint64_t)blockIdx.x * BLOCK;  // this workgroup's first node of the level being written
+  uint64_t count = n / 2;                         // nodes of that level
+  uint32_t *out = level + 8 * n;
+  uint32_t left[8], right[8], h[8];
+  if (first + t < count) {
+    const uint64_t c0 = 2 * (first + t);
+    if (LEAVES == 0) {
+      load_digest(level + 8 * c0, left);
+      load_digest(level + 8 * (c0 + 1), right);
+    } else {
+      if (LEAVES == 1) {
+        column_leaf_digest(cw, ncols, cw_len, c0, left);
+        column_leaf_digest(cw, ncols, cw_len, c0 + 1, right);
+      } else {
+        oracle_leaf_digest(cw, c0, left);
+        oracle_leaf_digest(cw, c0 + 1, right);
+      }
+      store_digest(level + 8 * c0, left);
+      store_digest(level + 8 * (c0 + 1), right);
+    }
+    b3_node(left, right, h);
+    store_digest(out + 8 * (first + t), h);
+#pragma unroll
+    for (int i = 0; i < 8; i++) lds[t][i] = h[i];
+  }
+  uint32_t width = BLOCK;  // nodes of the current level held by this workgroup (when full)
+  for (int s = 1; s < height; s++) {
+    __syncthreads();
+    out += 8 * count;
+    count /= 2, first /= 2, width /= 2;
+    const bool active = t < width && first + t < count;
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) left[i] = lds[2 * t][i], right[i] = lds[2 * t + 1][i];
+      b3_node(left, right, h);
+      store_digest(out + 8 * (first + t), h);
+    }
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) lds[t][i] = h[i];
+    }
+  }
+}
+
+// a tree of a single leaf: its digest is the whole tree
+template <int LEAVES>
+__global__ void single_leaf_kernel(uint32_t *level, const uint32_t *cw, int ncols, uint64_t cw_len) {
+  if (threadIdx.x || blockIdx.x) return;
+  uint32_t h[8];
+  if (LEAVES == 1)
+    column_leaf_digest(cw, ncols, cw_len, 0, h);
+  else
+    oracle_leaf_digest(cw, 0, h);
+  store_digest(level, h);
 }
 
 static int cap_level_of(uint64_t leaves) {  // src/pcs.lisp:57-59
@@ -315,25 +428,40 @@ static int cap_level_of(uint64_t leaves) {  // src/pcs.lisp:57-59
   return il - 1 - 7 > 0 ? il - 1 - 7 : 0;
 }
 
-// the levels above the leaf digests already at d_levels; returns the cap
-static int merkle_levels_device(uint32_t *d_levels, uint64_t nleaves, uint8_t *cap, uint64_t *cap_rows) {
+// Every level of the tree at d_levels (leaves first), a few launches of up to nine levels each; the
+// leaf digests are computed by the first launch (leaves 1: ncols codewords, 2: an oracle codeword) or
+// already there (0).  A single leaf (no node above it) is hashed by the same kernel's bottom step.
+static int merkle_tree_device(uint32_t *d_levels, uint64_t nleaves, int leaves, const uint32_t *cw, int ncols,
+                              uint64_t cw_len, uint8_t *cap, uint64_t *cap_rows) {
   Context &c = ctx();
   uint32_t *level = d_levels;
   uint64_t n = nleaves;
-  int lc = cap_level_of(nleaves), l = 0;
-  const uint32_t *cap_ptr = d_levels;
+  int lc = cap_level_of(nleaves);
+  uint64_t cap_off = 0;
+  for (int l = 0; l < lc; l++) cap_off += 8 * (nleaves >> l);
+  if (nleaves == 1 && leaves == 1)
+    hipLaunchKernelGGL(single_leaf_kernel<1>, dim3(1), dim3(64), 0, c.stream, level, cw, ncols, cw_len);
+  if (nleaves == 1 && leaves == 2)
+    hipLaunchKernelGGL(single_leaf_kernel<2>, dim3(1), dim3(64), 0, c.stream, level, cw, ncols, cw_len);
   while (n > 1) {
-    uint32_t *next = level + 8 * n;
+    int height = 0;
+    for (uint64_t v = n; v > 1 && height < 9; v >>= 1) height++;
     uint32_t grid = (uint32_t)((n / 2 + BLOCK - 1) / BLOCK);
-    hipLaunchKernelGGL(node_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, level, next, n / 2);
-    level = next;
-    n /= 2;
-    l++;
-    if (l == lc) cap_ptr = level;
+    if (leaves == 1)
+      hipLaunchKernelGGL(subtree_kernel<1>, dim3(grid), dim3(BLOCK), 0, c.stream, level, n, height, cw, ncols, cw_len);
+    else if (leaves == 2)
+      hipLaunchKernelGGL(subtree_kernel<2>, dim3(grid), dim3(BLOCK), 0, c.stream, level, n, height, cw, ncols, cw_len);
+    else
+      hipLaunchKernelGGL(subtree_kernel<0>, dim3(grid), dim3(BLOCK), 0, c.stream, level, n, height, cw, ncols, cw_len);
+    leaves = 0;
+    for (int s = 0; s < height; s++) {
+      level += 8 * n;
+      n /= 2;
+    }
   }
   EXH_HIP(hipGetLastError());
   *cap_rows = nleaves >> lc;
-  EXH_HIP(hipMemcpyAsync(cap, cap_ptr, 32 * *cap_rows, hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipMemcpyAsync(cap, d_levels + cap_off, 32 * *cap_rows, hipMemcpyDeviceToHost, c.stream));
   EXH_HIP(hipStreamSynchronize(c.stream));
   return OK;
 }
@@ -344,9 +472,7 @@ int merkle_commit_columns(const uint32_t *d_codewords, int ncols, int c, uint32_
   int status = cx.require();
   if (status) return status;
   uint64_t nleaves = (uint64_t)1 << (c - 1), cw_len = (uint64_t)1 << (c + 1);
-  uint32_t grid = (uint32_t)((nleaves + BLOCK - 1) / BLOCK);
-  hipLaunchKernelGGL(leaf_kernel, dim3(grid), dim3(BLOCK), 0, cx.stream, d_codewords, ncols, cw_len, nleaves, d_levels);
-  return merkle_levels_device(d_levels, nleaves, cap, cap_rows);
+  return merkle_tree_device(d_levels, nleaves, 1, d_codewords, ncols, cw_len, cap, cap_rows);
 }
 
 // ------------------------------------------------------------------ BaseFold
@@ -452,11 +578,11 @@ namespace {
 struct Owned {
   std::vector<void *> ptrs;
   ~Owned() {
-    for (void *p : ptrs) (void)hipFree(p);
+    for (void *p : ptrs) ctx().pool.release(p);
   }
   uint32_t *alloc(uint64_t words) {
-    void *p = nullptr;
-    if (hipMalloc(&p, words ? words * 4 : 4) != hipSuccess) {
+    void *p = ctx().pool.alloc(words * 4);
+    if (!p) {
       set_error("device-out-of-memory: BaseFold buffers");
       return nullptr;
     }
@@ -571,11 +697,9 @@ int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v
       o.levels = mem.alloc((2 * o.nleaves) * 8);
       if (!o.cw || !o.levels) return E_NOMEM;
       EXH_HIP(hipMemcpyAsync(o.cw, cw, cur * 32, hipMemcpyDeviceToDevice, c.stream));
-      uint32_t gl = (uint32_t)((o.nleaves + BLOCK - 1) / BLOCK);
-      hipLaunchKernelGGL(oracle_leaf_kernel, dim3(gl), dim3(BLOCK), 0, c.stream, o.cw, o.nleaves, o.levels);
       std::vector<uint8_t> cap(32 * 128);
       uint64_t rows = 0;
-      if ((status = merkle_levels_device(o.levels, o.nleaves, cap.data(), &rows))) return status;
+      if ((status = merkle_tree_device(o.levels, o.nleaves, 2, o.cw, 1, o.cw_len, cap.data(), &rows))) return status;
       if ((status = tr.send_bytes(cap.data(), (int64_t)(32 * rows), nullptr))) return status;
       oracles.push_back(o);
     }

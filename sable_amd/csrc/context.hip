@@ -34,6 +34,55 @@ void Arena::release() {
   bytes = 0;
 }
 
+static size_t pool_round(size_t bytes) {
+  size_t unit = bytes < ((size_t)1 << 20) ? 4096 : (size_t)1 << 20;
+  return bytes ? (bytes + unit - 1) / unit * unit : unit;
+}
+
+void *Pool::alloc(size_t bytes) {
+  size_t want = pool_round(bytes);
+  auto it = idle.find(want);
+  if (it != idle.end()) {
+    void *p = it->second;
+    idle.erase(it);
+    idle_bytes -= want;
+    return p;
+  }
+  void *p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) {
+    (void)hipGetLastError();
+    trim();
+    if (hipMalloc(&p, want) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+  }
+  sizes[p] = want;
+  return p;
+}
+
+void Pool::release(void *ptr) {
+  auto it = sizes.find(ptr);
+  if (it == sizes.end()) return;
+  constexpr size_t IDLE_LIMIT = (size_t)64 << 30;  // of the 288 GB
+  if (idle_bytes + it->second > IDLE_LIMIT) {
+    (void)hipFree(ptr);
+    sizes.erase(it);
+    return;
+  }
+  idle.emplace(it->second, ptr);
+  idle_bytes += it->second;
+}
+
+void Pool::trim() {
+  for (auto &kv : idle) {
+    (void)hipFree(kv.second);
+    sizes.erase(kv.second);
+  }
+  idle.clear();
+  idle_bytes = 0;
+}
+
 int Context::require() {
   if (!ready) {
     set_error("device-error: the library is not initialised (exh_init), or no MI355X is visible");
@@ -96,8 +145,9 @@ void ctx_shutdown() {
   (void)hipStreamSynchronize(c.stream);
   c.prof_clear();
   for (auto &kv : c.tables)
-    if (kv.second.owned && kv.second.ptr) (void)hipFree(kv.second.ptr);
+    if (kv.second.owned && kv.second.ptr) c.pool.release(kv.second.ptr);
   c.tables.clear();
+  c.pool.trim();
   c.fold_a.release();
   c.fold_b.release();
   c.misc.release();

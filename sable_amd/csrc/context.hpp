@@ -36,6 +36,19 @@ struct Arena {
   void release();
 };
 
+// Device buffers that are reused instead of returned to the driver: tables and per-proof buffers are
+// allocated and freed around every call, and hipMalloc / hipFree cost more than the kernels between
+// them.  Everything runs on the library's one stream, so a buffer given out again is safe to write
+// as soon as the earlier work queued on it has run: no wait on release.
+struct Pool {
+  std::multimap<size_t, void *> idle;  // by size
+  std::map<void *, size_t> sizes;      // every buffer the pool owns, live or idle
+  size_t idle_bytes = 0;
+  void *alloc(size_t bytes);  // nullptr when the device is out of memory (idle buffers are returned first)
+  void release(void *ptr);
+  void trim();                // hipFree of everything idle
+};
+
 // One timed kernel launch (HIP events on the library's stream), kept while profiling is on.
 struct ProfileEntry {
   std::string name;
@@ -59,6 +72,7 @@ struct Context {
   std::map<uint64_t, DeviceTable> tables;
   uint64_t next_handle = 1;
   Arena fold_a, fold_b;  // the two generations of folded tables
+  Pool pool;
   Arena misc;            // weights, partial sums, small results
   Arena tree;            // the layers of a fraction tree above its leaves, for the length of one proof
   uint32_t *host_pinned = nullptr;  // small pinned buffer for per-round results

@@ -153,11 +153,11 @@ int send_finals(Transcript &tr, int D, int ntables, const uint32_t *finals, hf::
 struct DeviceBuffers {  // frees what it allocated when the proof ends
   std::vector<void *> owned;
   ~DeviceBuffers() {
-    for (void *p : owned) (void)hipFree(p);
+    for (void *p : owned) ctx().pool.release(p);
   }
   uint32_t *alloc(uint64_t words) {
-    void *p = nullptr;
-    if (hipMalloc(&p, words ? words * 4 : 4) != hipSuccess) return nullptr;
+    void *p = ctx().pool.alloc(words * 4);
+    if (!p) return nullptr;
     owned.push_back(p);
     return (uint32_t *)p;
   }
