@@ -135,6 +135,7 @@ int ctx_init(int device) {
   c.host_pinned_words = 1 << 16;
   EXH_HIP(hipHostMalloc((void **)&c.host_pinned, c.host_pinned_words * 4, hipHostMallocDefault));
   c.device = device;
+  c.compute_units = prop.multiProcessorCount;
   c.ready = true;
   return OK;
 }

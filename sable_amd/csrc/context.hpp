@@ -68,6 +68,7 @@ struct Context {
   void prof_end();
   void prof_clear();
   int device = -1;
+  int compute_units = 0;
   hipStream_t stream = nullptr;
   std::map<uint64_t, DeviceTable> tables;
   uint64_t next_handle = 1;

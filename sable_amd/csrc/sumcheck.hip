@@ -103,8 +103,14 @@ static void launch_interp(const RoundArgs<D> &a, const StmtDesc &d, bool in_base
 }
 
 template <int D>
-static void launch_tail_interp(const TailArgs<D> &a, const StmtDesc &d, hipStream_t s) {
-  hipLaunchKernelGGL((tail_kernel_interp<D>), dim3(1), dim3(BLOCK), a.lds_bytes, s, a, d);
+static void launch_tail_interp(const TailArgs<D> &a, const StmtDesc &d, uint32_t grid, hipStream_t s) {
+  static bool large_lds = false;
+  if (a.lds_bytes > TAIL_LDS_BYTES && !large_lds) {
+    (void)hipFuncSetAttribute((const void *)tail_kernel_interp<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              SLICE_LDS_BYTES);
+    large_lds = true;
+  }
+  hipLaunchKernelGGL((tail_kernel_interp<D>), dim3(grid), dim3(BLOCK), a.lds_bytes, s, a, d);
 }
 
 // ------------------------------------------------------------------ registry of generated kernels
@@ -121,6 +127,7 @@ const KernelSet *find_kernels(const std::string &key, int D) {
 // ------------------------------------------------------------------ the session
 // regions of the context's pinned host buffer (in words): per-round results | the session's eq point
 // and block weights | the device loop's constants | the device loop's logs and final tables
+constexpr uint32_t SLICE_GROUPS = 16;  // rows of totals per round of a grid launch of LDS-resident slices
 constexpr size_t PIN_BEGIN = 16384, PIN_BEGIN_WORDS = 4096;
 constexpr size_t PIN_LOOP = PIN_BEGIN + PIN_BEGIN_WORDS, PIN_LOOP_WORDS = 12288;
 constexpr size_t PIN_DOWN = PIN_LOOP + PIN_LOOP_WORDS, PIN_DOWN_WORDS = 32768;
@@ -221,7 +228,9 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   if (max_grid > 1024) max_grid = 1024;
   pstride = next_pow2((uint64_t)std::max(st.nacc, 1) * D);
   uint64_t partial_off = pos * D;  // from here in words
-  uint64_t words = partial_off + (max_grid + 1) * (uint64_t)pstride + 64;
+  // (a grid of LDS-resident slices keeps 64-bit totals per round and group in the same place)
+  const uint64_t partial_rows = std::max<uint64_t>(max_grid, 2 * MAXTAIL * SLICE_GROUPS);
+  uint64_t words = partial_off + (partial_rows + 1) * (uint64_t)pstride + 64;
   // the device-driven loop's constants: control block | message map | constant-group terms
   // (message map | constant terms | control block: one upload covers the first two and the block's head)
   uint64_t mt_off = (words + 63) & ~(uint64_t)63;
@@ -248,7 +257,7 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   uint32_t *base = (uint32_t *)c.misc.ptr;
   d_weights = base;
   d_partials = base + partial_off;
-  d_sums = d_partials + max_grid * (uint64_t)pstride;
+  d_sums = d_partials + partial_rows * (uint64_t)pstride;
   d_ctrl = reinterpret_cast<Ctrl *>(base + ctrl_off);
   d_mtilde = base + mt_off;
   d_c0 = base + c0_off;
@@ -614,11 +623,32 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   device_loop = true;
   bool tail_done = false;
   int status = OK, j = 0;
+  bool fold_due = false;  // the tables still await the fold by the last challenge drawn
   for (; j < n && status == OK; j++) {
-    uint64_t n_pairs = (size / (j == 0 ? 1 : 2)) / 2;  // pairs summed in round j (after the pending fold)
+    uint64_t n_pairs = (size / (fold_due ? 2 : 1)) / 2;  // pairs summed in round j (after the pending fold)
     if (n_pairs <= tail_pairs(T, D) && n - j <= MAXTAIL) break;
     round = j;
-    if (j == 0) {
+    // once every workgroup of a resident grid can hold its slice of the tables in LDS, the rounds down
+    // to where one workgroup suffices run in one launch
+    const bool pow2 = (size & (size - 1)) == 0;
+    const uint64_t slice_max = SLICE_LDS_BYTES / ((uint64_t)T * 2 * D * 4);
+    const uint64_t grid_max = std::min<uint64_t>(256, c.compute_units > 0 ? c.compute_units : 1);
+    if (pow2 && n_pairs > tail_pairs(T, D) && n_pairs <= slice_max * grid_max) {
+      int count = 0;
+      while ((n_pairs >> count) > tail_pairs(T, D) && count < MAXTAIL && j + count < n) count++;
+      const uint64_t left = 2 * (n_pairs >> count);  // entries per table after these rounds
+      uint64_t grid = 1;
+      while (grid * 2 <= grid_max && grid * 2 <= left && (n_pairs / (grid * 2)) >= BLOCK) grid *= 2;
+      while (n_pairs / grid > slice_max && grid * 2 <= grid_max && grid * 2 <= left) grid *= 2;
+      if (count > 0 && grid > 1 && n_pairs / grid <= slice_max) {
+        status = launch_tail(j, count, (uint32_t)grid, fold_due);
+        fold_due = false;
+        tail_done = status == OK;  // the tables are contiguous in one arena, nothing pending
+        j += count - 1;
+        continue;
+      }
+    }
+    if (!fold_due) {
       status = D == 4 ? launch_round<4>(*this, false, true, out_buf, n_pairs, j)
                       : launch_round<8>(*this, false, true, out_buf, n_pairs, j);
     } else {
@@ -633,9 +663,12 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       size = out_size;
       generation++;
     }
+    fold_due = true;
+    tail_done = false;
   }
   if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
-    status = launch_tail(j);
+    status = launch_tail(j, n - j, 1, fold_due);
+    fold_due = false;
     tail_done = status == OK;
   }
   device_loop = false;
@@ -661,22 +694,27 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     memcpy(challenges + (size_t)r * D, rc->chal[r], (size_t)D * 4);
   }
   round = n;
-  pending_fold = !tail_done;  // without a tail the last challenge's fold is still to do
+  pending_fold = fold_due;  // after a round kernel the last challenge's fold is still to do
   if (pending_fold) memcpy(pending_r, rc->chal[n - 1], (size_t)D * 4);
   return OK;
 }
 
-int SumcheckSession::launch_tail(int j) {
+int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fold) {
   Context &c = ctx();
   const int T = st.T();
-  const bool first_fold = j > 0;
-  // it folds (first_fold ? 1 : 0) + (n - j) times; the result goes where alternating arenas would put it
-  int folds = (first_fold ? 1 : 0) + (n - j);
+  // it folds (first_fold ? 1 : 0) + rounds times; the result goes where alternating arenas would put it
+  int folds = (first_fold ? 1 : 0) + rounds;
   uint64_t final_size = size >> folds;
   int last_gen = generation + folds - 1;
   Arena &dst = (last_gen % 2 == 0) ? c.fold_a : c.fold_b;
   int status = dst.reserve((size_t)T * final_size * D * 4);
   if (status) return status;
+  const uint64_t slice_entries = (first_fold ? size / 2 : size) / grid;
+  // groups of workgroups share a row of totals: few enough that a round's rows fit the scratch the
+  // kernel sums them in (MAXPTS * MAXACC * 8 words)
+  uint32_t groups = 1;
+  while (groups * 2 <= SLICE_GROUPS && groups * 2 <= grid && groups * 2 * (uint32_t)st.nacc * D <= MAXPTS * MAXACC * 8)
+    groups *= 2;
   auto fill = [&](auto &a) {
     memset(&a, 0, sizeof(a));
     for (int t = 0; t < T; t++) a.in[t] = cur[t];
@@ -685,35 +723,42 @@ int SumcheckSession::launch_tail(int j) {
     a.entries = (uint32_t)size;
     a.in_base = cur_base ? 1 : 0;
     a.first_fold = first_fold ? 1 : 0;
-    a.rounds = (uint32_t)(n - j);
+    a.rounds = (uint32_t)rounds;
     a.first_round = (uint32_t)j;
-    a.capacity = (uint32_t)(2 * tail_pairs(T, D));
+    a.capacity = (uint32_t)(grid > 1 ? slice_entries : 2 * tail_pairs(T, D));
     a.lds_bytes = (uint32_t)(T * a.capacity * D * 4);
     a.points = (uint32_t)points;
     a.ctrl = d_ctrl;
     a.mtilde = d_mtilde;
     a.c0 = d_c0 + (size_t)j * points * D;
-    for (int jj = 0; jj < n - j; jj++) {
+    a.totals = reinterpret_cast<unsigned long long *>(d_partials);
+    a.pstride = pstride;
+    a.groups = groups;
+    a.spin_limit = 200000;
+    for (int jj = 0; jj < rounds; jj++) {
       a.low_off[jj] = low_off[j + jj];
       a.high_off[jj] = high_off[j + jj];
       a.low_bits[jj] = (uint32_t)low_bits[j + jj];
     }
   };
-  c.prof_begin("tail", j, (uint64_t)T * size * (cur_base ? 1 : D) * 4 + (uint64_t)T * final_size * D * 4);
+  if (grid > 1)  // the rounds' totals start at zero (64-bit words)
+    EXH_HIP(hipMemsetAsync(d_partials, 0, (size_t)rounds * groups * pstride * 8, c.stream));
+  c.prof_begin(grid > 1 ? "slices" : "tail", j,
+               (uint64_t)T * size * (cur_base ? 1 : D) * 4 + (uint64_t)T * final_size * D * 4);
   if (D == 4) {
     TailArgs<4> a;
     fill(a);
     if (generated)
-      kernels->launch_tail(&a, c.stream);
+      kernels->launch_tail(&a, grid, c.stream);
     else
-      launch_tail_interp<4>(a, desc, c.stream);
+      launch_tail_interp<4>(a, desc, grid, c.stream);
   } else {
     TailArgs<8> a;
     fill(a);
     if (generated)
-      kernels->launch_tail(&a, c.stream);
+      kernels->launch_tail(&a, grid, c.stream);
     else
-      launch_tail_interp<8>(a, desc, c.stream);
+      launch_tail_interp<8>(a, desc, grid, c.stream);
   }
   c.prof_end();
   EXH_HIP(hipGetLastError());

@@ -14,7 +14,7 @@ namespace exh {
 
 struct KernelSet {  // the launchers generated for one statement and one degree D
   void (*launch)(const void *args, bool in_base, bool fold, uint32_t grid, hipStream_t stream);
-  void (*launch_tail)(const void *args, hipStream_t stream);
+  void (*launch_tail)(const void *args, uint32_t grid, hipStream_t stream);
 };
 void register_kernels(const std::string &key, int D, KernelSet set);
 const KernelSet *find_kernels(const std::string &key, int D);
@@ -62,7 +62,8 @@ struct SumcheckSession {
   // given B3S state; afterwards messages[j] (points * D words) and challenges[j] (D words) hold what
   // was sent and drawn, and the session is ready for finish().  Needs points <= MAXPTS.
   int run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges);
-  int launch_tail(int first_round);
+  // rounds first_round .. first_round + rounds - 1 with the tables in LDS, over `grid` workgroups
+  int launch_tail(int first_round, int rounds, uint32_t grid, bool first_fold);
   bool device_capable() const { return points <= MAXPTS && n <= MAXROUNDS; }
   int fold(const uint32_t *r /* D */);
   // finals: T * D; folded[t] (optional): K * D each

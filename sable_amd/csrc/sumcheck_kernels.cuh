@@ -56,27 +56,36 @@ struct RoundArgs {
   uint32_t pstride;          // words per workgroup partial (a power of two >= nacc * D)
 };
 
-// The rounds at the end of a sumcheck, all in one workgroup with the tables resident in LDS: no global
-// memory round trip separates a round's sums, its transcript step and its fold.
-constexpr uint32_t TAIL_LDS_BYTES = 32768;  // LDS given to the tables
+// The rounds below 2^18 pairs, with the tables resident in LDS: no global memory round trip separates a
+// round's sums, its transcript step and its fold.  With one workgroup (the last rounds) everything
+// stays on one compute unit; with a grid (the rounds before them) every workgroup keeps a contiguous
+// slice of every table, the round's sums meet in global totals (integer atomics that count their
+// contributions), and every workgroup runs the same transcript step, so each knows the next challenge.
+// The grid must be resident at once: the host launches at most one workgroup per compute unit.
+constexpr uint32_t TAIL_LDS_BYTES = 32768;        // LDS given to the tables of the one-workgroup launch
+constexpr uint32_t SLICE_LDS_BYTES = 128 * 1024;  // and to a workgroup's slices in the grid launch
 template <int D>
 struct TailArgs {
   const uint32_t *in[MAXT];  // tables of `entries` entries each; base (stride 1) when in_base
   uint32_t *out;             // where the folded tables go: table t at t * final_entries * D
   const uint32_t *weights;   // base of the weight tables
-  uint64_t low_off[MAXTAIL], high_off[MAXTAIL];  // in EXTs, per tail round
+  uint64_t low_off[MAXTAIL], high_off[MAXTAIL];  // in EXTs, per round
   uint32_t low_bits[MAXTAIL];
-  uint32_t entries;
+  uint32_t entries;          // per table, over all workgroups
   uint32_t in_base;
   uint32_t first_fold;       // fold by ctrl's challenge while loading
   uint32_t rounds;           // rounds summed here; a fold follows each
   uint32_t first_round;      // index of the first of them
-  uint32_t capacity;         // entries per table in LDS
+  uint32_t capacity;         // entries per table in a workgroup's LDS
   uint32_t lds_bytes;        // T * capacity * D * 4
   uint32_t points;
   Ctrl *ctrl;
   const uint32_t *mtilde;
   const uint32_t *c0;        // [rounds][points][D]
+  unsigned long long *totals;  // grid launch: [rounds][groups][pstride] counted sums, zeroed by the host
+  uint32_t pstride;
+  uint32_t groups;           // workgroup w adds into group w % groups
+  uint32_t spin_limit;       // polls of a total before giving up
 };
 
 template <int D>
@@ -322,14 +331,16 @@ __device__ __forceinline__ void round_message(const uint32_t *sums, uint32_t nac
 // the first wavefront's part: send the message, draw the challenge, log both (every lane the same steps)
 template <int D>
 __device__ __forceinline__ void transcript_step(RunB3S &tr, Ctrl *ctrl, uint32_t round, uint32_t points,
-                                                EpilogueLds *e) {
+                                                EpilogueLds *e, bool log = true) {
   const uint32_t tid = threadIdx.x;
   dev_absorb_words(tr, e->msg, points * D);
   dev_challenge(tr, D, e->chal);
-  for (uint32_t o = tid; o < points * D; o += 64) ctrl->msg[round][o] = e->msg[o];
+  if (log)
+    for (uint32_t o = tid; o < points * D; o += 64) ctrl->msg[round][o] = e->msg[o];
   if (tid < (uint32_t)D) {
-    ctrl->chal[round][tid] = e->chal[tid];
-    ctrl->r_mont[tid] = e->r_mont[tid] = to_mont(e->chal[tid]);
+    const uint32_t rm = to_mont(e->chal[tid]);
+    e->r_mont[tid] = rm;
+    if (log) ctrl->chal[round][tid] = e->chal[tid], ctrl->r_mont[tid] = rm;
   }
 }
 
@@ -349,14 +360,26 @@ __device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums,
   }
 }
 
+// One workgroup's share of a round: pairs [block * tile, (block + 1) * tile) with tile = BLOCK *
+// pairs_per_thread, folded first when FOLD, summed into the workgroup's partial row.
+template <int D>
+struct RoundShape {
+  const uint32_t *low, *high;
+  uint64_t n_pairs;
+  uint32_t low_bits, pairs_per_thread;
+  bool deferred, do_sums;
+};
+
 template <int D, bool IN_BASE, bool FOLD, class Desc>
-__device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &args) {
+__device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const *in, uint32_t *const *out,
+                                           const RoundShape<D> &sh, const Ext<D> &r, uint32_t block,
+                                           uint32_t *partial_row) {
   constexpr bool BASE_MODE = IN_BASE && !FOLD;  // the pair's values are base-field
   using V = typename std::conditional<BASE_MODE, uint32_t, Ext<D>>::type;
   const uint32_t tid = threadIdx.x;
-  const uint64_t tile = (uint64_t)BLOCK * args.pairs_per_thread;
-  const uint64_t tile_start = (uint64_t)blockIdx.x * tile;
-  const uint64_t low_mask = ((uint64_t)1 << args.low_bits) - 1;
+  const uint64_t tile = (uint64_t)BLOCK * sh.pairs_per_thread;
+  const uint64_t tile_start = (uint64_t)block * tile;
+  const uint64_t low_mask = ((uint64_t)1 << sh.low_bits) - 1;
 
   Acc96 acc[MAXACC][D];
 #pragma unroll
@@ -364,25 +387,18 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
 #pragma unroll
     for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
 
-  Ext<D> r = ext_zero<D>();
-  if constexpr (FOLD) {
-    const uint32_t *rp = args.ctrl ? args.ctrl->r_mont : args.r_mont;
-#pragma unroll
-    for (int c = 0; c < D; c++) r.c[c] = rp[c];
-  }
-
-  for (uint32_t k = 0; k < args.pairs_per_thread; k++) {
+  for (uint32_t k = 0; k < sh.pairs_per_thread; k++) {
     const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
-    if (i >= args.n_pairs) break;
+    if (i >= sh.n_pairs) break;
     V lo[MAXT], hi[MAXT];
-    load_pair<D, IN_BASE, FOLD, V>(d, args.in, args.out, i, r, lo, hi);
-    if (args.do_sums) {
-      Ext<D> w = load_ext<D>(args.low + (i & low_mask) * D);
-      if (!args.deferred) w = ext_mul_mont<D>(w, load_ext<D>(args.high + (i >> args.low_bits) * D));
+    load_pair<D, IN_BASE, FOLD, V>(d, in, out, i, r, lo, hi);
+    if (sh.do_sums) {
+      Ext<D> w = load_ext<D>(sh.low + (i & low_mask) * D);
+      if (!sh.deferred) w = ext_mul_mont<D>(w, load_ext<D>(sh.high + (i >> sh.low_bits) * D));
       accumulate_pair<D, V>(d, lo, hi, w, acc);
     }
   }
-  if (!args.do_sums) return;
+  if (!sh.do_sums) return;
 
   __shared__ uint32_t lds[BLOCK / 64][MAXACC * D];
   __shared__ uint32_t sums[MAXACC * D];
@@ -391,15 +407,61 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
     Ext<D> s;
 #pragma unroll
     for (int c = 0; c < D; c++) s.c[c] = sums[tid * D + c];
-    if (args.deferred) s = ext_mul_mont<D>(s, load_ext<D>(args.high + (tile_start >> args.low_bits) * D));
-    store_ext<D>(args.partials + (uint64_t)blockIdx.x * args.pstride + tid * D, s);
+    if (sh.deferred) s = ext_mul_mont<D>(s, load_ext<D>(sh.high + (tile_start >> sh.low_bits) * D));
+    store_ext<D>(partial_row + tid * D, s);
   }
+}
+
+template <int D, bool IN_BASE, bool FOLD, class Desc>
+__device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &args) {
+  Ext<D> r = ext_zero<D>();
+  if constexpr (FOLD) {
+    const uint32_t *rp = args.ctrl ? args.ctrl->r_mont : args.r_mont;
+#pragma unroll
+    for (int c = 0; c < D; c++) r.c[c] = rp[c];
+  }
+  RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
+                   args.do_sums != 0};
+  round_core<D, IN_BASE, FOLD>(d, args.in, args.out, sh, r, blockIdx.x,
+                               args.partials + (uint64_t)blockIdx.x * args.pstride);
 }
 
 // The round's second launch when the device drives the loop: one workgroup adds the partials, forms the
 // message, runs the transcript and leaves the next challenge in ctrl.  (A last-workgroup-done scheme
 // inside the round kernel needs a device-scope fence per workgroup, which on this part writes back the
 // XCD's whole L2 and costs more than a launch.)
+// sums[o] = sum over the workgroups' partial rows of word o (o < width): thread t takes column
+// t % pstride of the rows t / pstride, t / pstride + rstep, ...; four loads in flight per thread.
+// All threads of the workgroup call; scratch holds blockDim.x words.
+__device__ __forceinline__ void sum_partials(const uint32_t *partials, uint32_t nblocks, uint32_t ps, uint32_t width,
+                                             uint32_t *scratch, uint32_t *sums) {
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
+  for (uint32_t col0 = 0; col0 < ps; col0 += nthreads) {
+    const uint32_t col = col0 + (ps < nthreads ? tid % ps : tid);
+    const uint32_t row0 = ps < nthreads ? tid / ps : 0, rstep = ps < nthreads ? nthreads / ps : 1;
+    uint32_t v0 = 0, v1 = 0, v2 = 0, v3 = 0;
+    if (col < width) {
+      const uint32_t *p = partials + col;
+      uint32_t b = row0;
+      for (; b + 3 * rstep < nblocks; b += 4 * rstep) {
+        uint32_t x0 = p[(uint64_t)b * ps], x1 = p[(uint64_t)(b + rstep) * ps], x2 = p[(uint64_t)(b + 2 * rstep) * ps],
+                 x3 = p[(uint64_t)(b + 3 * rstep) * ps];
+        v0 = fadd(v0, x0), v1 = fadd(v1, x1), v2 = fadd(v2, x2), v3 = fadd(v3, x3);
+      }
+      for (; b < nblocks; b += rstep) v0 = fadd(v0, p[(uint64_t)b * ps]);
+    }
+    __syncthreads();
+    scratch[tid] = fadd(fadd(v0, v1), fadd(v2, v3));
+    __syncthreads();
+    if (tid < (ps < nthreads ? ps : nthreads) && col0 + tid < width) {
+      uint32_t total = scratch[tid];
+      for (uint32_t g = 1; g < rstep; g++) total = fadd(total, scratch[g * ps + tid]);
+      sums[col0 + tid] = total;
+    }
+  }
+  __syncthreads();
+}
+
 struct EpilogueArgs {
   const uint32_t *partials;
   uint32_t nblocks, pstride, nacc, points;
@@ -421,37 +483,14 @@ __global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) 
   if (tid == 64) epi.round = args.ctrl->round;
   for (uint32_t u = tid; u < args.points * width; u += EPI_BLOCK) epi.mtilde[u] = args.mtilde[u];
   for (uint32_t u = tid; u < args.points * D; u += EPI_BLOCK) epi.c0[u] = args.c0[u];
-  // sums[o] = sum over workgroups of partial[o]: thread t takes column t % pstride of the rows
-  // t / pstride, t / pstride + rstep, ...; four loads in flight per thread
-  for (uint32_t col0 = 0; col0 < ps; col0 += EPI_BLOCK) {
-    const uint32_t col = col0 + (ps < EPI_BLOCK ? tid % ps : tid);
-    const uint32_t row0 = ps < EPI_BLOCK ? tid / ps : 0, rstep = ps < EPI_BLOCK ? EPI_BLOCK / ps : 1;
-    uint32_t v0 = 0, v1 = 0, v2 = 0, v3 = 0;
-    if (col < width) {
-      const uint32_t *p = args.partials + col;
-      uint32_t b = row0;
-      for (; b + 3 * rstep < args.nblocks; b += 4 * rstep) {
-        uint32_t x0 = p[(uint64_t)b * ps], x1 = p[(uint64_t)(b + rstep) * ps], x2 = p[(uint64_t)(b + 2 * rstep) * ps],
-                 x3 = p[(uint64_t)(b + 3 * rstep) * ps];
-        v0 = fadd(v0, x0), v1 = fadd(v1, x1), v2 = fadd(v2, x2), v3 = fadd(v3, x3);
-      }
-      for (; b < args.nblocks; b += rstep) v0 = fadd(v0, p[(uint64_t)b * ps]);
-    }
-    __syncthreads();
-    scratch[tid] = fadd(fadd(v0, v1), fadd(v2, v3));
-    __syncthreads();
-    if (tid < (ps < EPI_BLOCK ? ps : EPI_BLOCK) && col0 + tid < width) {
-      uint32_t total = scratch[tid];
-      for (uint32_t g = 1; g < rstep; g++) total = fadd(total, scratch[g * ps + tid]);
-      sums[col0 + tid] = total;
-    }
-  }
-  __syncthreads();
+  sum_partials(args.partials, args.nblocks, ps, width, scratch, sums);
   round_epilogue<D>(args.ctrl, sums, args.nacc, args.points, epi.mtilde, epi.c0, &epi, true);
 }
 
-// The last rounds in one workgroup: load (folding or lifting on the way in) into LDS, then per round
-// sums -> message -> challenge -> fold without leaving the compute unit.  Thread i owns pair i.
+// Load (folding or lifting on the way in) into LDS, then per round sums -> message -> challenge -> fold
+// on the slice this workgroup holds: entries [w * E, (w + 1) * E) of every table, E = entries / grid.
+// A grid launch ends when its rounds are done and leaves the slices in `out` for the one-workgroup
+// launch that follows; that one ends with the finals.
 template <int D, class Desc>
 __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args) {
   extern __shared__ __align__(16) uint32_t tail_tables[];  // [T][capacity][D]
@@ -459,10 +498,12 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   __shared__ uint32_t sums[MAXACC * D];
   __shared__ EpilogueLds epi;
   __shared__ uint32_t c0s[MAXTAIL * MAXPTS * D];
-  const uint32_t tid = threadIdx.x, cap = args.capacity;
+  const uint32_t tid = threadIdx.x, cap = args.capacity, G = gridDim.x, wg = blockIdx.x;
+  const uint32_t width = (uint32_t)d.nacc * D;
+  if (args.ctrl->round != args.first_round) return;  // an earlier launch gave up: leave the count as it is
   RunB3S tr;
   if (tid < 64) rb3s_load(tr, epi.ring, &args.ctrl->tr);
-  uint32_t entries = args.first_fold ? args.entries / 2 : args.entries;
+  uint32_t entries = (args.first_fold ? args.entries / 2 : args.entries) / G;  // of this workgroup's slice
   {
     Ext<D> r = ext_zero<D>();
     if (args.first_fold) {
@@ -474,33 +515,35 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
       if (t < d.T) {
         const uint32_t *in = args.in[t];
         for (uint32_t x = tid; x < entries; x += BLOCK) {
+          const uint64_t gx = (uint64_t)wg * entries + x;  // index after the fold on the way in
           Ext<D> v;
           if (args.in_base) {
             if (args.first_fold) {
-              uint2 e = *reinterpret_cast<const uint2 *>(in + 2 * x);
+              uint2 e = *reinterpret_cast<const uint2 *>(in + 2 * gx);
               v = fold_base<D>(e.x, e.y, r);
             } else {
               v = ext_zero<D>();
-              v.c[0] = in[x];
+              v.c[0] = in[gx];
             }
           } else if (args.first_fold) {
-            v = fold_ext<D>(load_ext<D>(in + (size_t)2 * x * D), load_ext<D>(in + (size_t)(2 * x + 1) * D), r);
+            v = fold_ext<D>(load_ext<D>(in + 2 * gx * D), load_ext<D>(in + (2 * gx + 1) * D), r);
           } else {
-            v = load_ext<D>(in + (size_t)x * D);
+            v = load_ext<D>(in + gx * D);
           }
           store_ext<D>(tail_tables + ((size_t)t * cap + x) * D, v);
         }
       }
     }
-    for (uint32_t u = tid; u < args.points * (uint32_t)d.nacc * D; u += BLOCK) epi.mtilde[u] = args.mtilde[u];
+    for (uint32_t u = tid; u < args.points * width; u += BLOCK) epi.mtilde[u] = args.mtilde[u];
     for (uint32_t u = tid; u < args.rounds * args.points * D; u += BLOCK) c0s[u] = args.c0[u];
   }
-  // the weight of this thread's pair, fetched one round ahead
+  // the weight factors of this thread's first pair of a round, fetched one round ahead
   Ext<D> wl = ext_zero<D>(), wh = ext_zero<D>();
   auto fetch_weight = [&](uint32_t jj, uint32_t pairs) {
     if (tid < pairs) {
-      wl = load_ext<D>(args.weights + (args.low_off[jj] + (tid & ((1u << args.low_bits[jj]) - 1))) * D);
-      wh = load_ext<D>(args.weights + (args.high_off[jj] + (tid >> args.low_bits[jj])) * D);
+      const uint64_t i = (uint64_t)wg * pairs + tid;
+      wl = load_ext<D>(args.weights + (args.low_off[jj] + (i & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
+      wh = load_ext<D>(args.weights + (args.high_off[jj] + (i >> args.low_bits[jj])) * D);
     }
   };
   fetch_weight(0, entries / 2);
@@ -512,48 +555,93 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
     for (int a = 0; a < MAXACC; a++)
 #pragma unroll
       for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
-    if (tid < pairs) {
+    for (uint32_t i = tid; i < pairs; i += BLOCK) {
       Ext<D> lo[MAXT], hi[MAXT];
 #pragma unroll
       for (int t = 0; t < MAXT; t++)
         if (t < d.T) {
-          const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * tid) * D;
+          const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * i) * D;
           lo[t] = load_ext<D>(p);
           hi[t] = load_ext<D>(p + D);
         }
+      if (i >= BLOCK) {  // beyond the prefetched pair
+        const uint64_t gi = (uint64_t)wg * pairs + i;
+        wl = load_ext<D>(args.weights + (args.low_off[jj] + (gi & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
+        wh = load_ext<D>(args.weights + (args.high_off[jj] + (gi >> args.low_bits[jj])) * D);
+      }
       accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
     }
     if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
     block_sums<D>(d, acc, lds, sums);
+    if (G > 1) {
+      // The round's sums over all workgroups.  Each workgroup adds its sums into its group's totals,
+      // one integer atomic per word that also counts the contribution in the word's top 16 bits; a
+      // word whose count equals the group's size is complete, so readers poll the words themselves:
+      // nothing else is exchanged (the tables live in LDS), and no fence or separate barrier is needed.
+      // Groups keep the atomics on one address few.
+      const uint32_t NG = args.groups, gsize = G / NG;
+      unsigned long long *totals = args.totals + (size_t)jj * NG * args.pstride;
+      for (uint32_t o = tid; o < width; o += BLOCK)
+        __hip_atomic_fetch_add(totals + (size_t)(wg % NG) * args.pstride + o, ((unsigned long long)1 << 48) + sums[o],
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      int complete = 1;
+      for (uint32_t u = tid; u < NG * width; u += BLOCK) {
+        const unsigned long long *word = totals + (size_t)(u / width) * args.pstride + u % width;
+        unsigned long long v;
+        uint32_t polls = 0;
+        while (((v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 48) != gsize) {
+          if (++polls > args.spin_limit) {  // the grid is not all there: give up, the host sees the round count
+            complete = 0;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        epi.prod[u] = (uint32_t)((v & (((unsigned long long)1 << 48) - 1)) % P);
+      }
+      if (!__syncthreads_and(complete)) return;
+      for (uint32_t o = tid; o < width; o += BLOCK) {
+        uint32_t v = 0;
+        for (uint32_t g = 0; g < NG; g++) v = fadd(v, epi.prod[g * width + o]);
+        sums[o] = v;
+      }
+      __syncthreads();
+    }
     round_message<D>(sums, (uint32_t)d.nacc, args.points, epi.mtilde, c0s + (size_t)jj * args.points * D, &epi);
-    if (tid < 64) transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi);
+    if (tid < 64) transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi, wg == 0);
     __syncthreads();
-    Ext<D> r, folded[MAXT];
+    Ext<D> r;
 #pragma unroll
     for (int c = 0; c < D; c++) r.c[c] = epi.r_mont[c];
-    if (tid < pairs) {
+    // fold in place, 256 entries at a time in ascending order: a chunk's reads come before its writes,
+    // and its writes land below everything a later chunk reads
+    for (uint32_t base = 0; base < pairs; base += BLOCK) {
+      const uint32_t x = base + tid;
+      Ext<D> folded[MAXT];
+      if (x < pairs) {
 #pragma unroll
-      for (int t = 0; t < MAXT; t++)
-        if (t < d.T) {
-          const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * tid) * D;
-          folded[t] = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
-        }
-    }
-    __syncthreads();
-    if (tid < pairs) {
+        for (int t = 0; t < MAXT; t++)
+          if (t < d.T) {
+            const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * x) * D;
+            folded[t] = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
+          }
+      }
+      __syncthreads();
+      if (x < pairs) {
 #pragma unroll
-      for (int t = 0; t < MAXT; t++)
-        if (t < d.T) store_ext<D>(tail_tables + ((size_t)t * cap + tid) * D, folded[t]);
+        for (int t = 0; t < MAXT; t++)
+          if (t < d.T) store_ext<D>(tail_tables + ((size_t)t * cap + x) * D, folded[t]);
+      }
+      __syncthreads();
     }
-    __syncthreads();
     entries = pairs;
   }
 #pragma unroll
   for (int t = 0; t < MAXT; t++)
     if (t < d.T)
       for (uint32_t x = tid; x < entries; x += BLOCK)
-        store_ext<D>(args.out + ((size_t)t * entries + x) * D, load_ext<D>(tail_tables + ((size_t)t * cap + x) * D));
-  if (tid < 64) {
+        store_ext<D>(args.out + (((size_t)t * G + wg) * entries + x) * D,
+                     load_ext<D>(tail_tables + ((size_t)t * cap + x) * D));
+  if (wg == 0 && tid < 64) {
     rb3s_store(tr, &args.ctrl->tr);
     if (tid == 0) args.ctrl->round = args.first_round + args.rounds;
   }
