@@ -232,3 +232,20 @@ def test_device_loop_entry_point_from_a_host_transcript_state():
     assert same(got_finals, finals) and tr.proof() == otr.proof()
     for t in dev:
         t.free()
+
+
+@pytest.mark.parametrize("form,names,cnames,d,base,with_eq,n", [
+    (CONFIG3, ["c0", "c1", "c2", "c3"], [], 8, True, True, 17),
+    (CONFIG2, ["t0", "t1", "t2"], ["alpha"], 4, False, True, 18),
+    ("(* t0 t1)", ["t0", "t1"], [], 8, False, False, 16),
+    ("(+ (* t0 t1 t2) (* 7 t1) -1)", ["t0", "t1", "t2"], [], 4, True, True, 19),
+])
+def test_rounds_on_a_grid_of_lds_resident_slices(form, names, cnames, d, base, with_eq, n):
+    """Sizes at which the rounds between the large kernels and the last workgroup run as one launch of
+    many workgroups (base and extension inputs, with and without a pending fold, interpreter and generated
+    kernels): the proof bytes are the oracle's."""
+    rng = np.random.default_rng(n * 100 + d)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) if base else rand_ext(rng, (1 << n,), d) for _ in names]
+    eq = rand_ext(rng, (n,), d) if with_eq else None
+    consts = rand_ext(rng, (len(cnames),), d) if cnames else None
+    prove_both("slices", d, n, form, names, tables, eq=eq, constants=consts, cnames=cnames)
