@@ -136,3 +136,21 @@ def test_basefold_matches_the_oracle(nv):
     with pytest.raises(sa.VerificationFailure):
         sa.basefold_verify(sa.Transcript("bf", 4, proof=tr.proof()), nv, rr, orc.ext_add(v, orc.base_to_ext(1, 8)))
     t.free()
+
+
+def test_basefold_round_trip_beyond_the_oracle_sizes():
+    """nv = 19 (the oracle stops near 12): the claim comes from the device's hypercube sum with eq = the
+    point, the prover's own round checks pass, the verifier accepts the proof and its queries' fold
+    consistency, and rejects another claim."""
+    nv = 19
+    rng = np.random.default_rng(19)
+    h = sa.Table.random(77, 1 << nv, 8)
+    rr = rng.integers(0, P, (nv, 8), dtype=np.uint32)
+    v = sa.hypercube_sum(sa.Statement("t0", ["t0"]), nv, [h], 8, eq=rr)
+    tr = sa.Transcript("bf-large", 4)
+    qs, chal, final = sa.basefold_prove(tr, nv, rr, v, h)
+    assert len(chal) == nv - 5 and final.shape == (32, 8)
+    assert sa.basefold_verify(sa.Transcript("bf-large", 4, proof=tr.proof()), nv, rr, v) == qs
+    with pytest.raises(sa.VerificationFailure):
+        sa.basefold_verify(sa.Transcript("bf-large", 4, proof=tr.proof()), nv, rr, orc.ext_add(v, orc.base_to_ext(1, 8)))
+    h.free()
