@@ -136,7 +136,9 @@ __device__ __forceinline__ Ext<D> v_mul(const Ext<D> &a, const Ext<D> &b) { retu
 template <int D>
 __device__ __forceinline__ void v_weigh(Acc96 *acc, const Ext<D> &w, uint32_t v) { ext_scale_acc<D>(acc, w, v); }
 template <int D>
-__device__ __forceinline__ void v_weigh(Acc96 *acc, const Ext<D> &w, const Ext<D> &v) { ext_mul_acc<D>(acc, w, v); }
+__device__ __forceinline__ void v_weigh(Acc96 *acc, const Ext<D> &w, const Ext<D> &v) {
+  ext_mul_acc<D>(acc, v, w);  // the weight second: its tripled wrap coefficients are shared by the pair's points
+}
 
 // integer multiples and integer offsets, for the linear forms
 template <int D>
@@ -157,6 +159,19 @@ __device__ __forceinline__ Ext<D> v_offset(Ext<D> a, uint32_t k) {
   a.c[0] = fadd(a.c[0], k);
   return a;
 }
+
+// helpers of the weighted first factor (never reached with base values)
+template <int D, class V>
+__device__ __forceinline__ V v_of(const Ext<D> &w) {
+  if constexpr (std::is_same<V, uint32_t>::value)
+    return w.c[0];
+  else
+    return w;
+}
+template <int D>
+__device__ __forceinline__ void v_mul_acc(Acc96 *acc, uint32_t a, uint32_t b) { acc_mad(acc[0], a, b); }
+template <int D>
+__device__ __forceinline__ void v_mul_acc(Acc96 *acc, const Ext<D> &a, const Ext<D> &b) { ext_mul_acc<D>(acc, a, b); }
 
 template <int D, class V, class Desc>
 __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, const V *hi, const Ext<D> &w,
@@ -184,6 +199,17 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
       cur[d.T + v] = v_offset<D>(c0, d.vconst[v]);
       slope[d.T + v] = s0;
     }
+  // A group evaluated at three points or more carries the weight on its first factor: w * factor is a
+  // line too (two products per pair), and each point then needs one product fewer.  Extension values
+  // only: in the base field the products are cheap and the weight is the one extension operation.
+  constexpr bool EXT = !std::is_same<V, uint32_t>::value;
+  V wcur[MAXG], wslope[MAXG];
+#pragma unroll
+  for (int g = 0; g < MAXG; g++)
+    if (g < d.G && EXT && d.nev[g] >= 3 && d.deg[g] >= 2) {
+      wcur[g] = v_mul<D>(cur[d.tab[g][0]], v_of<D, V>(w));
+      wslope[g] = v_mul<D>(slope[d.tab[g][0]], v_of<D, V>(w));
+    }
 #pragma unroll
   for (int x = 0; x <= MAXX; x++) {
     if (x <= d.maxx) {
@@ -195,6 +221,9 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
           else if (t < d.T + d.NV)
             cur[t] = v_add<D>(cur[t], slope[t]);
         }
+#pragma unroll
+        for (int g = 0; g < MAXG; g++)
+          if (g < d.G && EXT && d.nev[g] >= 3 && d.deg[g] >= 2) wcur[g] = v_add<D>(wcur[g], wslope[g]);
       }
       int a = 0;
 #pragma unroll
@@ -204,11 +233,16 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
           for (int k = 0; k < MAXEV; k++) {
             if (k < d.nev[g]) {
               if (d.ev[g][k] == x) {
-                V prod = cur[d.tab[g][0]];
+                // the product of the factors but the last; the last goes with the accumulation
+                const bool pre = EXT && d.nev[g] >= 3 && d.deg[g] >= 2;
+                V prod = pre ? wcur[g] : cur[d.tab[g][0]];
 #pragma unroll
                 for (int j = 1; j < MAXDEG; j++)
-                  if (j < d.deg[g]) prod = v_mul<D>(prod, cur[d.tab[g][j]]);
-                v_weigh<D>(acc[a], w, prod);
+                  if (j < d.deg[g] - (pre ? 1 : 0)) prod = v_mul<D>(prod, cur[d.tab[g][j]]);
+                if constexpr (EXT)
+                  v_mul_acc<D>(acc[a], prod, pre ? cur[d.tab[g][d.deg[g] - 1]] : v_of<D, V>(w));
+                else
+                  v_weigh<D>(acc[a], w, prod);
               }
               a++;
             }
