@@ -89,8 +89,9 @@ EXH_HD void acc_add(Acc96 &a, uint64_t t) {
 EXH_HD void acc_mad(Acc96 &a, uint32_t x, uint32_t y) { acc_add(a, (uint64_t)x * y); }
 // the accumulator mod p, exactly
 EXH_HD uint32_t acc_reduce(const Acc96 &a) {
-  uint64_t v = (uint64_t)a.hi * R2 + (a.lo >> 32) * (uint64_t)R1 + (uint32_t)a.lo;  // < 2^64
-  return (uint32_t)(v % P);
+  // hi 2^64 + mid 2^32 + lo = (hi R^3 + mid R^2 + lo R) / R: two Montgomery reductions, no division
+  uint64_t v = (a.lo >> 32) * (uint64_t)R2 + (uint64_t)(uint32_t)a.lo * R1;  // < 2^32 (p + R1) < 4 p^2
+  return fadd(mont_reduce4(v), mont_mul(a.hi, R3));
 }
 
 // ---- tower arithmetic on D = 4 or 8 words in tower order
