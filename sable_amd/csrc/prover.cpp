@@ -26,11 +26,13 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
   if (degree < 0) degree = st.degree;
   int points = degree > 1 ? degree : 1;
   SumcheckSession s;
-  int status = s.begin(st, D, n, d_tables, strides, eq, bw, K, consts, degree);
+  const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS");
+  // the device drives the rounds when it can: the session then sends all its constants in one copy
+  const bool device_rounds = n > 0 && n <= MAXROUNDS && points <= MAXPTS && !(host_rounds && host_rounds[0] == '1');
+  int status = s.begin(st, D, n, d_tables, strides, eq, bw, K, consts, degree, false, device_rounds);
   if (status) return status;
   absorb_header(tr, label, n, degree, bw ? K : 1);
-  const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS");
-  if (n > 0 && s.device_capable() && !(host_rounds && host_rounds[0] == '1')) {
+  if (device_rounds && s.device_capable()) {
     // the rounds run back to back on the device, transcript included; the messages are then replayed
     // into this transcript, which must draw the same challenges
     DevB3S state;

@@ -139,7 +139,7 @@ static inline uint32_t next_pow2(uint64_t v) {
 
 int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uint32_t *const *tables,
                            const int *strides, const uint32_t *eq, const uint32_t *bw, int K_, const uint32_t *consts,
-                           int degree, bool claim_mode_) {
+                           int degree, bool claim_mode_, bool defer_setup) {
   Context &c = ctx();
   int status = c.require();
   if (status) return status;
@@ -189,6 +189,11 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
     bw_off = pos;
     pos += K;
   }
+  // the device-driven loop's constants follow at once, so that one copy can bring the eq point, the
+  // block weights, the message map, the constant-group terms and the control block's head
+  const uint64_t mt_words = (uint64_t)points * std::max(st.nacc, 1) * D, c0_words = (uint64_t)std::max(n, 1) * points * D;
+  const uint64_t mt_off = pos * D, c0_off = mt_off + mt_words, ctrl_off = c0_off + c0_words;
+  pos += (mt_words + c0_words + (sizeof(Ctrl) + 3) / 4 + D - 1) / D;
   for (int j = 0; j < n; j++) {
     int from = j + 1, middle = has_bw ? n : from + (n - from) / 2;
     low_bits[j] = middle - from;
@@ -231,12 +236,7 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   // (a grid of LDS-resident slices keeps 64-bit totals per round and group in the same place)
   const uint64_t partial_rows = std::max<uint64_t>(max_grid, 2 * MAXTAIL * SLICE_GROUPS);
   uint64_t words = partial_off + (partial_rows + 1) * (uint64_t)pstride + 64;
-  // the device-driven loop's constants: control block | message map | constant-group terms
-  // (message map | constant terms | control block: one upload covers the first two and the block's head)
-  uint64_t mt_off = (words + 63) & ~(uint64_t)63;
-  uint64_t c0_off = mt_off + (uint64_t)points * std::max(st.nacc, 1) * D;
-  uint64_t ctrl_off = c0_off + (uint64_t)std::max(n, 1) * points * D;
-  words = ctrl_off + (sizeof(Ctrl) + 3) / 4 + 64;
+  words += 64;
   // mixed base / extension inputs: lift the base ones
   bool any_base = false, all_base = true;
   for (int t = 0; t < T; t++) {
@@ -296,28 +296,49 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
       }
   if (has_bw)
     for (size_t i = 0; i < (size_t)K * D; i++) host[(size_t)2 * n * D + i] = bw[i] % P;
-  if (host_words) EXH_HIP(hipMemcpyAsync(base, host, host_words * 4, hipMemcpyHostToDevice, c.stream));
-  if (!staged) EXH_HIP(hipStreamSynchronize(c.stream));
-  if (has_eq && total_eq) {
-    uint32_t grid = (uint32_t)((total_eq + BLOCK - 1) / BLOCK);
-    // tables are laid out in launch order, so thread gid maps to table k by running sums; the
-    // offsets themselves may skip the block weights, so they are taken from eqt.off
-    if (D == 4)
-      hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, total_eq);
-    else
-      hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, total_eq);
-  }
-  if (!has_eq && ones_len) {
-    uint32_t grid = (uint32_t)((ones_len + BLOCK - 1) / BLOCK);
-    if (D == 4)
-      hipLaunchKernelGGL(fill_ones_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, base + ones_off * D, ones_len);
-    else
-      hipLaunchKernelGGL(fill_ones_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, base + ones_off * D, ones_len);
+  static_assert(sizeof(EqTables) <= sizeof(setup.eqt), "EqTables outgrew its stash");
+  memcpy(setup.eqt, &eqt, sizeof(eqt));
+  setup.total_eq = has_eq ? total_eq : 0;
+  setup.ones_off = ones_off, setup.ones_len = has_eq ? 0 : ones_len;
+  setup_words = host_words;
+  setup_deferred = defer_setup && staged;
+  if (!setup_deferred) {
+    if (host_words) EXH_HIP(hipMemcpyAsync(base, host, host_words * 4, hipMemcpyHostToDevice, c.stream));
+    if (!staged) EXH_HIP(hipStreamSynchronize(c.stream));
+    if ((status = launch_setup())) return status;
   }
   // the folded generations: the first holds half the input, the second a quarter
   if (n > 0) {
     if ((status = c.fold_a.reserve((size_t)T * (size / 2) * D * 4))) return status;
     if (n > 1 && (status = c.fold_b.reserve((size_t)T * (size / 4) * D * 4))) return status;
+  }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+// the weight tables of every round from the eq point's factors (or all-ones tables without one)
+int SumcheckSession::launch_setup() {
+  Context &c = ctx();
+  uint32_t *base = d_weights;
+  EqTables eqt;
+  memcpy(&eqt, setup.eqt, sizeof(eqt));
+  if (setup.total_eq) {
+    uint32_t grid = (uint32_t)((setup.total_eq + BLOCK - 1) / BLOCK);
+    // tables are laid out in launch order, so thread gid maps to table k by running sums; the
+    // offsets themselves may skip other regions, so they are taken from eqt.off
+    if (D == 4)
+      hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq);
+    else
+      hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq);
+  }
+  if (setup.ones_len) {
+    uint32_t grid = (uint32_t)((setup.ones_len + BLOCK - 1) / BLOCK);
+    if (D == 4)
+      hipLaunchKernelGGL(fill_ones_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, base + setup.ones_off * D,
+                         setup.ones_len);
+    else
+      hipLaunchKernelGGL(fill_ones_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, base + setup.ones_off * D,
+                         setup.ones_len);
   }
   EXH_HIP(hipGetLastError());
   return OK;
@@ -396,6 +417,10 @@ static hf::E weight_sum(const SumcheckSession &s, int j) {
 
 int SumcheckSession::round_sums(uint32_t *out) {
   Context &c = ctx();
+  if (setup_deferred) {
+    set_error("invalid-parameter: the session was set up for the device-driven loop");
+    return E_PARAM;
+  }
   if (round >= n) {
     set_error("invalid-parameter: no rounds left");
     return E_PARAM;
@@ -572,11 +597,12 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   // (staged in pinned memory: message map | constant terms | head of the control block)
   const size_t mt_words = (size_t)points * std::max(nacc, 1) * D, c0_words = (size_t)n * points * D;
   const size_t head_words = offsetof(Ctrl, msg) / 4, up_words = mt_words + c0_words + head_words;
-  if (up_words > PIN_LOOP_WORDS) {
+  if (setup_words + up_words > PIN_BEGIN_WORDS + PIN_LOOP_WORDS) {
     set_error("invalid-parameter: statement beyond the device loop's staging buffer");
     return E_PARAM;
   }
-  uint32_t *up = c.host_pinned + PIN_LOOP;
+  // (right behind the session's staged eq point and block weights: the device keeps the same order)
+  uint32_t *up = c.host_pinned + PIN_BEGIN + setup_words;
   memset(up, 0, up_words * 4);
   uint32_t *mt = up, *c0 = mt + mt_words;
   Ctrl *hc = reinterpret_cast<Ctrl *>(c0 + c0_words);  // only its head is staged
@@ -618,7 +644,15 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       }
     }
   }
-  EXH_HIP(hipMemcpyAsync(d_mtilde, up, up_words * 4, hipMemcpyHostToDevice, c.stream));
+  if (setup_deferred) {  // one copy for the session's constants and the loop's, then the weight tables
+    EXH_HIP(hipMemcpyAsync(d_weights, c.host_pinned + PIN_BEGIN, (setup_words + up_words) * 4, hipMemcpyHostToDevice,
+                           c.stream));
+    setup_deferred = false;
+    int st_setup = launch_setup();
+    if (st_setup) return st_setup;
+  } else {
+    EXH_HIP(hipMemcpyAsync(d_mtilde, up, up_words * 4, hipMemcpyHostToDevice, c.stream));
+  }
 
   device_loop = true;
   bool tail_done = false;
@@ -678,12 +712,14 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   const size_t ctrl_words = (sizeof(Ctrl) + 3) / 4, final_words = (size_t)T * size * D;
   EXH_HIP(hipMemcpyAsync(down, d_ctrl, sizeof(Ctrl), hipMemcpyDeviceToHost, c.stream));
   final_cache.clear();
-  const bool with_finals = tail_done && ctrl_words + final_words <= PIN_DOWN_WORDS;
+  const bool in_ctrl = tail_done && size == 1;  // the tail left the finals in the control block
+  const bool with_finals = tail_done && !in_ctrl && ctrl_words + final_words <= PIN_DOWN_WORDS;
   if (with_finals)  // the tail wrote table t at t * size * D of one arena
     EXH_HIP(hipMemcpyAsync(down + ctrl_words, cur[0], final_words * 4, hipMemcpyDeviceToHost, c.stream));
   EXH_HIP(hipStreamSynchronize(c.stream));
-  if (with_finals) final_cache.assign(down + ctrl_words, down + ctrl_words + final_words);
   const Ctrl *rc = reinterpret_cast<const Ctrl *>(down);
+  if (with_finals) final_cache.assign(down + ctrl_words, down + ctrl_words + final_words);
+  if (in_ctrl) final_cache.assign(rc->finals, rc->finals + final_words);
   if ((int)rc->round != n) {
     set_error("device-error: the device loop completed " + std::to_string(rc->round) + " of " + std::to_string(n) +
               " rounds");

@@ -53,7 +53,16 @@ struct SumcheckSession {
   // eq: n * D host words or null; bw: K * D host words or null; consts: C * D host words.
   int begin(const Statement &statement, int D, int n, const uint32_t *const *tables, const int *strides,
             const uint32_t *eq, const uint32_t *bw, int K, const uint32_t *consts, int degree,
-            bool claim_mode = false);
+            bool claim_mode = false, bool defer_setup = false);
+  // With defer_setup the eq point and block weights stay staged on the host and the weight-table
+  // kernels are not launched: run_device sends them with its own constants in one copy and launches then.
+  bool setup_deferred = false;
+  size_t setup_words = 0;
+  struct {
+    uint64_t total_eq = 0, ones_off = 0, ones_len = 0;
+    unsigned char eqt[1536];  // the EqTables argument of eq_tables_kernel
+  } setup;
+  int launch_setup();
   // claim mode: round_sums returns the honest claim sum_x w(x) F(tables(x)) in out[0..D) (n >= 1)
   bool claim_mode = false;
   std::vector<uint32_t> eq0;  // the eq point's first coordinate, for the claim

@@ -38,6 +38,7 @@ struct Ctrl {
   uint32_t pad[3];
   uint32_t msg[MAXROUNDS][MAXPTS * 8];
   uint32_t chal[MAXROUNDS][8];
+  uint32_t finals[MAXT * 8];  // entry 0 of every table once a single entry is left
 };
 template <int D>
 struct RoundArgs {
@@ -675,6 +676,8 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
       for (uint32_t x = tid; x < entries; x += BLOCK)
         store_ext<D>(args.out + (((size_t)t * G + wg) * entries + x) * D,
                      load_ext<D>(tail_tables + ((size_t)t * cap + x) * D));
+  if (G == 1 && entries == 1 && tid < (uint32_t)d.T * D)  // the finals travel with the logs
+    args.ctrl->finals[tid] = tail_tables[(size_t)(tid / D) * cap * D + tid % D];
   if (wg == 0 && tid < 64) {
     rb3s_store(tr, &args.ctrl->tr);
     if (tid == 0) args.ctrl->round = args.first_round + args.rounds;
