@@ -299,18 +299,103 @@ __device__ __forceinline__ void load_pair(const Desc &d, const uint32_t *const *
   }
 }
 
-// the workgroup's sums of every accumulator, reduced mod p, into sums[nacc * D] (LDS); all threads call
-template <int D, class Desc>
+// the value of lane (l ^ M) of the wavefront
+template <int M>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v) {
+  if constexpr (M == 1)
+    return EXH_DPP(v, 0xB1);  // quad_perm [1,0,3,2]
+  else if constexpr (M == 2)
+    return EXH_DPP(v, 0x4E);  // quad_perm [2,3,0,1]
+  else if constexpr (M == 8)
+    return EXH_DPP(v, 0x128);  // row_ror:8
+  else if constexpr (M == 4 || M == 16)
+    return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (M << 10) | 0x1f);  // xor within 32 lanes
+  else
+    return (uint32_t)__builtin_amdgcn_ds_bpermute((int)(((threadIdx.x & 63) ^ 32) << 2), (int)v);
+}
+
+// One step of the transposing reduction: the 2 * H values a lane holds become H, each the sum over
+// the lane pair (l, l ^ M); lanes with bit M clear keep the lower half of the values, the others the
+// upper half.
+template <int M, int H>
+__device__ __forceinline__ void halve_step(uint32_t *a) {
+  const bool upper = (threadIdx.x & M) != 0;
+#pragma unroll
+  for (int k = 0; k < H; k++) {
+    uint32_t keep = upper ? a[k + H] : a[k], send = upper ? a[k] : a[k + H];
+    a[k] = fadd(keep, lane_xor<M>(send));
+  }
+}
+
+// The wavefront's sums of W = 8, 16 or 32 values per lane, value k given by val(k): afterwards lane l
+// holds the sum over all 64 lanes of value bitrev(l mod W).  About 2 W cross-lane operations instead of
+// the 6 W of one reduction tree per value.  The first step consumes the values as they are produced, so
+// only W / 2 are live at once.
+template <int W, class F>
+__device__ __forceinline__ uint32_t wave_sums_transposed(F val) {
+  uint32_t a[W / 2];
+  const bool upper = (threadIdx.x & 1) != 0;
+#pragma unroll
+  for (int k = 0; k < W / 2; k++) {
+    uint32_t lo = val(k), hi = val(k + W / 2);
+    a[k] = fadd(upper ? hi : lo, lane_xor<1>(upper ? lo : hi));
+  }
+  if constexpr (W == 32) {
+    halve_step<2, 8>(a), halve_step<4, 4>(a), halve_step<8, 2>(a), halve_step<16, 1>(a);
+  } else if constexpr (W == 16) {
+    halve_step<2, 4>(a), halve_step<4, 2>(a), halve_step<8, 1>(a);
+    a[0] = fadd(a[0], lane_xor<16>(a[0]));
+  } else {
+    halve_step<2, 2>(a), halve_step<4, 1>(a);
+    a[0] = fadd(a[0], lane_xor<8>(a[0]));
+    a[0] = fadd(a[0], lane_xor<16>(a[0]));
+  }
+  return fadd(a[0], lane_xor<32>(a[0]));
+}
+
+// accumulator words [first, first + W) of the lane, reduced mod p (zero beyond the statement's), summed
+// over the wavefront and left in lds_row[first ..]
+template <int D, int W, class Desc>
+__device__ __forceinline__ void chunk_sums(const Desc &d, Acc96 (*acc)[D], int first, uint32_t *lds_row) {
+  const uint32_t total = wave_sums_transposed<W>([&](int k) -> uint32_t {
+    const int o = first + k;
+    return o < d.nacc * D ? acc_reduce(acc[o / D][o % D]) : 0u;
+  });
+  const uint32_t l = threadIdx.x & 63;
+  constexpr int BITS = W == 32 ? 5 : W == 16 ? 4 : 3;
+  uint32_t idx = 0;
+#pragma unroll
+  for (int b = 0; b < BITS; b++) idx |= ((l >> b) & 1u) << (BITS - 1 - b);
+  if (l < W && first + idx < (uint32_t)d.nacc * D) lds_row[first + idx] = total;
+}
+
+// The workgroup's sums of every accumulator, reduced mod p, into sums[nacc * D] (LDS); all threads call.
+// TRANSPOSED picks the cross-lane scheme: the transposing reduction is the shorter path (the latency-bound
+// LDS-resident rounds use it), one tree per value keeps fewer registers live (the streaming round kernels,
+// whose occupancy it would cost, use that).
+template <int D, bool TRANSPOSED, class Desc>
 __device__ __forceinline__ void block_sums(const Desc &d, Acc96 (*acc)[D], uint32_t (*lds)[MAXACC * D],
                                            uint32_t *sums) {
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if constexpr (TRANSPOSED) {
+    if (d.nacc * D <= 8)
+      chunk_sums<D, 8>(d, acc, 0, lds[wave]);
+    else if (d.nacc * D <= 16)
+      chunk_sums<D, 16>(d, acc, 0, lds[wave]);
+    else {
 #pragma unroll
-  for (int a = 0; a < MAXACC; a++) {
-    if (a < d.nacc) {
+      for (int first = 0; first < MAXACC * D; first += 32)
+        if (first < d.nacc * D) chunk_sums<D, 32>(d, acc, first, lds[wave]);
+    }
+  } else {
 #pragma unroll
-      for (int c = 0; c < D; c++) {
-        uint32_t v = wave_sum(acc_reduce(acc[a][c]));
-        if (lane == 0) lds[wave][a * D + c] = v;
+    for (int a = 0; a < MAXACC; a++) {
+      if (a < d.nacc) {
+#pragma unroll
+        for (int c = 0; c < D; c++) {
+          uint32_t v = wave_sum(acc_reduce(acc[a][c]));
+          if (lane == 0) lds[wave][a * D + c] = v;
+        }
       }
     }
   }
@@ -437,7 +522,7 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
 
   __shared__ uint32_t lds[BLOCK / 64][MAXACC * D];
   __shared__ uint32_t sums[MAXACC * D];
-  block_sums<D>(d, acc, lds, sums);
+  block_sums<D, false>(d, acc, lds, sums);
   if (tid < (uint32_t)d.nacc) {
     Ext<D> s;
 #pragma unroll
@@ -607,7 +692,7 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
       accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
     }
     if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
-    block_sums<D>(d, acc, lds, sums);
+    block_sums<D, true>(d, acc, lds, sums);
     if (G > 1) {
       // The round's sums over all workgroups.  Each workgroup adds its sums into its group's totals,
       // one integer atomic per word that also counts the contribution in the word's top 16 bits; a
