@@ -77,7 +77,8 @@ int exh_stmt_free(exh_stmt stmt);
 /* ---- one sumcheck, round by round: the call sites inside PROVE (src/sumcheck.lisp:547-563).
    tables: n_tables handles of K * 2^n entries each (block-major); eq: n * D words or NULL;
    block_weights: K * D words or NULL (then K must be 1); constants: n_constants * D words;
-   degree < 0: the statement's degree. */
+   degree < 0: the statement's degree.  One session is open at a time: beginning another (or any
+   whole-protocol call) hands the library's scratch arenas on, and the earlier session's calls then fail. */
 int exh_sumcheck_begin(exh_stmt stmt, int degree_d, int n, const exh_table *tables, int n_tables,
                        const uint32_t *eq, const uint32_t *block_weights, int K, const uint32_t *constants,
                        int degree, exh_session *out);

@@ -73,6 +73,7 @@ struct Context {
   std::map<uint64_t, DeviceTable> tables;
   uint64_t next_handle = 1;
   Arena fold_a, fold_b;  // the two generations of folded tables
+  uint64_t session_epoch = 0;  // bumped by every session begin: the arenas belong to the latest session
   Pool pool;
   Arena misc;            // weights, partial sums, small results
   Arena tree;            // the layers of a fraction tree above its leaves, for the length of one proof

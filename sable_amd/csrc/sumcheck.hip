@@ -144,6 +144,7 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   int status = c.require();
   if (status) return status;
   D = D_, n = n_, K = K_;
+  epoch = ++c.session_epoch;
   if ((D != 4 && D != 8) || n < 0 || n > 40 || K < 1) {
     set_error("invalid-parameter: sumcheck shape");
     return E_PARAM;
@@ -415,8 +416,15 @@ static hf::E weight_sum(const SumcheckSession &s, int j) {
   return wsum;
 }
 
+int SumcheckSession::owns_arenas() const {
+  if (epoch == ctx().session_epoch) return OK;
+  set_error("invalid-parameter: another sumcheck session was begun since; one session is open at a time");
+  return E_PARAM;
+}
+
 int SumcheckSession::round_sums(uint32_t *out) {
   Context &c = ctx();
+  if (int owned = owns_arenas()) return owned;
   if (setup_deferred) {
     set_error("invalid-parameter: the session was set up for the device-driven loop");
     return E_PARAM;
@@ -505,6 +513,7 @@ int SumcheckSession::round_sums(uint32_t *out) {
 }
 
 int SumcheckSession::fold(const uint32_t *r) {
+  if (int owned = owns_arenas()) return owned;
   if (round >= n || pending_fold) {
     set_error("invalid-parameter: nothing to fold");
     return E_PARAM;
@@ -549,6 +558,7 @@ int SumcheckSession::flush() {
 
 int SumcheckSession::finish(uint32_t *finals, uint32_t *const *folded) {
   Context &c = ctx();
+  if (int owned = owns_arenas()) return owned;
   int status = flush();
   if (status) return status;
   int T = st.T();
@@ -587,6 +597,7 @@ static uint64_t tail_pairs(int T, int D) {
 
 int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges) {
   Context &c = ctx();
+  if (int owned = owns_arenas()) return owned;
   if (round != 0 || pending_fold || claim_mode || !device_capable()) {
     set_error("invalid-parameter: the device loop starts a fresh session of at most 7 wire points");
     return E_PARAM;

@@ -56,6 +56,9 @@ struct SumcheckSession {
             bool claim_mode = false, bool defer_setup = false);
   // With defer_setup the eq point and block weights stay staged on the host and the weight-table
   // kernels are not launched: run_device sends them with its own constants in one copy and launches then.
+  uint64_t epoch = 0;  // Context::session_epoch at begin
+  // OK while this is the latest session begun (its arenas have not been handed to another one)
+  int owns_arenas() const;
   bool setup_deferred = false;
   size_t setup_words = 0;
   struct {

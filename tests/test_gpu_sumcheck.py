@@ -176,6 +176,13 @@ def test_round_by_round_session_matches_the_oracle_rounds():
     assert same(finals, [t[0] for t in cur])
     with pytest.raises(sa.InvalidParameter):
         sa.SumcheckSession(st, d, n, dev[:2], eq=eq, constants=alpha)
+    # one session at a time: a second begin takes the scratch arenas, the first then refuses to go on
+    first = sa.SumcheckSession(st, d, n, dev, eq=eq, constants=alpha)
+    second = sa.SumcheckSession(st, d, n, dev, eq=eq, constants=alpha)
+    with pytest.raises(sa.InvalidParameter):
+        first.round()
+    assert same(second.round(), orc.round_sums(ost, d, 3, tables, orc.eq_table(eq[1:1 + (n - 1) // 2], d),
+                                               orc.eq_table(eq[1 + (n - 1) // 2:], d), alpha))
     for t in dev:
         t.free()
 
