@@ -196,7 +196,11 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   const uint64_t mt_off = pos * D, c0_off = mt_off + mt_words, ctrl_off = c0_off + c0_words;
   pos += (mt_words + c0_words + (sizeof(Ctrl) + 3) / 4 + D - 1) / D;
   for (int j = 0; j < n; j++) {
-    int from = j + 1, middle = has_bw ? n : from + (n - from) / 2;
+    // LOW takes the lower half of the remaining variables as in SPLIT-WEIGHTS, but at least as many as a
+    // workgroup's tile of pairs spans (2^13), so that one HIGH weight covers the tile and is applied
+    // once per workgroup; the weights are the same products either way
+    int from = j + 1, rest = n - from;
+    int middle = has_bw ? n : from + std::max(rest / 2, std::min(rest, 13));
     low_bits[j] = middle - from;
     n_high[j] = has_bw ? (uint64_t)K : (uint64_t)1 << (n - middle);
     if (has_eq) {
