@@ -236,7 +236,9 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   uint64_t pairs0 = size / 2;
   max_grid = pairs0 ? (pairs0 + BLOCK - 1) / BLOCK : 1;
   if (max_grid > 1024) max_grid = 1024;
-  pstride = next_pow2((uint64_t)std::max(st.nacc, 1) * D);
+  node_slots_n = 0;  // slots of the base-field round 1 (group, point, node)
+  for (int g = 0; g < desc.G; g++) node_slots_n += desc.nev[g] * (desc.deg[g] + 1);
+  pstride = next_pow2((uint64_t)std::max(std::max(st.nacc, 1), node_slots_n <= MAXACC ? node_slots_n : 0) * D);
   uint64_t partial_off = pos * D;  // from here in words
   // (a grid of LDS-resident slices keeps 64-bit totals per round and group in the same place)
   const uint64_t partial_rows = std::max<uint64_t>(max_grid, 2 * MAXTAIL * SLICE_GROUPS);
@@ -351,7 +353,7 @@ int SumcheckSession::launch_setup() {
 
 template <int D>
 static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::vector<uint32_t *> &outs,
-                        uint64_t n_pairs, int j) {
+                        uint64_t n_pairs, int j, bool double_fold = false) {
   Context &c = ctx();
   RoundArgs<D> a;
   memset(&a, 0, sizeof(a));
@@ -373,17 +375,23 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   a.deferred = do_sums && ((uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits)) ? 1 : 0;
   a.partials = s.d_partials;
   a.pstride = s.pstride;
+  a.double_fold = double_fold ? 1 : 0;
   if (s.device_loop) a.ctrl = s.d_ctrl;
   if (fold && !s.device_loop)
     for (int k = 0; k < D; k++) a.r_mont[k] = to_mont(s.pending_r[k]);
   uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
   {
     // bytes this launch must move: every table read once, the folded tables written once
-    uint64_t in_words = (fold ? 4 : 2) * n_pairs * (s.cur_base ? 1 : D), out_words = fold ? 2 * n_pairs * D : 0;
-    const char *name = fold ? (s.cur_base ? "round_fold_base" : "round_fold_ext") : (s.cur_base ? "round_base" : "round_ext");
+    uint64_t in_words = (double_fold ? 8 : fold ? 4 : 2) * n_pairs * (s.cur_base ? 1 : D),
+             out_words = fold ? 2 * n_pairs * D : 0;
+    const char *name = double_fold ? "round_fold2_base"
+                       : fold      ? (s.cur_base ? "round_fold_base" : "round_fold_ext")
+                                   : (s.cur_base ? "round_base" : "round_ext");
     c.prof_begin(name, j, (uint64_t)T * 4 * (in_words + out_words));
   }
-  if (s.generated)
+  if (double_fold)
+    s.kernels->launch_fold2(&a, grid, c.stream);
+  else if (s.generated)
     s.kernels->launch(&a, s.cur_base, fold, grid, c.stream);
   else
     launch_interp<D>(a, s.desc, s.cur_base, fold, grid, c.stream);
@@ -404,6 +412,48 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
     hipLaunchKernelGGL(reduce_partials_kernel, dim3(width), dim3(BLOCK), 0, c.stream, s.d_partials, grid, s.pstride,
                        s.d_sums);
   }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+// Round 1 from the base tables (fold by challenge 0 pending, not performed): the slot sums in as many
+// launches as the generated kernels need, then their epilogue.
+template <int D>
+static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs, int j) {
+  Context &c = ctx();
+  NodesArgs<D> a;
+  memset(&a, 0, sizeof(a));
+  int T = s.st.T();
+  for (int t = 0; t < T; t++) a.in[t] = s.cur[t];
+  a.low = s.d_weights + s.low_off[j] * D;
+  a.high = s.d_weights + s.high_off[j] * D;
+  a.low_bits = (uint32_t)s.low_bits[j];
+  a.n_pairs = n_pairs;
+  uint32_t ppt = 1;
+  while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > s.max_grid) ppt *= 2;
+  a.pairs_per_thread = ppt;
+  a.deferred = (uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits) ? 1 : 0;
+  a.partials = s.d_partials;
+  a.pstride = s.pstride;
+  uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
+  for (int pass = 0; pass < s.kernels->nodes_passes; pass++) {
+    c.prof_begin("round_nodes_base", j, (uint64_t)T * 16 * n_pairs);
+    s.kernels->launch_nodes(&a, pass, grid, c.stream);
+    c.prof_end();
+  }
+  NodesEpilogueArgs e;
+  memset(&e, 0, sizeof(e));
+  e.e.partials = s.d_partials, e.e.nblocks = grid, e.e.pstride = s.pstride, e.e.nacc = (uint32_t)s.st.nacc;
+  e.e.points = (uint32_t)s.points, e.e.mtilde = s.d_mtilde, e.e.c0 = s.d_c0 + (size_t)j * s.points * D;
+  e.e.ctrl = s.d_ctrl;
+  e.groups = (uint32_t)s.desc.G, e.slots = (uint32_t)s.node_slots_n;
+  for (int g = 0; g < s.desc.G; g++) e.deg[g] = (uint32_t)s.desc.deg[g], e.nev[g] = (uint32_t)s.desc.nev[g];
+  c.prof_begin("epilogue", j, 0);
+  if (D == 4)
+    hipLaunchKernelGGL(nodes_epilogue_kernel<4>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
+  else
+    hipLaunchKernelGGL(nodes_epilogue_kernel<8>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
+  c.prof_end();
   EXH_HIP(hipGetLastError());
   return OK;
 }
@@ -672,15 +722,35 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   device_loop = true;
   bool tail_done = false;
   int status = OK, j = 0;
-  bool fold_due = false;  // the tables still await the fold by the last challenge drawn
+  int folds_due = 0;  // folds by the last challenges drawn that the tables still await (2 after the base-field round 1)
+  const char *no_nodes = getenv("EXACTA_HIP_NO_BASE_ROUND1");
   for (; j < n && status == OK; j++) {
-    uint64_t n_pairs = (size / (fold_due ? 2 : 1)) / 2;  // pairs summed in round j (after the pending fold)
+    const bool fold_due = folds_due > 0;
+    uint64_t n_pairs = (size >> folds_due) / 2;  // pairs summed in round j (after the pending folds)
+    if (folds_due == 2) {  // round 2 after the base-field round 1: both folds at once, then the sums
+      round = j;
+      uint64_t out_size = size / 4;
+      Arena &dst = ((generation + 1) % 2 == 0) ? c.fold_a : c.fold_b;
+      out_buf.assign(T, nullptr);
+      for (int t = 0; t < T; t++) out_buf[t] = (uint32_t *)dst.ptr + (uint64_t)t * out_size * D;
+      status = D == 4 ? launch_round<4>(*this, true, true, out_buf, n_pairs, j, true)
+                      : launch_round<8>(*this, true, true, out_buf, n_pairs, j, true);
+      for (int t = 0; t < T; t++) cur[t] = out_buf[t];
+      cur_base = false;
+      size = out_size;
+      generation += 2;
+      folds_due = 1;
+      tail_done = false;
+      continue;
+    }
     if (n_pairs <= tail_pairs(T, D) && n - j <= MAXTAIL) break;
     round = j;
     // once every workgroup of a resident grid can hold its slice of the tables in LDS, the rounds down
     // to where one workgroup suffices run in one launch
     const bool pow2 = (size & (size - 1)) == 0;
-    const uint64_t slice_max = SLICE_LDS_BYTES / ((uint64_t)T * 2 * D * 4);
+    uint64_t slice_max = SLICE_LDS_BYTES / ((uint64_t)T * 2 * D * 4);
+    if (const char *cap = getenv("EXACTA_HIP_MAX_SLICE_PAIRS"))  // tests: keep more rounds on the streaming kernels
+      slice_max = std::min<uint64_t>(slice_max, strtoull(cap, nullptr, 10));
     const uint64_t grid_max = std::min<uint64_t>(256, c.compute_units > 0 ? c.compute_units : 1);
     if (pow2 && n_pairs > tail_pairs(T, D) && n_pairs <= slice_max * grid_max) {
       int count = 0;
@@ -691,11 +761,22 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       while (n_pairs / grid > slice_max && grid * 2 <= grid_max && grid * 2 <= left) grid *= 2;
       if (count > 0 && grid > 1 && n_pairs / grid <= slice_max) {
         status = launch_tail(j, count, (uint32_t)grid, fold_due);
-        fold_due = false;
+        folds_due = 0;
         tail_done = status == OK;  // the tables are contiguous in one arena, nothing pending
         j += count - 1;
         continue;
       }
+    }
+    // round 1 on base tables, when round 2 is a streaming round as well: its sums come from base-field
+    // products at the nodes of r0 and the tables are not folded until round 2 (both folds at once)
+    const bool nodes_round = j == 1 && cur_base && folds_due == 1 && n >= 3 && generated && kernels->nodes_passes > 0 &&
+                             node_slots_n <= MAXACC && pow2 && (n_pairs / 2) > slice_max * grid_max &&
+                             !(no_nodes && no_nodes[0] == '1');
+    if (nodes_round) {
+      status = D == 4 ? launch_nodes_round<4>(*this, n_pairs, j) : launch_nodes_round<8>(*this, n_pairs, j);
+      folds_due = 2;
+      tail_done = false;
+      continue;
     }
     if (!fold_due) {
       status = D == 4 ? launch_round<4>(*this, false, true, out_buf, n_pairs, j)
@@ -712,12 +793,12 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       size = out_size;
       generation++;
     }
-    fold_due = true;
+    folds_due = 1;
     tail_done = false;
   }
   if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
-    status = launch_tail(j, n - j, 1, fold_due);
-    fold_due = false;
+    status = launch_tail(j, n - j, 1, folds_due > 0);
+    folds_due = 0;
     tail_done = status == OK;
   }
   device_loop = false;
@@ -745,7 +826,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     memcpy(challenges + (size_t)r * D, rc->chal[r], (size_t)D * 4);
   }
   round = n;
-  pending_fold = fold_due;  // after a round kernel the last challenge's fold is still to do
+  pending_fold = folds_due > 0;  // after a round kernel the last challenge's fold is still to do
   if (pending_fold) memcpy(pending_r, rc->chal[n - 1], (size_t)D * 4);
   return OK;
 }

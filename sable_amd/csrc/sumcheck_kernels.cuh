@@ -55,6 +55,7 @@ struct RoundArgs {
   uint32_t r_mont[D];        // the fold challenge, times R (host-driven rounds)
   Ctrl *ctrl;                // device-driven rounds: the fold challenge is read from here (else null)
   uint32_t pstride;          // words per workgroup partial (a power of two >= nacc * D)
+  uint32_t double_fold;      // base tables, folded by challenges 0 and 1 at once (8 entries -> 2 per pair)
 };
 
 // The rounds below 2^18 pairs, with the tables resident in LDS: no global memory round trip separates a
@@ -267,14 +268,47 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
   return fadd(fadd(a, b), fadd(c, d));
 }
 
-// the pair (lo, hi) of every table at pair index i, folding first when FOLD
-template <int D, bool IN_BASE, bool FOLD, class V, class Desc>
+// eq((r0, r1), b) for b = 0..3 (bit 0 of b goes with r0), in Montgomery form: the weights that bind two
+// variables of a base table at once, entry <- sum_b e[b] * T[4 x + b] (BIND-PREFIX, src/sumcheck.lisp:496-510)
+template <int D>
+struct BindWeights {
+  Ext<D> e[4];
+};
+template <int D>
+__device__ __forceinline__ BindWeights<D> bind_weights(const Ext<D> &r0_mont, const Ext<D> &r1_mont) {
+  BindWeights<D> w;
+  w.e[3] = ext_mul_mont<D>(r0_mont, r1_mont);  // r0 r1 R
+  w.e[1] = ext_sub<D>(r0_mont, w.e[3]);        // r0 (1 - r1) R
+  w.e[2] = ext_sub<D>(r1_mont, w.e[3]);        // (1 - r0) r1 R
+  Ext<D> one = ext_lift<D>(R1);
+  w.e[0] = ext_add<D>(ext_sub<D>(ext_sub<D>(one, r0_mont), r1_mont), w.e[3]);
+  return w;
+}
+// sum_b e[b] * v[b], exact: four products per coordinate, one reduction
+template <int D>
+__device__ __forceinline__ Ext<D> bind4(const BindWeights<D> &w, uint32_t v0, uint32_t v1, uint32_t v2, uint32_t v3) {
+  Ext<D> o;
+#pragma unroll
+  for (int c = 0; c < D; c++)
+    o.c[c] = mont_reduce4((uint64_t)w.e[0].c[c] * v0 + (uint64_t)w.e[1].c[c] * v1 + (uint64_t)w.e[2].c[c] * v2 +
+                          (uint64_t)w.e[3].c[c] * v3);
+  return o;
+}
+
+// the pair (lo, hi) of every table at pair index i, folding first when FOLD (FOLD2: base tables folded
+// twice at once by the bind weights)
+template <int D, bool IN_BASE, bool FOLD, class V, class Desc, bool FOLD2 = false>
 __device__ __forceinline__ void load_pair(const Desc &d, const uint32_t *const *in, uint32_t *const *out, uint64_t i,
-                                          const Ext<D> &r, V *lo, V *hi) {
+                                          const Ext<D> &r, V *lo, V *hi, const BindWeights<D> *bw = nullptr) {
 #pragma unroll
   for (int t = 0; t < MAXT; t++) {
     if (t < d.T) {
-      if constexpr (FOLD && IN_BASE) {
+      if constexpr (FOLD2) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(in[t] + 8 * i);
+        uint4 e = p[0], f = p[1];
+        lo[t] = bind4<D>(*bw, e.x, e.y, e.z, e.w);
+        hi[t] = bind4<D>(*bw, f.x, f.y, f.z, f.w);
+      } else if constexpr (FOLD && IN_BASE) {
         uint4 e = *reinterpret_cast<const uint4 *>(in[t] + 4 * i);
         lo[t] = fold_base<D>(e.x, e.y, r);
         hi[t] = fold_base<D>(e.z, e.w, r);
@@ -490,10 +524,10 @@ struct RoundShape {
   bool deferred, do_sums;
 };
 
-template <int D, bool IN_BASE, bool FOLD, class Desc>
+template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false>
 __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const *in, uint32_t *const *out,
                                            const RoundShape<D> &sh, const Ext<D> &r, uint32_t block,
-                                           uint32_t *partial_row) {
+                                           uint32_t *partial_row, const BindWeights<D> *bw = nullptr) {
   constexpr bool BASE_MODE = IN_BASE && !FOLD;  // the pair's values are base-field
   using V = typename std::conditional<BASE_MODE, uint32_t, Ext<D>>::type;
   const uint32_t tid = threadIdx.x;
@@ -511,7 +545,7 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
     const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
     if (i >= sh.n_pairs) break;
     V lo[MAXT], hi[MAXT];
-    load_pair<D, IN_BASE, FOLD, V>(d, in, out, i, r, lo, hi);
+    load_pair<D, IN_BASE, FOLD, V, Desc, FOLD2>(d, in, out, i, r, lo, hi, bw);
     if (sh.do_sums) {
       Ext<D> w = load_ext<D>(sh.low + (i & low_mask) * D);
       if (!sh.deferred) w = ext_mul_mont<D>(w, load_ext<D>(sh.high + (i >> sh.low_bits) * D));
@@ -532,9 +566,20 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
   }
 }
 
-template <int D, bool IN_BASE, bool FOLD, class Desc>
+template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false>
 __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &args) {
   Ext<D> r = ext_zero<D>();
+  if constexpr (FOLD2) {  // challenge 0 from the log, challenge 1 is the latest
+    Ext<D> r0, r1;
+#pragma unroll
+    for (int c = 0; c < D; c++) r0.c[c] = to_mont(args.ctrl->chal[0][c]), r1.c[c] = args.ctrl->r_mont[c];
+    BindWeights<D> bw = bind_weights<D>(r0, r1);
+    RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
+                     args.do_sums != 0};
+    round_core<D, true, true, Desc, true>(d, args.in, args.out, sh, r, blockIdx.x,
+                                          args.partials + (uint64_t)blockIdx.x * args.pstride, &bw);
+    return;
+  }
   if constexpr (FOLD) {
     const uint32_t *rp = args.ctrl ? args.ctrl->r_mont : args.r_mont;
 #pragma unroll
@@ -769,6 +814,219 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   }
 }
 
+// ---- round 1 from the base tables.  After round 0 the tables are still base-field and the fold by
+// challenge r0 is pending.  A folded value at X is u(X) + r0 v(X) with base-field u, v (the four base
+// entries of the pair give the two lines), so a group of degree d at X is a polynomial of degree d in r0
+// with base-field coefficients: the kernel sums, weighted, its values at the nodes r0 = 0..d ("slots":
+// group, point, node), all in base-field products, and the round's epilogue interpolates at the real r0.
+// Neither the folded tables are written nor extension products taken; the next round folds twice.
+// A launch covers the slots [PASS * SPP, (PASS + 1) * SPP) so the accumulators stay in registers.
+template <int D>
+struct NodesArgs {
+  const uint32_t *in[MAXT];  // base tables
+  const uint32_t *low, *high;
+  uint32_t *partials;        // [gridDim.x][pstride]: slot s at word s * D
+  uint64_t n_pairs;          // pairs of round 1: four base entries each
+  uint32_t low_bits, pairs_per_thread, deferred, pstride;
+};
+
+template <class Desc>
+__host__ __device__ constexpr int node_slots(const Desc &d) {
+  int n = 0;
+  for (int g = 0; g < d.G; g++) n += d.nev[g] * (d.deg[g] + 1);
+  return n;
+}
+
+template <int D, int PASS, int SPP, class Desc>
+__device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &args) {
+  const uint32_t tid = threadIdx.x;
+  const uint64_t tile = (uint64_t)BLOCK * args.pairs_per_thread, tile_start = (uint64_t)blockIdx.x * tile;
+  const uint64_t low_mask = ((uint64_t)1 << args.low_bits) - 1;
+  Acc96 acc[SPP][D];
+#pragma unroll
+  for (int a = 0; a < SPP; a++)
+#pragma unroll
+    for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
+
+  for (uint32_t k = 0; k < args.pairs_per_thread; k++) {
+    const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
+    if (i >= args.n_pairs) break;
+    // per factor: the line in r0 at X = 0 (u0 + r0 v0) and at X = 1 (u1 + r0 v1)
+    uint32_t cu[MAXT], cv[MAXT], du[MAXT], dv[MAXT], u1[MAXT], v1[MAXT];
+#pragma unroll
+    for (int t = 0; t < MAXT; t++)
+      if (t < d.T) {
+        uint4 e = *reinterpret_cast<const uint4 *>(args.in[t] + 4 * i);
+        cu[t] = e.x, cv[t] = fsub(e.y, e.x), u1[t] = e.z, v1[t] = fsub(e.w, e.z);
+      }
+#pragma unroll
+    for (int v = 0; v < MAXV; v++)
+      if (v < d.NV) {  // a linear form of the tables: the same combination of the lines
+        uint32_t a0 = 0, b0 = 0, a1 = 0, b1 = 0;
+#pragma unroll
+        for (int q = 0; q < MAXVT; q++)
+          if (q < d.vn[v]) {
+            const int t = d.vtab[v][q];
+            a0 = fadd(a0, v_scale<D>(cu[t], d.vcoef[v][q], d.vcoefm[v][q]));
+            b0 = fadd(b0, v_scale<D>(cv[t], d.vcoef[v][q], d.vcoefm[v][q]));
+            a1 = fadd(a1, v_scale<D>(u1[t], d.vcoef[v][q], d.vcoefm[v][q]));
+            b1 = fadd(b1, v_scale<D>(v1[t], d.vcoef[v][q], d.vcoefm[v][q]));
+          }
+        cu[d.T + v] = fadd(a0, d.vconst[v]), cv[d.T + v] = b0;
+        u1[d.T + v] = fadd(a1, d.vconst[v]), v1[d.T + v] = b1;
+      }
+#pragma unroll
+    for (int t = 0; t < MAXT; t++)
+      if (t < d.T + d.NV) du[t] = fsub(u1[t], cu[t]), dv[t] = fsub(v1[t], cv[t]);
+    Ext<D> w = load_ext<D>(args.low + (i & low_mask) * D);
+    if (!args.deferred) w = ext_mul_mont<D>(w, load_ext<D>(args.high + (i >> args.low_bits) * D));
+
+    int slot = 0;  // numbered group by group, point by point, node by node -- but visited point-major
+#pragma unroll
+    for (int x = 0; x <= MAXX; x++) {
+      if (x <= d.maxx) {
+        if (x >= 1) {
+#pragma unroll
+          for (int t = 0; t < MAXT; t++)
+            if (t < d.T + d.NV) {
+              if (x == 1)
+                cu[t] = u1[t], cv[t] = v1[t];
+              else
+                cu[t] = fadd(cu[t], du[t]), cv[t] = fadd(cv[t], dv[t]);
+            }
+        }
+        int base = 0;  // first slot of group g
+#pragma unroll
+        for (int g = 0; g < MAXG; g++) {
+          if (g < d.G) {
+#pragma unroll
+            for (int e = 0; e < MAXEV; e++) {
+              if (e < d.nev[g] && d.ev[g][e] == x) {
+                uint32_t val[MAXDEG];
+#pragma unroll
+                for (int j = 0; j < MAXDEG; j++)
+                  if (j < d.deg[g]) val[j] = cu[d.tab[g][j]];
+#pragma unroll
+                for (int m = 0; m <= MAXDEG; m++) {
+                  if (m <= d.deg[g]) {
+                    slot = base + e * (d.deg[g] + 1) + m;
+                    if (slot >= PASS * SPP && slot < (PASS + 1) * SPP) {
+                      uint32_t prod = val[0];
+#pragma unroll
+                      for (int j = 1; j < MAXDEG; j++)
+                        if (j < d.deg[g]) prod = mont_mul(prod, val[j]);
+                      ext_scale_acc<D>(acc[slot - PASS * SPP], w, prod);
+                    }
+#pragma unroll
+                    for (int j = 0; j < MAXDEG; j++)
+                      if (j < d.deg[g]) val[j] = fadd(val[j], cv[d.tab[g][j]]);
+                  }
+                }
+              }
+            }
+            base += d.nev[g] * (d.deg[g] + 1);
+          }
+        }
+      }
+    }
+    (void)slot;
+  }
+
+  // the workgroup's sums of this launch's slots, HIGH applied once when deferred
+  __shared__ uint32_t lds[BLOCK / 64][SPP * D];
+  const uint32_t lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+  for (int a = 0; a < SPP; a++)
+#pragma unroll
+    for (int c = 0; c < D; c++) {
+      uint32_t v = wave_sum(acc_reduce(acc[a][c]));
+      if (lane == 0) lds[wave][a * D + c] = v;
+    }
+  __syncthreads();
+  const int total = node_slots(d);
+  if (tid < SPP && PASS * SPP + (int)tid < total) {
+    Ext<D> sum;
+#pragma unroll
+    for (int c = 0; c < D; c++) {
+      uint32_t v = lds[0][tid * D + c];
+#pragma unroll
+      for (int wv = 1; wv < BLOCK / 64; wv++) v = fadd(v, lds[wv][tid * D + c]);
+      sum.c[c] = v;
+    }
+    if (args.deferred) sum = ext_mul_mont<D>(sum, load_ext<D>(args.high + (tile_start >> args.low_bits) * D));
+    store_ext<D>(args.partials + (uint64_t)blockIdx.x * args.pstride + (PASS * SPP + tid) * D, sum);
+  }
+}
+
+// The epilogue of the base-field round 1: slot sums -> (interpolation at r0) -> the accumulator sums the
+// ordinary epilogue takes.  One workgroup; the statement's shape comes as run-time arrays.
+struct NodesEpilogueArgs {
+  EpilogueArgs e;
+  uint32_t groups, slots;
+  uint32_t deg[MAXG], nev[MAXG];
+};
+
+template <int D>
+__global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogueArgs args) {
+  __shared__ uint32_t scratch[EPI_BLOCK];
+  __shared__ uint32_t slot_sums[MAXACC * D];
+  __shared__ uint32_t sums[MAXACC * D];
+  __shared__ uint32_t basis[(MAXDEG + 1) * (MAXDEG + 1) * D];  // [deg][node]: Lagrange basis at r0, Montgomery form
+  __shared__ EpilogueLds epi;
+  const uint32_t tid = threadIdx.x, ps = args.e.pstride;
+  if (tid < sizeof(DevB3S) / 4) epi.state[tid] = reinterpret_cast<const uint32_t *>(&args.e.ctrl->tr)[tid];
+  if (tid == 64) epi.round = args.e.ctrl->round;
+  for (uint32_t u = tid; u < args.e.points * args.e.nacc * D; u += EPI_BLOCK) epi.mtilde[u] = args.e.mtilde[u];
+  for (uint32_t u = tid; u < args.e.points * D; u += EPI_BLOCK) epi.c0[u] = args.e.c0[u];
+  // the basis of nodes 0..deg at r0 = challenge 0: L_m = prod_{q != m} (r0 - q) / (m - q)
+  if (tid < (MAXDEG + 1) * (MAXDEG + 1)) {
+    const uint32_t deg = tid / (MAXDEG + 1), m = tid % (MAXDEG + 1);
+    if (deg >= 1 && m <= deg) {
+      Ext<D> r0, acc = ext_lift<D>(R1);  // 1 in Montgomery form
+#pragma unroll
+      for (int c = 0; c < D; c++) r0.c[c] = to_mont(args.e.ctrl->chal[0][c]);
+      uint32_t den = 1;
+      for (uint32_t q = 0; q <= deg; q++) {
+        if (q == m) continue;
+        Ext<D> f = r0;
+        f.c[0] = fsub(f.c[0], to_mont(q));  // (r0 - q) R
+        acc = ext_mul_mont<D>(acc, f);
+        den = fmul(den, m > q ? m - q : P - (q - m));
+      }
+      acc = ext_scale_mont<D>(acc, to_mont(finv(den)));
+#pragma unroll
+      for (int c = 0; c < D; c++) basis[tid * D + c] = acc.c[c];
+    }
+  }
+  sum_partials(args.e.partials, args.e.nblocks, ps, args.slots * D, scratch, slot_sums);
+  // accumulator (g, e) = sum over nodes of basis * slot
+  {
+    uint32_t a = 0, base = 0;
+    for (uint32_t g = 0; g < args.groups; g++) {
+      for (uint32_t e = 0; e < args.nev[g]; e++, a++) {
+        if (tid == a) {
+          const uint32_t deg = args.deg[g];
+          Ext<D> total = ext_zero<D>();
+          for (uint32_t m = 0; m <= deg; m++) {
+            Ext<D> sv, lb;
+#pragma unroll
+            for (int c = 0; c < D; c++) {
+              sv.c[c] = slot_sums[(base + e * (deg + 1) + m) * D + c];
+              lb.c[c] = basis[(deg * (MAXDEG + 1) + m) * D + c];
+            }
+            total = ext_add<D>(total, ext_mul_mont<D>(lb, sv));
+          }
+#pragma unroll
+          for (int c = 0; c < D; c++) sums[a * D + c] = total.c[c];
+        }
+      }
+      base += args.nev[g] * (args.deg[g] + 1);
+    }
+  }
+  __syncthreads();
+  round_epilogue<D>(args.e.ctrl, sums, args.e.nacc, args.e.points, epi.mtilde, epi.c0, &epi, true);
+}
+
 // a kernel generated for one statement: S::d is its descriptor, known at compile time
 template <int D, bool IN_BASE, bool FOLD, class S>
 __global__ __launch_bounds__(BLOCK) void round_kernel(RoundArgs<D> args) {
@@ -777,6 +1035,14 @@ __global__ __launch_bounds__(BLOCK) void round_kernel(RoundArgs<D> args) {
 template <int D, class S>
 __global__ __launch_bounds__(BLOCK) void tail_kernel(TailArgs<D> args) {
   tail_body<D>(S::d, args);
+}
+template <int D, class S>
+__global__ __launch_bounds__(BLOCK) void round_kernel_fold2(RoundArgs<D> args) {
+  round_body<D, true, true, decltype(S::d), true>(S::d, args);
+}
+template <int D, class S, int PASS, int SPP>
+__global__ __launch_bounds__(BLOCK) void nodes_kernel(NodesArgs<D> args) {
+  nodes_body<D, PASS, SPP>(S::d, args);
 }
 
 // the interpreter: the same bodies over a run-time descriptor

@@ -256,3 +256,35 @@ def test_rounds_on_a_grid_of_lds_resident_slices(form, names, cnames, d, base, w
     eq = rand_ext(rng, (n,), d) if with_eq else None
     consts = rand_ext(rng, (len(cnames),), d) if cnames else None
     prove_both("slices", d, n, form, names, tables, eq=eq, constants=consts, cnames=cnames)
+
+
+@pytest.mark.parametrize("form,names,cnames,d,n", [
+    (CONFIG2, ["t0", "t1", "t2"], ["alpha"], 4, 3),
+    (CONFIG2, ["t0", "t1", "t2"], ["alpha"], 4, 9),
+    (CONFIG2, ["t0", "t1", "t2"], ["alpha"], 4, 14),
+    (CONFIG3, ["c0", "c1", "c2", "c3"], [], 8, 4),
+    (CONFIG3, ["c0", "c1", "c2", "c3"], [], 8, 11),
+    ("(* t0 t1)", ["t0", "t1"], [], 4, 12),
+    ("(* t0 t1)", ["t0", "t1"], [], 8, 7),
+    ("(* t0 t1 t2)", ["t0", "t1", "t2"], [], 8, 10),
+])
+def test_round_one_in_the_base_field_and_the_double_fold(form, names, cnames, d, n, monkeypatch):
+    """With base tables and streaming rounds 1 and 2 (forced here at small n; the headline sizes take this path
+    by themselves) round 1 is summed from base-field products at the nodes of r0 and round 2 folds twice at
+    once: same proof bytes, finals and folded tables as the oracle."""
+    monkeypatch.setenv("EXACTA_HIP_MAX_SLICE_PAIRS", "0")
+    rng = np.random.default_rng(n * 10 + d)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in names]
+    eq = rand_ext(rng, (n,), d)
+    consts = rand_ext(rng, (len(cnames),), d) if cnames else None
+    st, _, proof, _ = prove_both("nodes", d, n, form, names, tables, eq=eq, constants=consts, cnames=cnames)
+    assert st.has_generated_kernel(d)
+    # and without the eq weights
+    prove_both("nodes", d, n, form, names, tables, constants=consts, cnames=cnames)
+    monkeypatch.setenv("EXACTA_HIP_NO_BASE_ROUND1", "1")
+    tr = sa.Transcript("nodes", d)
+    dev = [sa.Table.upload(t) for t in tables]
+    sa.prove(tr, n, st, dev, eq=eq, constants=consts)
+    assert tr.proof() == proof
+    for t in dev:
+        t.free()
