@@ -448,6 +448,13 @@ static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs, int j) {
   e.e.ctrl = s.d_ctrl;
   e.groups = (uint32_t)s.desc.G, e.slots = (uint32_t)s.node_slots_n;
   for (int g = 0; g < s.desc.G; g++) e.deg[g] = (uint32_t)s.desc.deg[g], e.nev[g] = (uint32_t)s.desc.nev[g];
+  for (int deg = 1; deg <= MAXDEG; deg++)
+    for (int m = 0; m <= deg; m++) {
+      uint32_t den = 1;
+      for (int q = 0; q <= deg; q++)
+        if (q != m) den = fmul(den, m > q ? (uint32_t)(m - q) : P - (uint32_t)(q - m));
+      e.inv_den[deg * (MAXDEG + 1) + m] = to_mont(finv(den));
+    }
   c.prof_begin("epilogue", j, 0);
   if (D == 4)
     hipLaunchKernelGGL(nodes_epilogue_kernel<4>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);

@@ -964,6 +964,7 @@ struct NodesEpilogueArgs {
   EpilogueArgs e;
   uint32_t groups, slots;
   uint32_t deg[MAXG], nev[MAXG];
+  uint32_t inv_den[(MAXDEG + 1) * (MAXDEG + 1)];  // [deg][m]: 1 / prod_{q != m, q <= deg} (m - q), Montgomery form
 };
 
 template <int D>
@@ -985,15 +986,13 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
       Ext<D> r0, acc = ext_lift<D>(R1);  // 1 in Montgomery form
 #pragma unroll
       for (int c = 0; c < D; c++) r0.c[c] = to_mont(args.e.ctrl->chal[0][c]);
-      uint32_t den = 1;
       for (uint32_t q = 0; q <= deg; q++) {
         if (q == m) continue;
         Ext<D> f = r0;
         f.c[0] = fsub(f.c[0], to_mont(q));  // (r0 - q) R
         acc = ext_mul_mont<D>(acc, f);
-        den = fmul(den, m > q ? m - q : P - (q - m));
       }
-      acc = ext_scale_mont<D>(acc, to_mont(finv(den)));
+      acc = ext_scale_mont<D>(acc, args.inv_den[tid]);
 #pragma unroll
       for (int c = 0; c < D; c++) basis[tid * D + c] = acc.c[c];
     }
