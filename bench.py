@@ -53,20 +53,30 @@ def profile_entries(sa):
     return out
 
 
-def cpu_baseline(n_sample, d, seed):
+def cpu_baseline(sa, n_sample, d, seed):
     """The CPU oracle (a C restatement of the reference's prover, single thread) on the same statement and
-    seeds at a smaller n, sized for roughly 10-30 s."""
+    seeds at a smaller n, sized for roughly 10-30 s.  The same sample then goes through the GPU path as the
+    checker of this run: the proof bytes must be the oracle's."""
     from oracle import binding as orc
     st = orc.Statement(FORM, TABLES, CONSTS)
     tables = [splitmix_field(seed * 1000 + k, 1 << n_sample) for k in range(3)]
     eq = splitmix_field(seed + 900, n_sample * d).reshape(n_sample, d)
     alpha = splitmix_field(seed + 901, d).reshape(1, d)
     t0 = time.perf_counter()
-    orc.prove(orc.Transcript("config2", d), n_sample, st, tables, eq=eq, constants=alpha)
+    otr = orc.Transcript("config2", d)
+    orc.prove(otr, n_sample, st, tables, eq=eq, constants=alpha)
     dt = time.perf_counter() - t0
+    dev = [sa.Table.upload(t) for t in tables]
+    tr = sa.Transcript("config2", d)
+    sa.prove(tr, n_sample, sa.Statement(FORM, TABLES, CONSTS), dev, eq=eq, constants=alpha)
+    for t in dev:
+        t.free()
+    if tr.proof() != otr.proof():
+        sys.exit(f"bench.py: the GPU proof at n={n_sample} differs from the CPU oracle's")
     return {"value": 3 * (1 << n_sample) / dt, "unit": "table entries/s", "cores": 1, "kind": "port",
             "sample": f"same statement, seeds and transcript at n={n_sample} (3*2^{n_sample} entries, "
-                      f"{dt:.1f} s); the reference's Lisp prover cannot run here (no SBCL)"}
+                      f"{dt:.1f} s); the GPU proof of the same sample is byte-identical; the reference's Lisp "
+                      f"prover cannot run here (no SBCL)"}
 
 
 def run_sumcheck_config(sa, name, form, tables, consts, n, d, seed, steps, warmup, cpu_n):
@@ -358,7 +368,7 @@ def main():
                      "longest_launch": {"kernel": f"{tname} (round {tround})", "avg_launch_ms": ttotal / tcalls,
                                         "note": "LDS-resident rounds are latency-bound" if not tname.startswith("round_") else ""}},
     }
-    result["cpu_baseline"] = cpu_baseline(args.cpu_n, d, seed) if args.cpu_n > 0 else None
+    result["cpu_baseline"] = cpu_baseline(sa, args.cpu_n, d, seed) if args.cpu_n > 0 else None
     print(json.dumps(result))
 
 
