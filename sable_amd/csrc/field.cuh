@@ -196,11 +196,37 @@ EXH_HD void ext_mul_acc(Acc96 *acc, const Ext<D> &a, const Ext<D> &b) {
   ext_mul_sums<D>(a, b, [&](int e, int, uint64_t t) { acc_add(acc[e], t); });
 }
 // acc += a * s for a base value s
+#if defined(__HIP_DEVICE_COMPILE__)
+// Four accumulators at once: the multiply-add's own carry-out feeds the add to the third word, two
+// instructions per accumulator (written in C++ the carry is recomputed by a 64-bit add and a compare: four).
+// The carries go through four scalar pairs so that three other instructions separate each write from its read.
+__device__ __forceinline__ void acc_mad4(Acc96 *acc, const uint32_t *a, uint32_t s) {
+  uint64_t c0, c1, c2, c3;
+  asm("v_mad_u64_u32 %0, %8, %12, %16, %0\n\t"
+      "v_mad_u64_u32 %1, %9, %13, %16, %1\n\t"
+      "v_mad_u64_u32 %2, %10, %14, %16, %2\n\t"
+      "v_mad_u64_u32 %3, %11, %15, %16, %3\n\t"
+      "v_addc_co_u32_e64 %4, %8, 0, %4, %8\n\t"
+      "v_addc_co_u32_e64 %5, %9, 0, %5, %9\n\t"
+      "v_addc_co_u32_e64 %6, %10, 0, %6, %10\n\t"
+      "v_addc_co_u32_e64 %7, %11, 0, %7, %11"
+      : "+v"(acc[0].lo), "+v"(acc[1].lo), "+v"(acc[2].lo), "+v"(acc[3].lo), "+v"(acc[0].hi), "+v"(acc[1].hi),
+        "+v"(acc[2].hi), "+v"(acc[3].hi), "=&s"(c0), "=&s"(c1), "=&s"(c2), "=&s"(c3)
+      : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(s));
+}
+template <int D>
+__device__ __forceinline__ void ext_scale_acc(Acc96 *acc, const Ext<D> &a, uint32_t s) {
+  static_assert(D % 4 == 0, "accumulators go four at a time");
+#pragma unroll
+  for (int i = 0; i < D; i += 4) acc_mad4(acc + i, a.c + i, s);
+}
+#else
 template <int D>
 EXH_HD void ext_scale_acc(Acc96 *acc, const Ext<D> &a, uint32_t s) {
 #pragma unroll
   for (int i = 0; i < D; i++) acc_mad(acc[i], a.c[i], s);
 }
+#endif
 template <int D>
 EXH_HD Ext<D> acc_reduce_ext(const Acc96 *acc) {
   Ext<D> o;

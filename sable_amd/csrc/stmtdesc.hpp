@@ -30,4 +30,31 @@ struct StmtDesc {
   unsigned vconst[MAXV];
 };
 
+#if defined(__HIPCC__)
+#define EXH_DESC_FN __host__ __device__
+#else
+#define EXH_DESC_FN
+#endif
+
+// ---- the slots of the base-field sweep that serves rounds 0 and 1 (the kernels and their generator agree here)
+// the index of X among group g's evaluation points, or -1
+template <class Desc>
+EXH_DESC_FN constexpr int ev_index(const Desc &d, int g, int x) {
+  int at = -1;
+  for (int e = 0; e < MAXEV; e++)
+    if (e < d.nev[g] && d.ev[g][e] == x) at = e;
+  return at;
+}
+// per group: nev * (deg + 1) slots of round 1, then nev extras unless X = 1 is an evaluation point anyway
+template <class Desc>
+EXH_DESC_FN constexpr int group_slots(const Desc &d, int g) {
+  return d.nev[g] * (d.deg[g] + 1) + (ev_index(d, g, 1) < 0 ? d.nev[g] : 0);
+}
+template <class Desc>
+EXH_DESC_FN constexpr int node_slots(const Desc &d) {
+  int n = 0;
+  for (int g = 0; g < d.G; g++) n += group_slots(d, g);
+  return n;
+}
+
 }  // namespace exh

@@ -236,8 +236,7 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   uint64_t pairs0 = size / 2;
   max_grid = pairs0 ? (pairs0 + BLOCK - 1) / BLOCK : 1;
   if (max_grid > 1024) max_grid = 1024;
-  node_slots_n = 0;  // slots of the base-field round 1 (group, point, node)
-  for (int g = 0; g < desc.G; g++) node_slots_n += desc.nev[g] * (desc.deg[g] + 1);
+  node_slots_n = node_slots(desc);  // grid sums of the sweep that serves rounds 0 and 1 from the base tables
   pstride = next_pow2((uint64_t)std::max(std::max(st.nacc, 1), node_slots_n <= MAXACC ? node_slots_n : 0) * D);
   uint64_t partial_off = pos * D;  // from here in words
   // (a grid of LDS-resident slices keeps 64-bit totals per round and group in the same place)
@@ -419,35 +418,42 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
 // Round 1 from the base tables (fold by challenge 0 pending, not performed): the slot sums in as many
 // launches as the generated kernels need, then their epilogue.
 template <int D>
-static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs, int j) {
+static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs) {
   Context &c = ctx();
   NodesArgs<D> a;
   memset(&a, 0, sizeof(a));
   int T = s.st.T();
   for (int t = 0; t < T; t++) a.in[t] = s.cur[t];
-  a.low = s.d_weights + s.low_off[j] * D;
-  a.high = s.d_weights + s.high_off[j] * D;
-  a.low_bits = (uint32_t)s.low_bits[j];
+  a.low = s.d_weights + s.low_off[1] * D;  // round 1's weights; round 0's extra factor goes in by the epilogue
+  a.high = s.d_weights + s.high_off[1] * D;
+  a.low_bits = (uint32_t)s.low_bits[1];
   a.n_pairs = n_pairs;
+  // two workgroups fit a compute unit beside the accumulators: a grid of that many, all resident at once,
+  // spreads each workgroup's fixed work (first loads, the reduction over lanes) over the most pairs
+  const uint64_t want_grid = std::min<uint64_t>(s.max_grid, 2 * (uint64_t)std::max(ctx().compute_units, 1));
   uint32_t ppt = 1;
-  while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > s.max_grid) ppt *= 2;
+  while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > want_grid) ppt *= 2;
   a.pairs_per_thread = ppt;
   a.deferred = (uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits) ? 1 : 0;
   a.partials = s.d_partials;
   a.pstride = s.pstride;
   uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
   for (int pass = 0; pass < s.kernels->nodes_passes; pass++) {
-    c.prof_begin("round_nodes_base", j, (uint64_t)T * 16 * n_pairs);
+    c.prof_begin("round_nodes_base", 0, (uint64_t)T * 16 * n_pairs);
     s.kernels->launch_nodes(&a, pass, grid, c.stream);
     c.prof_end();
   }
   NodesEpilogueArgs e;
   memset(&e, 0, sizeof(e));
   e.e.partials = s.d_partials, e.e.nblocks = grid, e.e.pstride = s.pstride, e.e.nacc = (uint32_t)s.st.nacc;
-  e.e.points = (uint32_t)s.points, e.e.mtilde = s.d_mtilde, e.e.c0 = s.d_c0 + (size_t)j * s.points * D;
+  e.e.points = (uint32_t)s.points, e.e.mtilde = s.d_mtilde, e.e.c0 = s.d_c0;
   e.e.ctrl = s.d_ctrl;
+  e.eq1 = s.has_eq ? s.d_weights + (size_t)2 * D : nullptr;  // the eq factors lead the arena: (w_v, 1 - w_v) per variable
   e.groups = (uint32_t)s.desc.G, e.slots = (uint32_t)s.node_slots_n;
-  for (int g = 0; g < s.desc.G; g++) e.deg[g] = (uint32_t)s.desc.deg[g], e.nev[g] = (uint32_t)s.desc.nev[g];
+  for (int g = 0; g < s.desc.G; g++) {
+    e.deg[g] = (uint32_t)s.desc.deg[g], e.nev[g] = (uint32_t)s.desc.nev[g];
+    for (int k = 0; k < s.desc.nev[g]; k++) e.ev[g][k] = (uint8_t)s.desc.ev[g][k];
+  }
   for (int deg = 1; deg <= MAXDEG; deg++)
     for (int m = 0; m <= deg; m++) {
       uint32_t den = 1;
@@ -455,7 +461,7 @@ static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs, int j) {
         if (q != m) den = fmul(den, m > q ? (uint32_t)(m - q) : P - (uint32_t)(q - m));
       e.inv_den[deg * (MAXDEG + 1) + m] = to_mont(finv(den));
     }
-  c.prof_begin("epilogue", j, 0);
+  c.prof_begin("epilogue", 0, 0);
   if (D == 4)
     hipLaunchKernelGGL(nodes_epilogue_kernel<4>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
   else
@@ -774,15 +780,16 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
         continue;
       }
     }
-    // round 1 on base tables, when round 2 is a streaming round as well: its sums come from base-field
-    // products at the nodes of r0 and the tables are not folded until round 2 (both folds at once)
-    const bool nodes_round = j == 1 && cur_base && folds_due == 1 && n >= 3 && generated && kernels->nodes_passes > 0 &&
-                             node_slots_n <= MAXACC && pow2 && (n_pairs / 2) > slice_max * grid_max &&
-                             !(no_nodes && no_nodes[0] == '1');
-    if (nodes_round) {
-      status = D == 4 ? launch_nodes_round<4>(*this, n_pairs, j) : launch_nodes_round<8>(*this, n_pairs, j);
+    // rounds 0 and 1 from one sweep of the base tables, when round 2 is a streaming round as well: their sums
+    // come from base-field products on a grid of (X0, X1) and the tables are not folded until round 2
+    const bool nodes_rounds = j == 0 && cur_base && folds_due == 0 && n >= 3 && generated && kernels->nodes_passes > 0 &&
+                              node_slots_n <= MAXACC && pow2 && (n_pairs / 4) > slice_max * grid_max &&
+                              !(no_nodes && no_nodes[0] == '1');
+    if (nodes_rounds) {
+      status = D == 4 ? launch_nodes_round<4>(*this, n_pairs / 2) : launch_nodes_round<8>(*this, n_pairs / 2);
       folds_due = 2;
       tail_done = false;
+      j++;  // two rounds done
       continue;
     }
     if (!fold_due) {

@@ -814,13 +814,17 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   }
 }
 
-// ---- round 1 from the base tables.  After round 0 the tables are still base-field and the fold by
-// challenge r0 is pending.  A folded value at X is u(X) + r0 v(X) with base-field u, v (the four base
-// entries of the pair give the two lines), so a group of degree d at X is a polynomial of degree d in r0
-// with base-field coefficients: the kernel sums, weighted, its values at the nodes r0 = 0..d ("slots":
-// group, point, node), all in base-field products, and the round's epilogue interpolates at the real r0.
-// Neither the folded tables are written nor extension products taken; the next round folds twice.
-// A launch covers the slots [PASS * SPP, (PASS + 1) * SPP) so the accumulators stay in registers.
+// ---- rounds 0 and 1 from one sweep of the base tables.  A pair of round 1 is four base entries per table:
+// the value at (X0, X1) is bilinear in them, u(X1) + X0 v(X1) with base-field u, v.  A group of degree d is
+// therefore a polynomial of degree d in X0 with base-field coefficients at every X1, and the kernel sums,
+// weighted by round 1's weights, its values on a grid ("slots"):
+//   (point e, node m):  X1 = the group's e-th evaluation point, X0 = m in 0..d     -- round 1, whose epilogue
+//                       interpolates in X0 at the challenge r0,
+//   (extra e):          X1 = 1, X0 = the e-th evaluation point                     -- round 0: its sum at X0 is
+//                       eq(w1, 0) * slot(X1 = 0, X0) + eq(w1, 1) * slot(X1 = 1, X0), the weight of variable 1
+//                       being the one factor round 0's weights have beyond round 1's.
+// All products are base-field; no folded table is written; round 2 folds twice.  A launch covers the slots
+// [PASS * SPP, (PASS + 1) * SPP) so the accumulators stay in registers.
 template <int D>
 struct NodesArgs {
   const uint32_t *in[MAXT];  // base tables
@@ -830,61 +834,109 @@ struct NodesArgs {
   uint32_t low_bits, pairs_per_thread, deferred, pstride;
 };
 
-template <class Desc>
-__host__ __device__ constexpr int node_slots(const Desc &d) {
-  int n = 0;
-  for (int g = 0; g < d.G; g++) n += d.nev[g] * (d.deg[g] + 1);
-  return n;
+// ---- KoalaBear in double precision, for the products of base-field values that are sums and differences of
+// table entries: integers below 2^53 are exact there, so the lines' values need no reduction between additions
+// (three integer operations each otherwise) and a product mod p takes six operations, as a Montgomery product
+// with its final correction does.  Every step below is exact integer arithmetic: a product a b is held as the pair (h, l) of its rounded value and the rounding error, the
+// quotient estimate q = rint(h / p) is off by far less than one, and h - q p + l is then a small integer.
+constexpr double F_P = 2130706433.0, F_PINV = 1.0 / 2130706433.0, F_MAGIC = 6755399441055744.0;  // 1.5 * 2^52
+// v mod p in about [-p/2, p/2] for an integer |v| < 2^80
+__device__ __forceinline__ double f_reduce(double v) {
+  double q = __builtin_fma(v, F_PINV, F_MAGIC) - F_MAGIC;  // rint(v / p) for |v / p| < 2^51
+  return __builtin_fma(-q, F_P, v);
+}
+// a b mod p in about [-p/2 - 2^27, p/2 + 2^27] for integers |a b| < 2^80
+__device__ __forceinline__ double f_mul(double a, double b) {
+  double h = a * b;
+  double l = __builtin_fma(a, b, -h);
+  double q = __builtin_fma(h, F_PINV, F_MAGIC) - F_MAGIC;
+  return __builtin_fma(-q, F_P, h) + l;
+}
+// c x for a table value x and a statement's integer coefficient c (a residue: large ones stand for negatives)
+__device__ __forceinline__ double f_scale(double x, uint32_t c) {
+  return c == 1 ? x : c == P - 1 ? -x : f_mul(x, c > P / 2 ? (double)c - F_P : (double)c);
+}
+// a residue of v below 2^32 as an integer, for |v| < p + 2^28: v + p sits in the low word of v + p + 1.5 * 2^52
+__device__ __forceinline__ uint32_t f_residue32(double v) {
+  return (uint32_t)__double_as_longlong(v + (F_P + F_MAGIC));
 }
 
+// the base-field slot sums as above, on the floating-point pipe
 template <int D, int PASS, int SPP, class Desc>
 __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &args) {
+  // magnitudes, in units of p: a table line's ends < 1, a linear form < 5 (MAXVT terms and the constant),
+  // the step between X points < 10, so at X <= 7 a line's end < 65 and its slope < 52, a node's value
+  // < 65 + 6 * 52 = 377; a product of two < 377^2 p^2 < 2^80 and its quotient by p < 2^49.
+  static_assert(MAXVT <= 4 && MAXX <= 7 && MAXDEG <= 6, "the bounds of the double-precision products");
   const uint32_t tid = threadIdx.x;
   const uint64_t tile = (uint64_t)BLOCK * args.pairs_per_thread, tile_start = (uint64_t)blockIdx.x * tile;
   const uint64_t low_mask = ((uint64_t)1 << args.low_bits) - 1;
+  // the weighted sums themselves are integer: one 32 x 32 -> 64 multiply-add per word into 96 bits (twelve
+  // registers a slot where two exact double sums would take sixteen); up to 2^32 terms below 2^63 fit
   Acc96 acc[SPP][D];
 #pragma unroll
   for (int a = 0; a < SPP; a++)
 #pragma unroll
     for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
 
+  // the loads run PREFETCH pairs ahead of the arithmetic: few waves fit beside 16 registers per slot
+  constexpr int PREFETCH = 2;
+  uint4 ahead[PREFETCH][MAXT];
+  Ext<D> wahead[PREFETCH];
+  auto fetch = [&](uint32_t k, uint4 *e, Ext<D> &w) {
+    const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
+    if (k < args.pairs_per_thread && i < args.n_pairs) {
+#pragma unroll
+      for (int t = 0; t < MAXT; t++)
+        if (t < d.T) e[t] = *reinterpret_cast<const uint4 *>(args.in[t] + 4 * i);
+      w = load_ext<D>(args.low + (i & low_mask) * D);
+    }
+  };
+#pragma unroll
+  for (int a = 0; a < PREFETCH; a++) fetch(a, ahead[a], wahead[a]);
+
   for (uint32_t k = 0; k < args.pairs_per_thread; k++) {
     const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
     if (i >= args.n_pairs) break;
     // per factor: the line in r0 at X = 0 (u0 + r0 v0) and at X = 1 (u1 + r0 v1)
-    uint32_t cu[MAXT], cv[MAXT], du[MAXT], dv[MAXT], u1[MAXT], v1[MAXT];
+    double cu[MAXT], cv[MAXT], du[MAXT], dv[MAXT], u1[MAXT], v1[MAXT];
 #pragma unroll
     for (int t = 0; t < MAXT; t++)
       if (t < d.T) {
-        uint4 e = *reinterpret_cast<const uint4 *>(args.in[t] + 4 * i);
-        cu[t] = e.x, cv[t] = fsub(e.y, e.x), u1[t] = e.z, v1[t] = fsub(e.w, e.z);
+        const uint4 e = ahead[0][t];
+        cu[t] = (double)e.x, cv[t] = (double)e.y - cu[t], u1[t] = (double)e.z, v1[t] = (double)e.w - u1[t];
       }
+    Ext<D> we = wahead[0];
+#pragma unroll
+    for (int a = 0; a + 1 < PREFETCH; a++) {
+#pragma unroll
+      for (int t = 0; t < MAXT; t++)
+        if (t < d.T) ahead[a][t] = ahead[a + 1][t];
+      wahead[a] = wahead[a + 1];
+    }
+    fetch(k + PREFETCH, ahead[PREFETCH - 1], wahead[PREFETCH - 1]);
 #pragma unroll
     for (int v = 0; v < MAXV; v++)
       if (v < d.NV) {  // a linear form of the tables: the same combination of the lines
-        uint32_t a0 = 0, b0 = 0, a1 = 0, b1 = 0;
+        double a0 = (double)d.vconst[v], b0 = 0, a1 = a0, b1 = 0;
 #pragma unroll
         for (int q = 0; q < MAXVT; q++)
           if (q < d.vn[v]) {
             const int t = d.vtab[v][q];
-            a0 = fadd(a0, v_scale<D>(cu[t], d.vcoef[v][q], d.vcoefm[v][q]));
-            b0 = fadd(b0, v_scale<D>(cv[t], d.vcoef[v][q], d.vcoefm[v][q]));
-            a1 = fadd(a1, v_scale<D>(u1[t], d.vcoef[v][q], d.vcoefm[v][q]));
-            b1 = fadd(b1, v_scale<D>(v1[t], d.vcoef[v][q], d.vcoefm[v][q]));
+            a0 += f_scale(cu[t], d.vcoef[v][q]), b0 += f_scale(cv[t], d.vcoef[v][q]);
+            a1 += f_scale(u1[t], d.vcoef[v][q]), b1 += f_scale(v1[t], d.vcoef[v][q]);
           }
-        cu[d.T + v] = fadd(a0, d.vconst[v]), cv[d.T + v] = b0;
-        u1[d.T + v] = fadd(a1, d.vconst[v]), v1[d.T + v] = b1;
+        cu[d.T + v] = a0, cv[d.T + v] = b0, u1[d.T + v] = a1, v1[d.T + v] = b1;
       }
 #pragma unroll
     for (int t = 0; t < MAXT; t++)
-      if (t < d.T + d.NV) du[t] = fsub(u1[t], cu[t]), dv[t] = fsub(v1[t], cv[t]);
-    Ext<D> w = load_ext<D>(args.low + (i & low_mask) * D);
-    if (!args.deferred) w = ext_mul_mont<D>(w, load_ext<D>(args.high + (i >> args.low_bits) * D));
+      if (t < d.T + d.NV) du[t] = u1[t] - cu[t], dv[t] = v1[t] - cv[t];
+    if (!args.deferred) we = ext_mul_mont<D>(we, load_ext<D>(args.high + (i >> args.low_bits) * D));
 
-    int slot = 0;  // numbered group by group, point by point, node by node -- but visited point-major
+    int slot = 0;  // numbered group by group (point by point, node by node, then the extras) -- visited X1-major
 #pragma unroll
     for (int x = 0; x <= MAXX; x++) {
-      if (x <= d.maxx) {
+      if (x <= d.maxx || x == 1) {
         if (x >= 1) {
 #pragma unroll
           for (int t = 0; t < MAXT; t++)
@@ -892,39 +944,41 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
               if (x == 1)
                 cu[t] = u1[t], cv[t] = v1[t];
               else
-                cu[t] = fadd(cu[t], du[t]), cv[t] = fadd(cv[t], dv[t]);
+                cu[t] += du[t], cv[t] += dv[t];
             }
         }
         int base = 0;  // first slot of group g
 #pragma unroll
         for (int g = 0; g < MAXG; g++) {
           if (g < d.G) {
+            const int e = ev_index(d, g, x);  // an evaluation point's row, or at X1 = 1 the row of extras
+            if (e >= 0 || x == 1) {
+              double val[MAXDEG];
 #pragma unroll
-            for (int e = 0; e < MAXEV; e++) {
-              if (e < d.nev[g] && d.ev[g][e] == x) {
-                uint32_t val[MAXDEG];
+              for (int j = 0; j < MAXDEG; j++)
+                if (j < d.deg[g]) val[j] = cu[d.tab[g][j]];
 #pragma unroll
-                for (int j = 0; j < MAXDEG; j++)
-                  if (j < d.deg[g]) val[j] = cu[d.tab[g][j]];
-#pragma unroll
-                for (int m = 0; m <= MAXDEG; m++) {
-                  if (m <= d.deg[g]) {
+              for (int m = 0; m <= MAXDEG; m++) {
+                if (m <= d.deg[g]) {
+                  if (e >= 0)
                     slot = base + e * (d.deg[g] + 1) + m;
-                    if (slot >= PASS * SPP && slot < (PASS + 1) * SPP) {
-                      uint32_t prod = val[0];
+                  else  // only the nodes that are evaluation points
+                    slot = ev_index(d, g, m) < 0 ? -1 : base + d.nev[g] * (d.deg[g] + 1) + ev_index(d, g, m);
+                  if (slot >= PASS * SPP && slot < (PASS + 1) * SPP) {
+                    double prod = val[0];
 #pragma unroll
-                      for (int j = 1; j < MAXDEG; j++)
-                        if (j < d.deg[g]) prod = mont_mul(prod, val[j]);
-                      ext_scale_acc<D>(acc[slot - PASS * SPP], w, prod);
-                    }
-#pragma unroll
-                    for (int j = 0; j < MAXDEG; j++)
-                      if (j < d.deg[g]) val[j] = fadd(val[j], cv[d.tab[g][j]]);
+                    for (int j = 1; j < MAXDEG; j++)
+                      if (j < d.deg[g]) prod = f_mul(prod, val[j]);
+                    if (d.deg[g] == 1) prod = f_reduce(prod);
+                    ext_scale_acc<D>(acc[slot - PASS * SPP], we, f_residue32(prod));
                   }
+#pragma unroll
+                  for (int j = 0; j < MAXDEG; j++)
+                    if (j < d.deg[g]) val[j] += cv[d.tab[g][j]];
                 }
               }
             }
-            base += d.nev[g] * (d.deg[g] + 1);
+            base += group_slots(d, g);
           }
         }
       }
@@ -933,37 +987,56 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
   }
 
   // the workgroup's sums of this launch's slots, HIGH applied once when deferred
-  __shared__ uint32_t lds[BLOCK / 64][SPP * D];
+  constexpr int WORDS = SPP * D, CHUNKS = (WORDS + 31) / 32;
+  __shared__ uint32_t lds[BLOCK / 64][CHUNKS * 32];
   const uint32_t lane = tid & 63, wave = tid >> 6;
+  {  // the wavefront's sums, 32 words at a time by the transposing reduction
+    uint32_t idx = 0;
 #pragma unroll
-  for (int a = 0; a < SPP; a++)
+    for (int b = 0; b < 5; b++) idx |= ((lane >> b) & 1u) << (4 - b);
 #pragma unroll
-    for (int c = 0; c < D; c++) {
-      uint32_t v = wave_sum(acc_reduce(acc[a][c]));
-      if (lane == 0) lds[wave][a * D + c] = v;
+    for (int first = 0; first < WORDS; first += 32) {
+      const uint32_t total = wave_sums_transposed<32>([&](int k) -> uint32_t {
+        const int o = first + k;
+        return o < WORDS ? acc_reduce(acc[o / D][o % D]) : 0u;
+      });
+      if (lane < 32) lds[wave][first + idx] = total;
     }
+  }
   __syncthreads();
   const int total = node_slots(d);
   if (tid < SPP && PASS * SPP + (int)tid < total) {
+    // The sums above are of w * (the plain product of the group's factors); the integer kernels' products
+    // carry 1/R per multiplication, which the epilogue's constants expect: times R^(1 - degree) here.
+    int base = 0, deg = 1;
+    for (int g = 0; g < d.G; g++) {
+      if (PASS * SPP + (int)tid >= base) deg = d.deg[g];
+      base += group_slots(d, g);
+    }
+    uint32_t fix = R1;  // mont_mul(v, fix) = v R^(1 - degree)
+    for (int q = 1; q < deg; q++) fix = mont_mul(fix, 1u);
     Ext<D> sum;
 #pragma unroll
     for (int c = 0; c < D; c++) {
       uint32_t v = lds[0][tid * D + c];
 #pragma unroll
       for (int wv = 1; wv < BLOCK / 64; wv++) v = fadd(v, lds[wv][tid * D + c]);
-      sum.c[c] = v;
+      sum.c[c] = mont_mul(v, fix);
     }
     if (args.deferred) sum = ext_mul_mont<D>(sum, load_ext<D>(args.high + (tile_start >> args.low_bits) * D));
     store_ext<D>(args.partials + (uint64_t)blockIdx.x * args.pstride + (PASS * SPP + tid) * D, sum);
   }
 }
 
-// The epilogue of the base-field round 1: slot sums -> (interpolation at r0) -> the accumulator sums the
-// ordinary epilogue takes.  One workgroup; the statement's shape comes as run-time arrays.
+// The epilogue of that sweep, both rounds in one workgroup: slot sums -> round 0's accumulator sums -> its
+// message, through the transcript, to r0 -> the Lagrange basis at r0 -> round 1's accumulator sums -> its
+// message and r1.  The statement's shape comes as run-time arrays.
 struct NodesEpilogueArgs {
-  EpilogueArgs e;
+  EpilogueArgs e;            // c0 points at round 0's rows, round 1's follow
+  const uint32_t *eq1;       // eq(w1, 1) and eq(w1, 0) as two elements, Montgomery form; null: both weights 1
   uint32_t groups, slots;
   uint32_t deg[MAXG], nev[MAXG];
+  uint8_t ev[MAXG][MAXEV];
   uint32_t inv_den[(MAXDEG + 1) * (MAXDEG + 1)];  // [deg][m]: 1 / prod_{q != m, q <= deg} (m - q), Montgomery form
 };
 
@@ -974,18 +1047,61 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
   __shared__ uint32_t sums[MAXACC * D];
   __shared__ uint32_t basis[(MAXDEG + 1) * (MAXDEG + 1) * D];  // [deg][node]: Lagrange basis at r0, Montgomery form
   __shared__ EpilogueLds epi;
-  const uint32_t tid = threadIdx.x, ps = args.e.pstride;
+  const uint32_t tid = threadIdx.x, ps = args.e.pstride, points = args.e.points, nacc = args.e.nacc;
   if (tid < sizeof(DevB3S) / 4) epi.state[tid] = reinterpret_cast<const uint32_t *>(&args.e.ctrl->tr)[tid];
-  if (tid == 64) epi.round = args.e.ctrl->round;
-  for (uint32_t u = tid; u < args.e.points * args.e.nacc * D; u += EPI_BLOCK) epi.mtilde[u] = args.e.mtilde[u];
-  for (uint32_t u = tid; u < args.e.points * D; u += EPI_BLOCK) epi.c0[u] = args.e.c0[u];
-  // the basis of nodes 0..deg at r0 = challenge 0: L_m = prod_{q != m} (r0 - q) / (m - q)
+  for (uint32_t u = tid; u < points * nacc * D; u += EPI_BLOCK) epi.mtilde[u] = args.e.mtilde[u];
+  for (uint32_t u = tid; u < points * D; u += EPI_BLOCK) epi.c0[u] = args.e.c0[u];
+  sum_partials(args.e.partials, args.e.nblocks, ps, args.slots * D, scratch, slot_sums);
+  auto slot = [&](uint32_t index) {
+    Ext<D> v;
+#pragma unroll
+    for (int c = 0; c < D; c++) v.c[c] = slot_sums[index * D + c];
+    return v;
+  };
+  auto row_of = [&](uint32_t g, uint32_t x) {  // the index of X among group g's points, or nev
+    uint32_t at = args.nev[g];
+    for (uint32_t e = 0; e < args.nev[g]; e++)
+      if (args.ev[g][e] == x) at = e;
+    return at;
+  };
+  // ---- round 0: accumulator (g, e) = eq(w1, 0) * slot(X1 = 0, node ev_e) + eq(w1, 1) * slot(X1 = 1, node ev_e)
+  {
+    uint32_t a = 0, base = 0;
+    for (uint32_t g = 0; g < args.groups; g++) {
+      const uint32_t deg = args.deg[g], nev = args.nev[g], row0 = row_of(g, 0), row1 = row_of(g, 1);
+      for (uint32_t e = 0; e < nev; e++, a++) {
+        if (tid == a) {
+          const uint32_t node = args.ev[g][e];
+          Ext<D> at0 = slot(base + row0 * (deg + 1) + node);
+          Ext<D> at1 = row1 < nev ? slot(base + row1 * (deg + 1) + node) : slot(base + nev * (deg + 1) + e);
+          if (args.eq1) {
+            at1 = ext_mul_mont<D>(at1, load_ext<D>(args.eq1));
+            at0 = ext_mul_mont<D>(at0, load_ext<D>(args.eq1 + D));
+          }
+          const Ext<D> total = ext_add<D>(at0, at1);
+#pragma unroll
+          for (int c = 0; c < D; c++) sums[a * D + c] = total.c[c];
+        }
+      }
+      base += nev * (deg + 1) + (row1 < nev ? 0 : nev);
+    }
+  }
+  __syncthreads();
+  round_message<D>(sums, nacc, points, epi.mtilde, epi.c0, &epi);
+  RunB3S tr;
+  if (tid < 64) {
+    rb3s_load(tr, epi.ring, reinterpret_cast<const DevB3S *>(epi.state));
+    transcript_step<D>(tr, args.e.ctrl, 0, points, &epi);
+  }
+  __syncthreads();
+  // ---- round 1: the basis of nodes 0..deg at r0, L_m = prod_{q != m} (r0 - q) / (m - q)
+  for (uint32_t u = tid; u < points * D; u += EPI_BLOCK) epi.c0[u] = args.e.c0[points * D + u];
   if (tid < (MAXDEG + 1) * (MAXDEG + 1)) {
     const uint32_t deg = tid / (MAXDEG + 1), m = tid % (MAXDEG + 1);
     if (deg >= 1 && m <= deg) {
       Ext<D> r0, acc = ext_lift<D>(R1);  // 1 in Montgomery form
 #pragma unroll
-      for (int c = 0; c < D; c++) r0.c[c] = to_mont(args.e.ctrl->chal[0][c]);
+      for (int c = 0; c < D; c++) r0.c[c] = epi.r_mont[c];
       for (uint32_t q = 0; q <= deg; q++) {
         if (q == m) continue;
         Ext<D> f = r0;
@@ -997,33 +1113,35 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
       for (int c = 0; c < D; c++) basis[tid * D + c] = acc.c[c];
     }
   }
-  sum_partials(args.e.partials, args.e.nblocks, ps, args.slots * D, scratch, slot_sums);
+  __syncthreads();
   // accumulator (g, e) = sum over nodes of basis * slot
   {
     uint32_t a = 0, base = 0;
     for (uint32_t g = 0; g < args.groups; g++) {
-      for (uint32_t e = 0; e < args.nev[g]; e++, a++) {
+      const uint32_t deg = args.deg[g], nev = args.nev[g];
+      for (uint32_t e = 0; e < nev; e++, a++) {
         if (tid == a) {
-          const uint32_t deg = args.deg[g];
           Ext<D> total = ext_zero<D>();
           for (uint32_t m = 0; m <= deg; m++) {
-            Ext<D> sv, lb;
+            Ext<D> lb;
 #pragma unroll
-            for (int c = 0; c < D; c++) {
-              sv.c[c] = slot_sums[(base + e * (deg + 1) + m) * D + c];
-              lb.c[c] = basis[(deg * (MAXDEG + 1) + m) * D + c];
-            }
-            total = ext_add<D>(total, ext_mul_mont<D>(lb, sv));
+            for (int c = 0; c < D; c++) lb.c[c] = basis[(deg * (MAXDEG + 1) + m) * D + c];
+            total = ext_add<D>(total, ext_mul_mont<D>(lb, slot(base + e * (deg + 1) + m)));
           }
 #pragma unroll
           for (int c = 0; c < D; c++) sums[a * D + c] = total.c[c];
         }
       }
-      base += args.nev[g] * (args.deg[g] + 1);
+      base += nev * (deg + 1) + (row_of(g, 1) < nev ? 0 : nev);
     }
   }
   __syncthreads();
-  round_epilogue<D>(args.e.ctrl, sums, args.e.nacc, args.e.points, epi.mtilde, epi.c0, &epi, true);
+  round_message<D>(sums, nacc, points, epi.mtilde, epi.c0, &epi);
+  if (tid < 64) {
+    transcript_step<D>(tr, args.e.ctrl, 1, points, &epi);
+    rb3s_store(tr, &args.e.ctrl->tr);
+    if (tid == 0) args.e.ctrl->round = 2;
+  }
 }
 
 // a kernel generated for one statement: S::d is its descriptor, known at compile time
