@@ -108,9 +108,10 @@ static int get_domain(int n, Domain **out) {
 // workgroup barrier are touched once per four stages.  LDS words are padded by one per 32 so that
 // the strided gathers fall on distinct banks.
 // A tile is 2^12 words, 16 per thread: a domain of 2^24 takes three passes (6 + 5 + 12 stages) with
-// global segments of at least 64 words.  The passes are bound by the butterflies' modular multiplies
-// (three quarter-rate integer multiplies each), not by their bytes: tiles of 2^14 words, which need
-// two passes only, measured slower (338 us against 295 us for both columns of 2^24).
+// global segments of at least 64 words.  The passes are bound by the butterflies' instructions (a
+// Montgomery product and two modular additions each, plus the LDS traffic), not by their bytes: tiles
+// of 2^14 words, which need two passes only, measured slower (338 us against 295 us for both columns
+// of 2^24).
 constexpr int NTT_TILE_BITS = 12;
 constexpr int NTT_BLOCK = 256;
 constexpr int NTT_MAX_UPPER_STAGES = 7;  // per pass above the last: segments of 2^(12-7) words at least

@@ -595,34 +595,34 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
 // message, runs the transcript and leaves the next challenge in ctrl.  (A last-workgroup-done scheme
 // inside the round kernel needs a device-scope fence per workgroup, which on this part writes back the
 // XCD's whole L2 and costs more than a launch.)
-// sums[o] = sum over the workgroups' partial rows of word o (o < width): thread t takes column
-// t % pstride of the rows t / pstride, t / pstride + rstep, ...; four loads in flight per thread.
+// sums[o] = sum over the workgroups' partial rows of word o (o < width <= blockDim.x): thread t takes column
+// t % width of the rows t / width, t / width + groups, ... with groups = blockDim.x / width, so that all
+// threads share the rows whatever the row stride; eight loads in flight per thread.
 // All threads of the workgroup call; scratch holds blockDim.x words.
 __device__ __forceinline__ void sum_partials(const uint32_t *partials, uint32_t nblocks, uint32_t ps, uint32_t width,
                                              uint32_t *scratch, uint32_t *sums) {
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
-  for (uint32_t col0 = 0; col0 < ps; col0 += nthreads) {
-    const uint32_t col = col0 + (ps < nthreads ? tid % ps : tid);
-    const uint32_t row0 = ps < nthreads ? tid / ps : 0, rstep = ps < nthreads ? nthreads / ps : 1;
-    uint32_t v0 = 0, v1 = 0, v2 = 0, v3 = 0;
-    if (col < width) {
-      const uint32_t *p = partials + col;
-      uint32_t b = row0;
-      for (; b + 3 * rstep < nblocks; b += 4 * rstep) {
-        uint32_t x0 = p[(uint64_t)b * ps], x1 = p[(uint64_t)(b + rstep) * ps], x2 = p[(uint64_t)(b + 2 * rstep) * ps],
-                 x3 = p[(uint64_t)(b + 3 * rstep) * ps];
-        v0 = fadd(v0, x0), v1 = fadd(v1, x1), v2 = fadd(v2, x2), v3 = fadd(v3, x3);
-      }
-      for (; b < nblocks; b += rstep) v0 = fadd(v0, p[(uint64_t)b * ps]);
+  const uint32_t groups = width ? nthreads / width : 0, col = width ? tid % width : 0, row0 = width ? tid / width : 0;
+  uint32_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (row0 < groups) {
+    const uint32_t *p = partials + col;
+    uint32_t b = row0;
+    for (; b + 7 * groups < nblocks; b += 8 * groups) {
+      uint32_t x[8];
+#pragma unroll
+      for (int q = 0; q < 8; q++) x[q] = p[(uint64_t)(b + q * groups) * ps];
+#pragma unroll
+      for (int q = 0; q < 8; q++) v[q] = fadd(v[q], x[q]);
     }
-    __syncthreads();
-    scratch[tid] = fadd(fadd(v0, v1), fadd(v2, v3));
-    __syncthreads();
-    if (tid < (ps < nthreads ? ps : nthreads) && col0 + tid < width) {
-      uint32_t total = scratch[tid];
-      for (uint32_t g = 1; g < rstep; g++) total = fadd(total, scratch[g * ps + tid]);
-      sums[col0 + tid] = total;
-    }
+    for (; b < nblocks; b += groups) v[0] = fadd(v[0], p[(uint64_t)b * ps]);
+  }
+  __syncthreads();
+  scratch[tid] = fadd(fadd(fadd(v[0], v[1]), fadd(v[2], v[3])), fadd(fadd(v[4], v[5]), fadd(v[6], v[7])));
+  __syncthreads();
+  if (tid < width) {
+    uint32_t total = scratch[tid];
+    for (uint32_t g = 1; g < groups; g++) total = fadd(total, scratch[g * width + tid]);
+    sums[tid] = total;
   }
   __syncthreads();
 }

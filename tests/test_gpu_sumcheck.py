@@ -270,8 +270,8 @@ def test_rounds_on_a_grid_of_lds_resident_slices(form, names, cnames, d, base, w
 ])
 def test_round_one_in_the_base_field_and_the_double_fold(form, names, cnames, d, n, monkeypatch):
     """With base tables and streaming rounds 1 and 2 (forced here at small n; the headline sizes take this path
-    by themselves) round 1 is summed from base-field products at the nodes of r0 and round 2 folds twice at
-    once: same proof bytes, finals and folded tables as the oracle."""
+    by themselves) rounds 0 and 1 are summed from base-field products on a grid of (X0, X1) and round 2 folds
+    twice at once: same proof bytes, finals and folded tables as the oracle."""
     monkeypatch.setenv("EXACTA_HIP_MAX_SLICE_PAIRS", "0")
     rng = np.random.default_rng(n * 10 + d)
     tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in names]
@@ -288,3 +288,16 @@ def test_round_one_in_the_base_field_and_the_double_fold(form, names, cnames, d,
     assert tr.proof() == proof
     for t in dev:
         t.free()
+
+
+@pytest.mark.parametrize("K,n,d,with_eq", [(2, 8, 4, True), (4, 10, 4, False), (2, 6, 8, True)])
+def test_base_field_sweep_with_block_weights(K, n, d, with_eq, monkeypatch):
+    """The same opening sweep when block weights are the HIGH factor (K a power of two, base tables)."""
+    monkeypatch.setenv("EXACTA_HIP_MAX_SLICE_PAIRS", "0")
+    rng = np.random.default_rng(K * 100 + n)
+    tables = [rng.integers(0, P, K << n, dtype=np.uint32) for _ in range(3)]
+    bw = rand_ext(rng, (K,), d)
+    eq = rand_ext(rng, (n,), d) if with_eq else None
+    consts = rand_ext(rng, (1,), d)
+    prove_both("nodes-bw", d, n, CONFIG2, ["t0", "t1", "t2"], tables, eq=eq, constants=consts, cnames=["alpha"],
+               block_weights=bw)
