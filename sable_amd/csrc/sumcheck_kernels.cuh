@@ -333,6 +333,70 @@ __device__ __forceinline__ void load_pair(const Desc &d, const uint32_t *const *
   }
 }
 
+// The same in two steps, so that a pair's loads can be issued one pair ahead of its arithmetic: the words as
+// they lie in memory (QUADS 16-byte quads per table), then the pair from them.
+template <int D, bool IN_BASE, bool FOLD, bool FOLD2>
+constexpr int raw_quads() {
+  return FOLD2 ? 2 : (FOLD && IN_BASE) ? 1 : FOLD ? D : IN_BASE ? 1 : D / 2;
+}
+template <int D, bool IN_BASE, bool FOLD, bool FOLD2, int Q, class Desc>
+__device__ __forceinline__ void fetch_raw(const Desc &d, const uint32_t *const *in, uint64_t i, uint4 (*raw)[Q]) {
+#pragma unroll
+  for (int t = 0; t < MAXT; t++) {
+    if (t < d.T) {
+      if constexpr (!FOLD2 && !FOLD && IN_BASE) {
+        uint2 e = *reinterpret_cast<const uint2 *>(in[t] + 2 * i);
+        raw[t][0] = make_uint4(e.x, e.y, 0u, 0u);
+      } else {
+        // words per pair: 8 (FOLD2), 4 (base, folding), 4 D (extension, folding), 2 D (extension)
+        const uint4 *p = reinterpret_cast<const uint4 *>(in[t]) + (uint64_t)Q * i;
+#pragma unroll
+        for (int q = 0; q < Q; q++) raw[t][q] = p[q];
+      }
+    }
+  }
+}
+template <int D>
+__device__ __forceinline__ Ext<D> ext_from_quads(const uint4 *q) {
+  Ext<D> e;
+  e.c[0] = q[0].x, e.c[1] = q[0].y, e.c[2] = q[0].z, e.c[3] = q[0].w;
+  if constexpr (D == 8) e.c[4] = q[1].x, e.c[5] = q[1].y, e.c[6] = q[1].z, e.c[7] = q[1].w;
+  return e;
+}
+template <int D, bool IN_BASE, bool FOLD, class V, bool FOLD2, int Q, class Desc>
+__device__ __forceinline__ void pair_from_raw(const Desc &d, const uint4 (*raw)[Q], uint32_t *const *out, uint64_t i,
+                                              const Ext<D> &r, V *lo, V *hi, const BindWeights<D> *bw) {
+#pragma unroll
+  for (int t = 0; t < MAXT; t++) {
+    if (t < d.T) {
+      if constexpr (FOLD2) {
+        const uint4 e = raw[t][0], f = raw[t][1];
+        lo[t] = bind4<D>(*bw, e.x, e.y, e.z, e.w);
+        hi[t] = bind4<D>(*bw, f.x, f.y, f.z, f.w);
+      } else if constexpr (FOLD && IN_BASE) {
+        const uint4 e = raw[t][0];
+        lo[t] = fold_base<D>(e.x, e.y, r);
+        hi[t] = fold_base<D>(e.z, e.w, r);
+      } else if constexpr (FOLD) {
+        constexpr int E = D / 4;  // quads per element
+        lo[t] = fold_ext<D>(ext_from_quads<D>(raw[t]), ext_from_quads<D>(raw[t] + E), r);
+        hi[t] = fold_ext<D>(ext_from_quads<D>(raw[t] + 2 * E), ext_from_quads<D>(raw[t] + 3 * E), r);
+      } else if constexpr (IN_BASE) {
+        lo[t] = raw[t][0].x;
+        hi[t] = raw[t][0].y;
+      } else {
+        constexpr int E = D / 4;
+        lo[t] = ext_from_quads<D>(raw[t]);
+        hi[t] = ext_from_quads<D>(raw[t] + E);
+      }
+      if constexpr (FOLD) {
+        store_ext<D>(out[t] + 2 * i * D, lo[t]);
+        store_ext<D>(out[t] + (2 * i + 1) * D, hi[t]);
+      }
+    }
+  }
+}
+
 // the value of lane (l ^ M) of the wavefront
 template <int M>
 __device__ __forceinline__ uint32_t lane_xor(uint32_t v) {
@@ -524,7 +588,7 @@ struct RoundShape {
   bool deferred, do_sums;
 };
 
-template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false>
+template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false, bool GENERATED = false>
 __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const *in, uint32_t *const *out,
                                            const RoundShape<D> &sh, const Ext<D> &r, uint32_t block,
                                            uint32_t *partial_row, const BindWeights<D> *bw = nullptr) {
@@ -541,15 +605,47 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
 #pragma unroll
     for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
 
-  for (uint32_t k = 0; k < sh.pairs_per_thread; k++) {
-    const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
-    if (i >= sh.n_pairs) break;
-    V lo[MAXT], hi[MAXT];
-    load_pair<D, IN_BASE, FOLD, V, Desc, FOLD2>(d, in, out, i, r, lo, hi, bw);
-    if (sh.do_sums) {
-      Ext<D> w = load_ext<D>(sh.low + (i & low_mask) * D);
-      if (!sh.deferred) w = ext_mul_mont<D>(w, load_ext<D>(sh.high + (i >> sh.low_bits) * D));
-      accumulate_pair<D, V>(d, lo, hi, w, acc);
+  // With a statement known at compile time and D = 4 the next pair's words are fetched before this pair's
+  // arithmetic (two workgroups per compute unit leave the registers for it, and too few wavefronts to hide the
+  // loads behind one another); the interpreter and D = 8 keep the plain order.
+  constexpr bool AHEAD = GENERATED && D == 4;
+  if constexpr (AHEAD) {
+    constexpr int Q = raw_quads<D, IN_BASE, FOLD, FOLD2>();
+    uint4 raw[MAXT][Q], ahead[MAXT][Q];
+    if (tile_start + tid < sh.n_pairs) fetch_raw<D, IN_BASE, FOLD, FOLD2, Q>(d, in, tile_start + tid, raw);
+    for (uint32_t k = 0; k < sh.pairs_per_thread; k++) {
+      const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
+      if (i >= sh.n_pairs) break;
+      const bool more = k + 1 < sh.pairs_per_thread && i + BLOCK < sh.n_pairs;
+      if (more) fetch_raw<D, IN_BASE, FOLD, FOLD2, Q>(d, in, i + BLOCK, ahead);
+      Ext<D> w;
+      if (sh.do_sums) w = load_ext<D>(sh.low + (i & low_mask) * D);
+      V lo[MAXT], hi[MAXT];
+      pair_from_raw<D, IN_BASE, FOLD, V, FOLD2, Q>(d, raw, out, i, r, lo, hi, bw);
+      if (sh.do_sums) {
+        if (!sh.deferred) w = ext_mul_mont<D>(w, load_ext<D>(sh.high + (i >> sh.low_bits) * D));
+        accumulate_pair<D, V>(d, lo, hi, w, acc);
+      }
+      if (more) {
+#pragma unroll
+        for (int t = 0; t < MAXT; t++)
+          if (t < d.T) {
+#pragma unroll
+            for (int q = 0; q < Q; q++) raw[t][q] = ahead[t][q];
+          }
+      }
+    }
+  } else {
+    for (uint32_t k = 0; k < sh.pairs_per_thread; k++) {
+      const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
+      if (i >= sh.n_pairs) break;
+      V lo[MAXT], hi[MAXT];
+      load_pair<D, IN_BASE, FOLD, V, Desc, FOLD2>(d, in, out, i, r, lo, hi, bw);
+      if (sh.do_sums) {
+        Ext<D> w = load_ext<D>(sh.low + (i & low_mask) * D);
+        if (!sh.deferred) w = ext_mul_mont<D>(w, load_ext<D>(sh.high + (i >> sh.low_bits) * D));
+        accumulate_pair<D, V>(d, lo, hi, w, acc);
+      }
     }
   }
   if (!sh.do_sums) return;
@@ -566,7 +662,7 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
   }
 }
 
-template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false>
+template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false, bool GENERATED = false>
 __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &args) {
   Ext<D> r = ext_zero<D>();
   if constexpr (FOLD2) {  // challenge 0 from the log, challenge 1 is the latest
@@ -576,7 +672,7 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
     BindWeights<D> bw = bind_weights<D>(r0, r1);
     RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
                      args.do_sums != 0};
-    round_core<D, true, true, Desc, true>(d, args.in, args.out, sh, r, blockIdx.x,
+    round_core<D, true, true, Desc, true, GENERATED>(d, args.in, args.out, sh, r, blockIdx.x,
                                           args.partials + (uint64_t)blockIdx.x * args.pstride, &bw);
     return;
   }
@@ -587,7 +683,7 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
   }
   RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
                    args.do_sums != 0};
-  round_core<D, IN_BASE, FOLD>(d, args.in, args.out, sh, r, blockIdx.x,
+  round_core<D, IN_BASE, FOLD, Desc, false, GENERATED>(d, args.in, args.out, sh, r, blockIdx.x,
                                args.partials + (uint64_t)blockIdx.x * args.pstride);
 }
 
@@ -1146,16 +1242,16 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
 
 // a kernel generated for one statement: S::d is its descriptor, known at compile time
 template <int D, bool IN_BASE, bool FOLD, class S>
-__global__ __launch_bounds__(BLOCK) void round_kernel(RoundArgs<D> args) {
-  round_body<D, IN_BASE, FOLD>(S::d, args);
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(2, 2))) void round_kernel(RoundArgs<D> args) {
+  round_body<D, IN_BASE, FOLD, decltype(S::d), false, true>(S::d, args);
 }
 template <int D, class S>
 __global__ __launch_bounds__(BLOCK) void tail_kernel(TailArgs<D> args) {
   tail_body<D>(S::d, args);
 }
 template <int D, class S>
-__global__ __launch_bounds__(BLOCK) void round_kernel_fold2(RoundArgs<D> args) {
-  round_body<D, true, true, decltype(S::d), true>(S::d, args);
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(2, 2))) void round_kernel_fold2(RoundArgs<D> args) {
+  round_body<D, true, true, decltype(S::d), true, true>(S::d, args);
 }
 template <int D, class S, int PASS, int SPP>
 __global__ __launch_bounds__(BLOCK) void nodes_kernel(NodesArgs<D> args) {
