@@ -1160,27 +1160,35 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
       if (args.ev[g][e] == x) at = e;
     return at;
   };
-  // ---- round 0: accumulator (g, e) = eq(w1, 0) * slot(X1 = 0, node ev_e) + eq(w1, 1) * slot(X1 = 1, node ev_e)
+  // accumulator tid is point e of group g, whose slots start at `base` (every thread finds its own, so that the
+  // accumulators' sums below run side by side on the lanes of one wavefront)
+  uint32_t g = 0, e = 0, base = 0;
+  bool mine = false;
   {
-    uint32_t a = 0, base = 0;
-    for (uint32_t g = 0; g < args.groups; g++) {
-      const uint32_t deg = args.deg[g], nev = args.nev[g], row0 = row_of(g, 0), row1 = row_of(g, 1);
-      for (uint32_t e = 0; e < nev; e++, a++) {
-        if (tid == a) {
-          const uint32_t node = args.ev[g][e];
-          Ext<D> at0 = slot(base + row0 * (deg + 1) + node);
-          Ext<D> at1 = row1 < nev ? slot(base + row1 * (deg + 1) + node) : slot(base + nev * (deg + 1) + e);
-          if (args.eq1) {
-            at1 = ext_mul_mont<D>(at1, load_ext<D>(args.eq1));
-            at0 = ext_mul_mont<D>(at0, load_ext<D>(args.eq1 + D));
-          }
-          const Ext<D> total = ext_add<D>(at0, at1);
-#pragma unroll
-          for (int c = 0; c < D; c++) sums[a * D + c] = total.c[c];
-        }
+    uint32_t a = 0;
+    for (uint32_t k = 0; k < args.groups && !mine; k++) {
+      const uint32_t nev = args.nev[k];
+      if (tid < a + nev) {
+        g = k, e = tid - a, mine = true;
+      } else {
+        a += nev;
+        base += nev * (args.deg[k] + 1) + (row_of(k, 1) < nev ? 0 : nev);
       }
-      base += nev * (deg + 1) + (row1 < nev ? 0 : nev);
     }
+  }
+  // ---- round 0: accumulator (g, e) = eq(w1, 0) * slot(X1 = 0, node ev_e) + eq(w1, 1) * slot(X1 = 1, node ev_e)
+  if (mine) {
+    const uint32_t deg = args.deg[g], nev = args.nev[g], row0 = row_of(g, 0), row1 = row_of(g, 1);
+    const uint32_t node = args.ev[g][e];
+    Ext<D> at0 = slot(base + row0 * (deg + 1) + node);
+    Ext<D> at1 = row1 < nev ? slot(base + row1 * (deg + 1) + node) : slot(base + nev * (deg + 1) + e);
+    if (args.eq1) {
+      at1 = ext_mul_mont<D>(at1, load_ext<D>(args.eq1));
+      at0 = ext_mul_mont<D>(at0, load_ext<D>(args.eq1 + D));
+    }
+    const Ext<D> total = ext_add<D>(at0, at1);
+#pragma unroll
+    for (int c = 0; c < D; c++) sums[tid * D + c] = total.c[c];
   }
   __syncthreads();
   round_message<D>(sums, nacc, points, epi.mtilde, epi.c0, &epi);
@@ -1211,25 +1219,17 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
   }
   __syncthreads();
   // accumulator (g, e) = sum over nodes of basis * slot
-  {
-    uint32_t a = 0, base = 0;
-    for (uint32_t g = 0; g < args.groups; g++) {
-      const uint32_t deg = args.deg[g], nev = args.nev[g];
-      for (uint32_t e = 0; e < nev; e++, a++) {
-        if (tid == a) {
-          Ext<D> total = ext_zero<D>();
-          for (uint32_t m = 0; m <= deg; m++) {
-            Ext<D> lb;
+  if (mine) {
+    const uint32_t deg = args.deg[g];
+    Ext<D> total = ext_zero<D>();
+    for (uint32_t m = 0; m <= deg; m++) {
+      Ext<D> lb;
 #pragma unroll
-            for (int c = 0; c < D; c++) lb.c[c] = basis[(deg * (MAXDEG + 1) + m) * D + c];
-            total = ext_add<D>(total, ext_mul_mont<D>(lb, slot(base + e * (deg + 1) + m)));
-          }
-#pragma unroll
-          for (int c = 0; c < D; c++) sums[a * D + c] = total.c[c];
-        }
-      }
-      base += nev * (deg + 1) + (row_of(g, 1) < nev ? 0 : nev);
+      for (int c = 0; c < D; c++) lb.c[c] = basis[(deg * (MAXDEG + 1) + m) * D + c];
+      total = ext_add<D>(total, ext_mul_mont<D>(lb, slot(base + e * (deg + 1) + m)));
     }
+#pragma unroll
+    for (int c = 0; c < D; c++) sums[tid * D + c] = total.c[c];
   }
   __syncthreads();
   round_message<D>(sums, nacc, points, epi.mtilde, epi.c0, &epi);
