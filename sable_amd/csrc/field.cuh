@@ -235,4 +235,39 @@ EXH_HD Ext<D> acc_reduce_ext(const Acc96 *acc) {
   return o;
 }
 
+#if defined(__HIPCC__)
+// ---- KoalaBear in double precision, for the products of base-field values that are sums and differences of
+// table entries: integers below 2^53 are exact there, so the lines' values need no reduction between additions
+// (three integer operations each otherwise) and a product mod p takes six operations, as a Montgomery product
+// with its final correction does.  Every step below is exact integer arithmetic: a product a b is held as the
+// pair (h, l) of its rounded value and the rounding error, the quotient estimate q = rint(h / p) is off by far
+// less than one, and h - q p + l is then a small integer.
+constexpr double F_P = 2130706433.0, F_PINV = 1.0 / 2130706433.0, F_MAGIC = 6755399441055744.0;  // 1.5 * 2^52
+// v mod p in about [-p/2, p/2] for an integer |v| < 2^80
+__device__ __forceinline__ double f_reduce(double v) {
+  double q = __builtin_fma(v, F_PINV, F_MAGIC) - F_MAGIC;  // rint(v / p) for |v / p| < 2^51
+  return __builtin_fma(-q, F_P, v);
+}
+// a b mod p in about [-p/2 - 2^27, p/2 + 2^27] for integers |a b| < 2^80
+__device__ __forceinline__ double f_mul(double a, double b) {
+  double h = a * b;
+  double l = __builtin_fma(a, b, -h);
+  double q = __builtin_fma(h, F_PINV, F_MAGIC) - F_MAGIC;
+  return __builtin_fma(-q, F_P, h) + l;
+}
+// c x for a table value x and a statement's integer coefficient c (a residue: large ones stand for negatives)
+__device__ __forceinline__ double f_scale(double x, uint32_t c) {
+  return c == 1 ? x : c == P - 1 ? -x : f_mul(x, c > P / 2 ? (double)c - F_P : (double)c);
+}
+// a residue of v below 2^32 as an integer, for |v| < p + 2^28: v + p sits in the low word of v + p + 1.5 * 2^52
+__device__ __forceinline__ uint32_t f_residue32(double v) {
+  return (uint32_t)__double_as_longlong(v + (F_P + F_MAGIC));
+}
+// the canonical residue of an integer |v| < 2^80
+__device__ __forceinline__ uint32_t f_canonical(double v) {
+  const int32_t r = (int32_t)f_reduce(v);
+  return r < 0 ? (uint32_t)(r + (int32_t)P) : (uint32_t)r;
+}
+#endif
+
 }  // namespace exh
