@@ -20,6 +20,8 @@ u64p = C.POINTER(C.c_uint64)
 
 
 def _u32(a):
+    if isinstance(a, np.ndarray) and a.dtype == np.uint32 and a.flags.c_contiguous and a.max(initial=0) < P:
+        return a
     a = np.asarray(a, dtype=np.uint64)
     out = np.empty(a.shape, np.uint32)
     out[...] = a % P
@@ -27,7 +29,13 @@ def _u32(a):
 
 
 def _p(a):
-    return a.ctypes.data_as(u32p) if a is not None else None
+    """The array as a C pointer argument.  A ctypes array over the same buffer costs a fifth of ndarray.ctypes
+    (0.6 us against 3.5 us, and a prove passes seven of them)."""
+    if a is None:
+        return None
+    if a.size and a.flags.c_contiguous and a.flags.writeable and a.dtype == np.uint32:
+        return (C.c_uint32 * a.size).from_buffer(a)
+    return a.ctypes.data_as(u32p)
 
 
 def _bytes(label):
