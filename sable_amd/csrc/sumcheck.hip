@@ -21,10 +21,13 @@ struct EqTables {
   int first[64], bits[64];
 };
 
+// (both set-up kernels also clear the totals of the grid launch of LDS-resident slices: the first launch of a
+// session is the one place that comes before every use)
 template <int D>
 __global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const uint32_t *factors, uint32_t *out,
-                                                          uint64_t total) {
+                                                          uint64_t total, uint32_t *zero, uint64_t zero_words) {
   uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  for (uint64_t z = gid; z < zero_words; z += (uint64_t)gridDim.x * BLOCK) zero[z] = 0;
   if (gid >= total) return;
   int k = 0;
   uint64_t start = 0;
@@ -42,8 +45,9 @@ __global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const u
 }
 
 template <int D>
-__global__ __launch_bounds__(BLOCK) void fill_ones_kernel(uint32_t *out, uint64_t n) {
+__global__ __launch_bounds__(BLOCK) void fill_ones_kernel(uint32_t *out, uint64_t n, uint32_t *zero, uint64_t zero_words) {
   uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  for (uint64_t z = gid; z < zero_words; z += (uint64_t)gridDim.x * BLOCK) zero[z] = 0;
   if (gid < n) store_ext<D>(out + gid * D, ext_lift<D>(1));
 }
 
@@ -243,10 +247,12 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   node_slots_n = node_slots(desc);  // grid sums of the sweep that serves rounds 0 and 1 from the base tables
   pstride = next_pow2((uint64_t)std::max(std::max(st.nacc, 1), node_slots_n <= MAXACC ? node_slots_n : 0) * D);
   uint64_t partial_off = pos * D;  // from here in words
-  // (a grid of LDS-resident slices keeps 64-bit totals per round and group in the same place)
-  const uint64_t partial_rows = std::max<uint64_t>(max_grid, 2 * MAXTAIL * SLICE_GROUPS);
+  const uint64_t partial_rows = max_grid;
   uint64_t words = partial_off + (partial_rows + 1) * (uint64_t)pstride + 64;
   words += 64;
+  words += words & 1;  // the 64-bit totals of the grid launch of slices: [MAXTAIL][SLICE_GROUPS][pstride]
+  const uint64_t slice_totals_off = words;
+  words += (uint64_t)2 * MAXTAIL * SLICE_GROUPS * pstride;
   // mixed base / extension inputs: lift the base ones
   bool any_base = false, all_base = true;
   for (int t = 0; t < T; t++) {
@@ -268,6 +274,7 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   d_weights = base;
   d_partials = base + partial_off;
   d_sums = d_partials + partial_rows * (uint64_t)pstride;
+  d_slice_totals = reinterpret_cast<unsigned long long *>(base + slice_totals_off);
   d_ctrl = reinterpret_cast<Ctrl *>(base + ctrl_off);
   d_mtilde = base + mt_off;
   d_c0 = base + c0_off;
@@ -327,29 +334,43 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
 }
 
 // the weight tables of every round from the eq point's factors (or all-ones tables without one)
+static uint64_t tail_pairs(int T, int D);
+
 int SumcheckSession::launch_setup() {
   Context &c = ctx();
   uint32_t *base = d_weights;
   EqTables eqt;
   memcpy(&eqt, setup.eqt, sizeof(eqt));
+  // a session whose first round fits the one-workgroup launch never takes the grid launch
+  uint32_t *zero = reinterpret_cast<uint32_t *>(d_slice_totals);
+  uint64_t zero_words = size / 2 > tail_pairs(st.T(), D) ? (uint64_t)2 * MAXTAIL * SLICE_GROUPS * pstride : 0;
+  const uint32_t zero_grid = (uint32_t)((zero_words + 4 * BLOCK - 1) / (4 * BLOCK));  // four words a thread
+  bool cleared = false;
   if (setup.total_eq) {
-    uint32_t grid = (uint32_t)((setup.total_eq + BLOCK - 1) / BLOCK);
+    uint32_t grid = std::max((uint32_t)((setup.total_eq + BLOCK - 1) / BLOCK), zero_grid);
     // tables are laid out in launch order, so thread gid maps to table k by running sums; the
     // offsets themselves may skip other regions, so they are taken from eqt.off
     if (D == 4)
-      hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq);
+      hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq,
+                         zero, zero_words);
     else
-      hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq);
+      hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq,
+                         zero, zero_words);
+    cleared = zero_words > 0;
+    zero_words = 0;
   }
   if (setup.ones_len) {
-    uint32_t grid = (uint32_t)((setup.ones_len + BLOCK - 1) / BLOCK);
+    uint32_t grid = std::max((uint32_t)((setup.ones_len + BLOCK - 1) / BLOCK), zero_words ? zero_grid : 0u);
     if (D == 4)
       hipLaunchKernelGGL(fill_ones_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, base + setup.ones_off * D,
-                         setup.ones_len);
+                         setup.ones_len, zero, zero_words);
     else
       hipLaunchKernelGGL(fill_ones_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, base + setup.ones_off * D,
-                         setup.ones_len);
+                         setup.ones_len, zero, zero_words);
+    cleared = cleared || zero_words > 0;
+    zero_words = 0;
   }
+  slice_totals_clear = cleared;  // else (no set-up kernel ran) the grid launch clears them itself
   EXH_HIP(hipGetLastError());
   return OK;
 }
@@ -880,7 +901,7 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
     a.ctrl = d_ctrl;
     a.mtilde = d_mtilde;
     a.c0 = d_c0 + (size_t)j * points * D;
-    a.totals = reinterpret_cast<unsigned long long *>(d_partials);
+    a.totals = d_slice_totals;
     a.pstride = pstride;
     a.groups = groups;
     a.spin_limit = 200000;
@@ -890,8 +911,9 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
       a.low_bits[jj] = (uint32_t)low_bits[j + jj];
     }
   };
-  if (grid > 1)  // the rounds' totals start at zero (64-bit words)
-    EXH_HIP(hipMemsetAsync(d_partials, 0, (size_t)rounds * groups * pstride * 8, c.stream));
+  if (grid > 1 && !slice_totals_clear)  // the rounds' totals start at zero (64-bit words)
+    EXH_HIP(hipMemsetAsync(d_slice_totals, 0, (size_t)rounds * groups * pstride * 8, c.stream));
+  if (grid > 1) slice_totals_clear = false;
   c.prof_begin(grid > 1 ? "slices" : "tail", j,
                (uint64_t)T * size * (cur_base ? 1 : D) * 4 + (uint64_t)T * final_size * D * 4);
   if (D == 4) {
