@@ -133,7 +133,9 @@ int ctx_init(int device) {
   }
   EXH_HIP(hipStreamCreate(&c.stream));
   c.host_pinned_words = 1 << 16;
-  EXH_HIP(hipHostMalloc((void **)&c.host_pinned, c.host_pinned_words * 4, hipHostMallocDefault));
+  // coherent and mapped: a kernel writes a sumcheck's logs into it directly and the host polls for them
+  EXH_HIP(hipHostMalloc((void **)&c.host_pinned, c.host_pinned_words * 4, hipHostMallocMapped | hipHostMallocCoherent));
+  EXH_HIP(hipHostGetDevicePointer((void **)&c.host_pinned_dev, c.host_pinned, 0));
   c.device = device;
   c.compute_units = prop.multiProcessorCount;
   c.ready = true;

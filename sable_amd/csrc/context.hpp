@@ -79,6 +79,8 @@ struct Context {
   Arena tree;            // the layers of a fraction tree above its leaves, for the length of one proof
   uint32_t *host_pinned = nullptr;  // small pinned buffer for per-round results
   size_t host_pinned_words = 0;
+  uint32_t *host_pinned_dev = nullptr;  // the same buffer as kernels address it
+  uint32_t log_seq = 0;  // counts the control blocks that launches delivered to host_pinned themselves
   int require();  // OK, or E_DEVICE with the reason when the library is not initialised
 };
 

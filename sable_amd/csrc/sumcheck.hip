@@ -1,5 +1,6 @@
 // sumcheck.hip -- sumcheck session: weight tables, round launches, partial-sum reduction, folds.
 #include "sumcheck.hpp"
+#include <atomic>
 
 #include <string.h>
 
@@ -834,23 +835,52 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     folds_due = 1;
     tail_done = false;
   }
+  uint32_t *down = c.host_pinned + PIN_DOWN;
+  const size_t ctrl_words = (sizeof(Ctrl) + 3) / 4;
+  bool logged_to_host = false;
   if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
+    // when a single entry per table is left at the end (the finals travel in the control block), the launch
+    // itself delivers the control block to pinned host memory
+    const bool deliver = !c.profiling && (size >> ((folds_due > 0 ? 1 : 0) + (n - j))) == 1;
+    if (deliver) {
+      host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = ++c.log_seq;
+      reinterpret_cast<volatile uint32_t *>(down)[ctrl_words] = 0;
+    }
     status = launch_tail(j, n - j, 1, folds_due > 0);
+    host_log = nullptr;
     folds_due = 0;
     tail_done = status == OK;
+    logged_to_host = deliver && tail_done;
   }
   device_loop = false;
   if (status) return status;
   // ---- read the logs back, and with them what the tail left of the tables: one wait for both
-  uint32_t *down = c.host_pinned + PIN_DOWN;
-  const size_t ctrl_words = (sizeof(Ctrl) + 3) / 4, final_words = (size_t)T * size * D;
-  EXH_HIP(hipMemcpyAsync(down, d_ctrl, sizeof(Ctrl), hipMemcpyDeviceToHost, c.stream));
+  const size_t final_words = (size_t)T * size * D;
   final_cache.clear();
   const bool in_ctrl = tail_done && size == 1;  // the tail left the finals in the control block
   const bool with_finals = tail_done && !in_ctrl && ctrl_words + final_words <= PIN_DOWN_WORDS;
-  if (with_finals)  // the tail wrote table t at t * size * D of one arena
-    EXH_HIP(hipMemcpyAsync(down + ctrl_words, cur[0], final_words * 4, hipMemcpyDeviceToHost, c.stream));
-  EXH_HIP(hipStreamSynchronize(c.stream));
+  if (logged_to_host) {
+    // the flag follows the block through the same path, so seeing it means the block is there; a stream that
+    // ends without raising it (a launch gave up) is caught by the query
+    volatile uint32_t *flag = reinterpret_cast<volatile uint32_t *>(down) + ctrl_words;
+    uint32_t spins = 0;
+    while (*flag != c.log_seq) {
+      if ((++spins & 1023) == 0 && hipStreamQuery(c.stream) == hipSuccess) break;
+    }
+    if (*flag != c.log_seq) {
+      EXH_HIP(hipStreamSynchronize(c.stream));
+      if (*flag != c.log_seq) {
+        set_error("device-error: the device loop ended without delivering its logs");
+        return E_DEVICE;
+      }
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
+  } else {
+    EXH_HIP(hipMemcpyAsync(down, d_ctrl, sizeof(Ctrl), hipMemcpyDeviceToHost, c.stream));
+    if (with_finals)  // the tail wrote table t at t * size * D of one arena
+      EXH_HIP(hipMemcpyAsync(down + ctrl_words, cur[0], final_words * 4, hipMemcpyDeviceToHost, c.stream));
+    EXH_HIP(hipStreamSynchronize(c.stream));
+  }
   const Ctrl *rc = reinterpret_cast<const Ctrl *>(down);
   if (with_finals) final_cache.assign(down + ctrl_words, down + ctrl_words + final_words);
   if (in_ctrl) final_cache.assign(rc->finals, rc->finals + final_words);
@@ -905,6 +935,7 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
     a.pstride = pstride;
     a.groups = groups;
     a.spin_limit = 200000;
+    a.host_log = host_log, a.host_flag_at = host_flag_at, a.host_seq = host_seq;
     for (int jj = 0; jj < rounds; jj++) {
       a.low_off[jj] = low_off[j + jj];
       a.high_off[jj] = high_off[j + jj];

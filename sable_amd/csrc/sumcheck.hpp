@@ -44,6 +44,8 @@ struct SumcheckSession {
   uint32_t *d_partials = nullptr, *d_sums = nullptr, *d_lifted = nullptr;
   unsigned long long *d_slice_totals = nullptr;  // the totals of the grid launch of slices
   bool slice_totals_clear = false;               // cleared by the session's set-up kernel and not used since
+  uint32_t *host_log = nullptr;                  // set around the loop's last launch: where it delivers the logs
+  uint32_t host_flag_at = 0, host_seq = 0;
   uint64_t max_grid = 0;
   uint32_t pstride = 0;  // words per workgroup partial
   int node_slots_n = 0;  // (group, point, node) sums of the base-field round 1

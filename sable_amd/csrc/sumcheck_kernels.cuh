@@ -88,6 +88,11 @@ struct TailArgs {
   uint32_t pstride;
   uint32_t groups;           // workgroup w adds into group w % groups
   uint32_t spin_limit;       // polls of a total before giving up
+  // the last launch of a device-driven loop (one workgroup): it ends by copying the control block into pinned
+  // host memory and raising host_log[host_flag_at] to host_seq, so that the host needs neither a copy nor a wait
+  // on the stream to read the logs (null: it does both)
+  uint32_t *host_log;
+  uint32_t host_flag_at, host_seq;
 };
 
 template <int D>
@@ -907,6 +912,18 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   if (wg == 0 && tid < 64) {
     rb3s_store(tr, &args.ctrl->tr);
     if (tid == 0) args.ctrl->round = args.first_round + args.rounds;
+  }
+  if (args.host_log && G == 1) {
+    __syncthreads();
+    // every word through the L2 (this workgroup wrote some of them a moment ago, other launches the rest)
+    const uint32_t *words = reinterpret_cast<const uint32_t *>(args.ctrl);
+    for (uint32_t u = tid; u < sizeof(Ctrl) / 4; u += BLOCK)
+      args.host_log[u] = __hip_atomic_load(words + u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence_system();
+    __syncthreads();
+    if (tid == 0) {
+      __hip_atomic_store(args.host_log + args.host_flag_at, args.host_seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
   }
 }
 
