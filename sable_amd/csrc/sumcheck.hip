@@ -910,11 +910,10 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
   int status = dst.reserve((size_t)T * final_size * D * 4);
   if (status) return status;
   const uint64_t slice_entries = (first_fold ? size / 2 : size) / grid;
-  // groups of workgroups share a row of totals: few enough that a round's rows fit the scratch the
-  // kernel sums them in (MAXPTS * MAXACC * 8 words)
+  // groups of workgroups share a row of totals: few enough that a workgroup polls all the rows' words at
+  // once, one per thread (a second pass of polls is a second trip to memory in every round)
   uint32_t groups = 1;
-  while (groups * 2 <= SLICE_GROUPS && groups * 2 <= grid && groups * 2 * (uint32_t)st.nacc * D <= MAXPTS * MAXACC * 8)
-    groups *= 2;
+  while (groups * 2 <= SLICE_GROUPS && groups * 2 <= grid && groups * 2 * (uint32_t)st.nacc * D <= BLOCK) groups *= 2;
   auto fill = [&](auto &a) {
     memset(&a, 0, sizeof(a));
     for (int t = 0; t < T; t++) a.in[t] = cur[t];
