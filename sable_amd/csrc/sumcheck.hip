@@ -441,8 +441,8 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   return OK;
 }
 
-// Round 1 from the base tables (fold by challenge 0 pending, not performed): the slot sums in as many
-// launches as the generated kernels need, then their epilogue.
+// Rounds 0 and 1 from one sweep of the base tables (nothing folded): the slot sums in as many launches as the
+// generated kernels need, then the epilogue that sends both rounds' messages.
 template <int D>
 static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs) {
   Context &c = ctx();
@@ -760,12 +760,12 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   device_loop = true;
   bool tail_done = false;
   int status = OK, j = 0;
-  int folds_due = 0;  // folds by the last challenges drawn that the tables still await (2 after the base-field round 1)
+  int folds_due = 0;  // folds by the last challenges drawn that the tables still await (2 after the base-field sweep for rounds 0 and 1)
   const char *no_nodes = getenv("EXACTA_HIP_NO_BASE_ROUND1");
   for (; j < n && status == OK; j++) {
     const bool fold_due = folds_due > 0;
     uint64_t n_pairs = (size >> folds_due) / 2;  // pairs summed in round j (after the pending folds)
-    if (folds_due == 2) {  // round 2 after the base-field round 1: both folds at once, then the sums
+    if (folds_due == 2) {  // round 2 after the base-field sweep: both folds at once, then the sums
       round = j;
       uint64_t out_size = size / 4;
       Arena &dst = ((generation + 1) % 2 == 0) ? c.fold_a : c.fold_b;

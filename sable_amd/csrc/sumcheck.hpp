@@ -15,7 +15,7 @@ namespace exh {
 struct KernelSet {  // the launchers generated for one statement and one degree D
   void (*launch)(const void *args, bool in_base, bool fold, uint32_t grid, hipStream_t stream);
   void (*launch_tail)(const void *args, uint32_t grid, hipStream_t stream);
-  // base tables folded twice at once (after the base-field round 1), and that round's slot sums
+  // base tables folded twice at once (round 2 after the base-field sweep), and that sweep's slot sums
   void (*launch_fold2)(const void *args, uint32_t grid, hipStream_t stream);
   void (*launch_nodes)(const void *args, int pass, uint32_t grid, hipStream_t stream);
   int nodes_passes;  // launches of launch_nodes per round (0: not available)
@@ -48,7 +48,7 @@ struct SumcheckSession {
   uint32_t host_flag_at = 0, host_seq = 0;
   uint64_t max_grid = 0;
   uint32_t pstride = 0;  // words per workgroup partial
-  int node_slots_n = 0;  // (group, point, node) sums of the base-field round 1
+  int node_slots_n = 0;  // slot sums of the base-field sweep that serves rounds 0 and 1
   bool device_loop = false;
   Ctrl *d_ctrl = nullptr;
   std::vector<uint32_t> final_cache;  // the tables as the device loop's tail left them, when read back with its logs
