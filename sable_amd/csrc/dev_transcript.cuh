@@ -22,13 +22,18 @@ struct DevB3S {
   uint32_t counter_lo, counter_hi;
 };
 
-// message word used by G number g (0..7: columns 0-3, then diagonals 0-3) of round r, first and second
-// operand: the BLAKE3 message permutation applied r times (src/blake3.lisp:37-40)
-__device__ const uint8_t B3_SCHEDULE[7][16] = {
-    {0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15}, {2, 6, 3, 10, 7, 0, 4, 13, 1, 11, 12, 5, 9, 14, 15, 8},
-    {3, 4, 10, 12, 13, 2, 7, 14, 6, 5, 9, 0, 11, 15, 8, 1}, {10, 7, 12, 9, 14, 3, 13, 15, 4, 0, 11, 2, 5, 8, 1, 6},
-    {12, 13, 9, 11, 15, 10, 14, 8, 7, 2, 5, 3, 0, 1, 6, 4}, {9, 14, 11, 5, 8, 12, 15, 1, 13, 3, 0, 10, 2, 6, 4, 7},
-    {11, 15, 5, 0, 1, 9, 8, 6, 14, 10, 2, 12, 3, 4, 7, 13}};
+// S[r][k]: the message word used k-th in round r (G number g = k / 2 of columns 0-3 then diagonals 0-3, first
+// and second operand): the BLAKE3 message permutation applied r times (src/blake3.lisp:37-40).  Lane i of a
+// quad needs S[r][first + 2 i]: the four numbers, one nibble each, as a compile-time constant.
+__host__ __device__ constexpr uint32_t b3_lane_words(int r, int first) {
+  constexpr uint8_t S[7][16] = {
+      {0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15}, {2, 6, 3, 10, 7, 0, 4, 13, 1, 11, 12, 5, 9, 14, 15, 8},
+      {3, 4, 10, 12, 13, 2, 7, 14, 6, 5, 9, 0, 11, 15, 8, 1}, {10, 7, 12, 9, 14, 3, 13, 15, 4, 0, 11, 2, 5, 8, 1, 6},
+      {12, 13, 9, 11, 15, 10, 14, 8, 7, 2, 5, 3, 0, 1, 6, 4}, {9, 14, 11, 5, 8, 12, 15, 1, 13, 3, 0, 10, 2, 6, 4, 7},
+      {11, 15, 5, 0, 1, 9, 8, 6, 14, 10, 2, 12, 3, 4, 7, 13}};
+  return (uint32_t)S[r][first] | (uint32_t)S[r][first + 2] << 4 | (uint32_t)S[r][first + 4] << 8 |
+         (uint32_t)S[r][first + 6] << 12;
+}
 
 #define EXH_QUAD(v, ctrl) ((uint32_t)__builtin_amdgcn_update_dpp(0, (int)(v), (ctrl), 0xf, 0xf, false))
 
@@ -47,8 +52,9 @@ __device__ __forceinline__ void b3_compress_quad(const uint32_t cv[8], const uin
   uint32_t mx[7][2], my[7][2];
 #pragma unroll
   for (int r = 0; r < 7; r++) {  // no dependence on the state: issued ahead of the rounds
-    mx[r][0] = m[B3_SCHEDULE[r][2 * i]], my[r][0] = m[B3_SCHEDULE[r][2 * i + 1]];
-    mx[r][1] = m[B3_SCHEDULE[r][8 + 2 * i]], my[r][1] = m[B3_SCHEDULE[r][9 + 2 * i]];
+    // the four lanes' word numbers sit in the nibbles of a compile-time constant: no table in memory to read
+    mx[r][0] = m[(b3_lane_words(r, 0) >> (4 * i)) & 15u], my[r][0] = m[(b3_lane_words(r, 1) >> (4 * i)) & 15u];
+    mx[r][1] = m[(b3_lane_words(r, 8) >> (4 * i)) & 15u], my[r][1] = m[(b3_lane_words(r, 9) >> (4 * i)) & 15u];
   }
 #pragma unroll
   for (int r = 0; r < 7; r++) {
