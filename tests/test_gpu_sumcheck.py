@@ -246,6 +246,7 @@ def test_device_loop_entry_point_from_a_host_transcript_state():
     (CONFIG2, ["t0", "t1", "t2"], ["alpha"], 4, False, True, 18),
     ("(* t0 t1)", ["t0", "t1"], [], 8, False, False, 16),
     ("(+ (* t0 t1 t2) (* 7 t1) -1)", ["t0", "t1", "t2"], [], 4, True, True, 19),
+    ("(* (+ (* 5 t0) (* -3 t1) 7) (- t2 (* 2 t0)))", ["t0", "t1", "t2"], [], 4, True, True, 16),
 ])
 def test_rounds_on_a_grid_of_lds_resident_slices(form, names, cnames, d, base, with_eq, n):
     """Sizes at which the rounds between the large kernels and the last workgroup run as one launch of
@@ -267,6 +268,9 @@ def test_rounds_on_a_grid_of_lds_resident_slices(form, names, cnames, d, base, w
     ("(* t0 t1)", ["t0", "t1"], [], 4, 12),
     ("(* t0 t1)", ["t0", "t1"], [], 8, 7),
     ("(* t0 t1 t2)", ["t0", "t1", "t2"], [], 8, 10),
+    # linear forms with coefficients other than +-1 (a generated kernel exists for this one, too)
+    ("(* (+ (* 5 t0) (* -3 t1) 7) (- t2 (* 2 t0)))", ["t0", "t1", "t2"], [], 4, 9),
+    ("(* (+ (* 5 t0) (* -3 t1) 7) (- t2 (* 2 t0)))", ["t0", "t1", "t2"], [], 4, 13),
 ])
 def test_round_one_in_the_base_field_and_the_double_fold(form, names, cnames, d, n, monkeypatch):
     """With base tables and streaming rounds 1 and 2 (forced here at small n; the headline sizes take this path
