@@ -251,6 +251,52 @@ def run_commit(sa, steps, warmup, cpu_c):
     return out
 
 
+def run_combine(sa, steps, warmup, cpu_c):
+    """combine-columns at config 5's shape: the two committed columns of 2^23 base values into the table of
+    2^23 EXT8s that BaseFold opens (src/pcs.lisp:434-441)."""
+    c, ncols, d = 23, 2, 8
+    cols = sa.Table.random(5005, ncols << c)
+    cf = splitmix_field(5006, ncols * d).reshape(ncols, d)
+    lib = sa.load()
+
+    def step():
+        sa.combine_columns(cols, ncols, cf).free()
+
+    for _ in range(warmup):
+        step()
+    sa.check(lib.exh_synchronize())
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    sa.check(lib.exh_synchronize())
+    dt = (time.perf_counter() - t0) / steps
+    sa.check(lib.exh_profile_enable(1))
+    for _ in range(steps):
+        step()
+    entries = [e for e in profile_entries(sa) if e[0] == "combine_columns"]
+    sa.check(lib.exh_profile_enable(0))
+    avg_ms = sum(e[2] for e in entries) / len(entries)
+    nbytes = (1 << c) * (4 * ncols + 4 * d)
+    out = {"metric": "combine-columns entries/s (config 5's columns)", "value": ncols * (1 << c) / dt,
+           "unit": "column entries/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": 1e3 * dt,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32 (Montgomery KoalaBear, F_p^8)",
+           "data": "synthetic (SplitMix64-seeded uniform field elements)",
+           "config": {"workload": "combine-columns: 2 base columns of 2^23 with F_p^8 coefficients -> 2^23 EXT8s"},
+           "roofline": {"bound": "hbm", "kernel": "combine_columns", "achieved": nbytes / (avg_ms * 1e-3) / 1e9,
+                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "avg_launch_ms": avg_ms, "alg_bytes_per_launch": nbytes, "traffic": None}}
+    if cpu_c > 0:
+        from oracle import binding as orc
+        hc = np.stack([splitmix_field(77 + k, 1 << cpu_c) for k in range(ncols)])
+        t0 = time.perf_counter()
+        orc.combine_columns(hc, cf)
+        cdt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": ncols * (1 << cpu_c) / cdt, "unit": "column entries/s", "cores": 1, "kind": "port",
+                               "sample": f"2 columns of 2^{cpu_c} ({cdt:.2f} s)"}
+    cols.free()
+    return out
+
+
 # HBM bytes per launch of the dominant kernel at the headline workload, from two rocprofv3 --pmc runs of this
 # file (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the plain
 # copy kernel of `--workload copy`, whose traffic is known (the summary of those runs is kept with the profiles)
@@ -273,7 +319,7 @@ def run_copy(steps):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "copy"],
+    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "combine", "copy"],
                     help="config2 (default) is the headline; the others are the remaining configured workloads; "
                          "copy is the known-size kernel the traffic counters are calibrated on")
     ap.add_argument("--gpus", type=int, default=1)
@@ -305,6 +351,9 @@ def main():
         return
     if args.workload == "config5":
         print(json.dumps(run_commit(sa, args.steps, args.warmup, 18 if args.cpu_n else 0)))
+        return
+    if args.workload == "combine":
+        print(json.dumps(run_combine(sa, args.steps, args.warmup, 20 if args.cpu_n else 0)))
         return
     n, d, seed = args.n, 4, 2
     st = sa.Statement(FORM, TABLES, CONSTS)

@@ -112,6 +112,11 @@ int exh_merkle_commit(exh_table codewords, int ncols, int c, exh_table *levels, 
    2^n_domain tables (src/rs.lisp:93-101) */
 int exh_rs_fold(exh_table codeword, int degree_d, uint64_t m, int n_domain, int level, const uint32_t *r,
                 exh_table *out);
+/* COMBINE-COLUMNS (src/pcs.lisp:434-441): g[x] = sum_k coefficient_k * column_k[x], the extension table BaseFold
+   opens, from a class's ncols base columns of len values each (column k at k * len of `columns`, as PCS-COMMIT
+   takes them) and ncols coefficients of degree D (canonical, tower order); out: a new table of len elements */
+int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int degree_d, const uint32_t *coefficients,
+                        exh_table *out);
 
 /* ---- LogUp-GKR layer reductions: FRACTION-TREES (src/gkr.lisp:149-170), one in-block layer:
    p, q: K * 2^(m+1) EXTs each; out_p, out_q: K * 2^m EXTs (children (b,x), (b,x+2^m)) */

@@ -415,6 +415,16 @@ def rs_fold(codeword, twiddle_level, r):
     return out
 
 
+def combine_columns(columns, coefficients):
+    """combine-columns (src/pcs.lisp:434-441): columns (ncols, len) base values, coefficients (ncols, D)."""
+    cols, cf = _u32(columns), _u32(coefficients)
+    ncols, length = cols.shape
+    d = cf.shape[1]
+    out = np.zeros((length, d), np.uint32)
+    lib().orc_combine_columns(d, ncols, C.c_uint64(length), _p(cols), _p(cf), _p(out))
+    return out
+
+
 # ------------------------------------------------------------------ statements and sumcheck
 class Statement:
     """A statement form with its table and constant variables fixed: the oracle's monomial IR."""

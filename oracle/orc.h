@@ -147,6 +147,9 @@ void orc_rs_brute_eval(const uint32_t *message, int n, uint32_t *out);
 /* fold a codeword of 2m elements of degree D (D = 1: base) on a twiddle level of m values */
 void orc_rs_fold(int D, uint64_t m, const uint32_t *codeword, const uint32_t *twiddle_level,
                  const uint32_t *r, uint32_t *out);
+/* COMBINE-COLUMNS, src/pcs.lisp:434-441 */
+void orc_combine_columns(int D, int ncols, uint64_t len, const uint32_t *columns, const uint32_t *coefficients,
+                         uint32_t *out);
 
 /* ---- statements: a sum of monomials, the canonical form of src/forms.lisp:57-78.
    Variable v < T is table v; v >= T is constant v - T.  */

@@ -333,3 +333,17 @@ int orc_basefold_verify(orc_tr *tr, int nv, const uint32_t *rr, const uint32_t *
   if (!out_qs) free(qs);
   return ORC_OK;
 }
+
+/* COMBINE-COLUMNS, src/pcs.lisp:434-441: g[x] = sum_k coefficient_k * column_k[x] for base columns (column k at
+   columns + k * len) and extension coefficients; the sum starts from zero and runs in column order */
+void orc_combine_columns(int D, int ncols, uint64_t len, const uint32_t *columns, const uint32_t *coefficients,
+                         uint32_t *out) {
+  for (uint64_t x = 0; x < len; x++) {
+    uint32_t g[ORC_MAXD] = {0}, term[ORC_MAXD];
+    for (int k = 0; k < ncols; k++) {
+      orc_ext_scale(D, coefficients + (size_t)k * D, columns[(uint64_t)k * len + x], term);
+      orc_ext_add(D, g, term, g);
+    }
+    memcpy(out + x * D, g, D * sizeof(uint32_t));
+  }
+}

@@ -386,6 +386,17 @@ def rs_fold(codeword, d, n_domain, level, r):
     return Table(h.value, m * d, d)
 
 
+def combine_columns(columns, ncols, coefficients):
+    """combine-columns: sum_k coefficient_k * column_k over a Table of ncols base columns -> Table of EXTs."""
+    cf = _u32(coefficients)
+    d = cf.shape[-1]
+    length = columns.n_u32 // ncols
+    h = C.c_uint64()
+    check(load().exh_combine_columns(C.c_uint64(columns.handle), ncols, C.c_uint64(length), d, _p(cf.reshape(-1, d)),
+                                     C.byref(h)))
+    return Table(h.value, length * d, d)
+
+
 def pcs_commit(tr, columns, ncols, c):
     """pcs-commit of one class: encode, leaf digests, Merkle levels; the cap is sent on the transcript."""
     hc, hl = C.c_uint64(), C.c_uint64()

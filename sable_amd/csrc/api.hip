@@ -586,6 +586,21 @@ int exh_rs_fold(exh_table codeword, int D, uint64_t m, int n_domain, int level, 
   return rs_fold_device(D, m, n_domain, level, cw->ptr, r, table_of(*out)->ptr);
 }
 
+int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int D, const uint32_t *coefficients, exh_table *out) {
+  DeviceTable *cols = table_of(columns);
+  if (!cols) return E_PARAM;
+  if ((D != 4 && D != 8) || ncols < 1 || len < 1 || !coefficients || !out || cols->stride != 1 ||
+      cols->n_u32 != (uint64_t)ncols * len) {
+    set_error("invalid-parameter: columns must hold ncols * len base values, coefficients ncols elements of degree 4 or 8");
+    return E_PARAM;
+  }
+  int status = exh_table_alloc(len * D, D, out);
+  if (status) return status;
+  status = combine_columns_device(D, cols->ptr, ncols, len, coefficients, table_of(*out)->ptr);
+  if (status) exh_table_free(*out);
+  return status;
+}
+
 int exh_pcs_commit(exh_transcript h, exh_table columns, int ncols, int c, exh_table *codewords, exh_table *levels) {
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;

@@ -290,6 +290,65 @@ int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d
   return rs_fold_launch(D, m, dom->tw_inv2 + dom->off[level], d_cw, r, d_out);
 }
 
+// ------------------------------------------------------------------ COMBINE-COLUMNS (src/pcs.lisp:434-441)
+// g[x] = sum_k coefficient_k * column_k[x]: base columns (column k at cols + k * len), extension coefficients,
+// the table BaseFold opens.  One pass: 4 ncols bytes read and 4 D written per x, one x per thread (four per
+// thread measured a third slower: the 128-byte strides between lanes' stores).  The coefficients arrive as
+// kernel arguments in Montgomery form, so a reduction of four products gives their exact sum.
+constexpr int COMBINE_COLS = 32;  // columns per launch; more accumulate over launches
+template <int D>
+struct CombineArgs {
+  uint32_t coef_mont[COMBINE_COLS][D];
+};
+template <int D>
+__global__ __launch_bounds__(BLOCK) void combine_columns_kernel(const uint32_t *cols, uint64_t len, int ncols,
+                                                                CombineArgs<D> a, uint32_t *out, int accumulate) {
+  const uint64_t x = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (x >= len) return;
+  Ext<D> g = accumulate ? load_ext<D>(out + x * D) : ext_zero<D>();
+  for (int k0 = 0; k0 < ncols; k0 += 4) {  // four columns per reduction: 4 p^2 < 2^64
+    uint32_t val[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) val[q] = k0 + q < ncols ? cols[(uint64_t)(k0 + q) * len + x] : 0u;
+#pragma unroll
+    for (int c = 0; c < D; c++) {
+      uint64_t t = 0;
+#pragma unroll
+      for (int q = 0; q < 4; q++) t += (uint64_t)(k0 + q < ncols ? a.coef_mont[k0 + q][c] : 0u) * val[q];
+      g.c[c] = fadd(g.c[c], mont_reduce4(t));
+    }
+  }
+  store_ext<D>(out + x * D, g);  // (non-temporal stores measured a third slower)
+}
+
+template <int D>
+static int combine_launch(const uint32_t *d_cols, int ncols, uint64_t len, const uint32_t *coef, uint32_t *d_out) {
+  Context &c = ctx();
+  for (int first = 0; first < ncols; first += COMBINE_COLS) {
+    const int count = ncols - first < COMBINE_COLS ? ncols - first : COMBINE_COLS;
+    CombineArgs<D> a;
+    memset(&a, 0, sizeof(a));
+    for (int k = 0; k < count; k++)
+      for (int cc = 0; cc < D; cc++) a.coef_mont[k][cc] = to_mont(coef[(size_t)(first + k) * D + cc] % P);
+    const uint32_t *cols = d_cols + (uint64_t)first * len;
+    uint32_t grid = (uint32_t)((len + BLOCK - 1) / BLOCK);
+    hipLaunchKernelGGL((combine_columns_kernel<D>), dim3(grid), dim3(BLOCK), 0, c.stream, cols, len, count, a, d_out,
+                       first > 0 ? 1 : 0);
+  }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+int combine_columns_device(int D, const uint32_t *d_cols, int ncols, uint64_t len, const uint32_t *coef,
+                           uint32_t *d_out) {
+  int status = ctx().require();
+  if (status) return status;
+  ctx().prof_begin("combine_columns", 0, len * (4 * (uint64_t)ncols + 4 * (uint64_t)D));
+  status = D == 4 ? combine_launch<4>(d_cols, ncols, len, coef, d_out) : combine_launch<8>(d_cols, ncols, len, coef, d_out);
+  ctx().prof_end();
+  return status;
+}
+
 // ------------------------------------------------------------------ Merkle trees
 // LEAF-DIGEST (src/pcs.lisp:44-52) of leaf l of ncols codewords: one row of 4 symbols per column,
 // rows hashed 64 at a time and chained h = BLAKE3(h || d).

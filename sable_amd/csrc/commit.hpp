@@ -13,6 +13,10 @@ int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_
 // fold a codeword of 2m elements of degree D on level `level` of the 2^n_domain twiddle tables
 int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d_codeword, const uint32_t *r,
                    uint32_t *d_out);
+// COMBINE-COLUMNS (src/pcs.lisp:434-441): d_out[x] = sum_k coef_k * column_k[x]; ncols base columns of len values,
+// coefficients canonical on the host (ncols * D words), d_out len * D words
+int combine_columns_device(int D, const uint32_t *d_cols, int ncols, uint64_t len, const uint32_t *coef,
+                           uint32_t *d_out);
 // leaf digests and all Merkle levels (8-word digests, leaves first) of ncols codewords of
 // 2^(c+1) symbols; cap: the level max(0, log2(leaves) - 7), as bytes
 int merkle_commit_columns(const uint32_t *d_codewords, int ncols, int c, uint32_t *d_levels, uint8_t *cap,

@@ -154,3 +154,43 @@ def test_basefold_round_trip_beyond_the_oracle_sizes():
     with pytest.raises(sa.VerificationFailure):
         sa.basefold_verify(sa.Transcript("bf-large", 4, proof=tr.proof()), nv, rr, orc.ext_add(v, orc.base_to_ext(1, 8)))
     h.free()
+
+
+@pytest.mark.parametrize("d,ncols,length", [(8, 1, 16), (8, 2, 1 << 12), (8, 5, 1001), (4, 3, 4096), (8, 40, 512),
+                                            (4, 33, 7)])
+def test_combine_columns_matches_the_oracle(d, ncols, length):
+    """combine-columns (src/pcs.lisp:434-441): lengths that are not multiples of four and more columns than one
+    launch takes included."""
+    rng = np.random.default_rng(ncols * 1000 + length)
+    cols = rng.integers(0, P, (ncols, length), dtype=np.uint32)
+    cf = rng.integers(0, P, (ncols, d), dtype=np.uint32)
+    t = sa.Table.upload(cols.reshape(-1))
+    g = sa.combine_columns(t, ncols, cf)
+    assert same(g.download().reshape(length, d), orc.combine_columns(cols, cf))
+    g.free()
+    t.free()
+
+
+def test_combine_columns_feeds_basefold_at_size():
+    """Two base columns of 2^19 combined into the table BaseFold opens: the claim is the same combination of the
+    columns' own evaluations at the point (combine-columns is linear, as pcs.lisp:425-430 uses it), and the
+    verifier accepts exactly that claim."""
+    nv, ncols = 19, 2
+    rng = np.random.default_rng(1434)
+    cols = sa.Table.random(91, ncols << nv)
+    cf = rng.integers(0, P, (ncols, 8), dtype=np.uint32)
+    rr = rng.integers(0, P, (nv, 8), dtype=np.uint32)
+    g = sa.combine_columns(cols, ncols, cf)
+    host = cols.download().reshape(ncols, 1 << nv)
+    v = np.zeros(8, np.uint32)
+    for k in range(ncols):
+        col = sa.Table.upload(host[k])
+        y = sa.hypercube_sum(sa.Statement("t0", ["t0"]), nv, [col], 8, eq=rr)  # the column's MLE at the point
+        v = orc.ext_add(v, orc.ext_mul(cf[k], y))
+        col.free()
+    assert same(sa.hypercube_sum(sa.Statement("t0", ["t0"]), nv, [g], 8, eq=rr), v)
+    tr = sa.Transcript("bf-combined", 4)
+    qs, _, _ = sa.basefold_prove(tr, nv, rr, v, g)
+    assert sa.basefold_verify(sa.Transcript("bf-combined", 4, proof=tr.proof()), nv, rr, v) == qs
+    g.free()
+    cols.free()

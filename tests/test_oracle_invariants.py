@@ -297,3 +297,24 @@ def test_basefold_roundtrip(nv):
         forged[k].reshape(-1)[0] = (int(forged[k].reshape(-1)[0]) + 1) % P
         with pytest.raises(orc.VerificationFailure):
             orc.basefold_verify(orc.Transcript("bf", 4, proof=orc.encode_messages(forged)), nv, rr, v)
+
+
+def test_combine_columns_from_the_definition():
+    """combine-columns (src/pcs.lisp:434-441) against an independent big-integer evaluation of
+    g[x] = sum_k coefficient_k * column_k[x], coordinate by coordinate; unit coefficients give back a column
+    embedded in the extension; the map is linear in the coefficients."""
+    rng = np.random.default_rng(434)
+    for d, ncols, length in ((8, 1, 5), (8, 3, 17), (4, 6, 32)):
+        cols = rng.integers(0, P, (ncols, length), dtype=np.uint32)
+        cf = rng.integers(0, P, (ncols, d), dtype=np.uint32)
+        got = orc.combine_columns(cols, cf)
+        want = [[sum(int(cf[k][c]) * int(cols[k][x]) for k in range(ncols)) % P for c in range(d)] for x in range(length)]
+        assert got.tolist() == want
+        unit = np.zeros((ncols, d), np.uint32)
+        unit[ncols - 1, 0] = 1
+        only = orc.combine_columns(cols, unit)
+        assert only[:, 0].tolist() == cols[ncols - 1].tolist() and not only[:, 1:].any()
+        cf2 = rng.integers(0, P, (ncols, d), dtype=np.uint32)
+        both = orc.combine_columns(cols, ((cf.astype(np.uint64) + cf2) % P).astype(np.uint32))
+        apart = (got.astype(np.uint64) + orc.combine_columns(cols, cf2)) % P
+        assert both.tolist() == apart.tolist()
