@@ -27,6 +27,10 @@
  *                                             every hash shape used, path checks against the cap,
  *                                             fold(encode(m)) = encode(fold(m)), final table = message
  *                                             folded at the challenges
+ *   combine-columns                           the definition evaluated with big integers coordinate by
+ *                                             coordinate (ext-scale is coordinate-wise, :ext vectors), unit
+ *                                             coefficients, linearity; its output opening under BaseFold to
+ *                                             the same combination of the columns' evaluations
  */
 #ifndef ORC_H
 #define ORC_H

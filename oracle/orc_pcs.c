@@ -1,5 +1,6 @@
 /* orc_pcs.c -- the commitment's data-parallel part: leaf digests, Merkle trees with caps, column
- * commitment and the BaseFold loop, restated from src/pcs.lisp:37-101, 271-304, 473-483, 569-657
+ * commitment, combine-columns and the BaseFold loop, restated from src/pcs.lisp:37-101, 271-304, 434-441, 473-483,
+ * 569-657
  * (test oracle; see orc.h).  The multi-unit bookkeeping around them (units, merge sets, segments,
  * point reductions, query verification) is not restated: BaseFold runs here on one class. */
 #include "orc.h"
