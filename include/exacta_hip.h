@@ -117,6 +117,10 @@ int exh_rs_fold(exh_table codeword, int degree_d, uint64_t m, int n_domain, int 
    takes them) and ncols coefficients of degree D (canonical, tower order); out: a new table of len elements */
 int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int degree_d, const uint32_t *coefficients,
                         exh_table *out);
+/* EQ-TABLE (src/field.lisp:354-363) of the point r (k coordinates of degree D, canonical), as a device table of
+   2^k elements: entry x = prod_b (x_b ? r_b : 1 - r_b).  What REDUCE-POINTS pairs with the combined columns
+   (src/pcs.lisp:352) before it calls PROVE */
+int exh_eq_table_device(int degree_d, int k, const uint32_t *r, exh_table *out);
 
 /* ---- LogUp-GKR layer reductions: FRACTION-TREES (src/gkr.lisp:149-170), one in-block layer:
    p, q: K * 2^(m+1) EXTs each; out_p, out_q: K * 2^m EXTs (children (b,x), (b,x+2^m)) */

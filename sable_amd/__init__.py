@@ -229,6 +229,14 @@ def eq_table(r, d):
     return out
 
 
+def eq_table_device(r, d):
+    """eq-table of the point r as a device Table of 2^len(r) EXTs."""
+    r = _u32(r).reshape(-1, d)
+    h = C.c_uint64()
+    check(load().exh_eq_table_device(d, len(r), _p(r), C.byref(h)))
+    return Table(h.value, d << len(r), d)
+
+
 # ------------------------------------------------------------------ sumcheck (src/sumcheck.lisp)
 def _opt(a, d):
     return None if a is None else _u32(a).reshape(-1, d)

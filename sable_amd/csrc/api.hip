@@ -319,6 +319,18 @@ int exh_eq_table(int D, int k, const uint32_t *r, uint32_t *out) {
   return OK;
 }
 
+int exh_eq_table_device(int D, int k, const uint32_t *r, exh_table *out) {
+  if ((D != 4 && D != 8) || k < 0 || k > 26 || (k > 0 && !r) || !out) {
+    set_error("invalid-parameter: eq table of k <= 26 coordinates of degree 4 or 8");
+    return E_PARAM;
+  }
+  int status = exh_table_alloc(((uint64_t)D) << k, D, out);
+  if (status) return status;
+  status = eq_table_device(D, k, r, table_of(*out)->ptr);
+  if (status) exh_table_free(*out);
+  return status;
+}
+
 // ------------------------------------------------------------------ transcript
 int exh_blake3(const uint8_t *in, uint64_t len, uint8_t *out, uint64_t out_len) {
   blake3_hash(in, len, out, out_len);

@@ -335,6 +335,48 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
 }
 
 // the weight tables of every round from the eq point's factors (or all-ones tables without one)
+// EQ-TABLE (src/field.lisp:354-363) of a point of k coordinates, left on the device: entry x is the product over
+// b of (x_b ? r_b : 1 - r_b).  The same kernel as the sessions' weight tables, over one table.
+int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  if (k == 0) {
+    uint32_t one[8] = {1, 0, 0, 0, 0, 0, 0, 0};
+    EXH_HIP(hipMemcpyAsync(d_out, one, (size_t)D * 4, hipMemcpyHostToDevice, c.stream));
+    EXH_HIP(hipStreamSynchronize(c.stream));
+    return OK;
+  }
+  std::vector<uint32_t> factors((size_t)2 * k * D);
+  for (int v = 0; v < k; v++)
+    for (int cc = 0; cc < D; cc++) {
+      uint32_t rv = r[(size_t)v * D + cc] % P;
+      factors[((size_t)v * 2) * D + cc] = to_mont(rv);
+      factors[((size_t)v * 2 + 1) * D + cc] = to_mont(fsub(cc == 0 ? 1u : 0u, rv));
+    }
+  uint32_t *d_factors = (uint32_t *)c.pool.alloc(factors.size() * 4);
+  if (!d_factors) {
+    set_error("device-out-of-memory: eq factors");
+    return E_NOMEM;
+  }
+  EXH_HIP(hipMemcpyAsync(d_factors, factors.data(), factors.size() * 4, hipMemcpyHostToDevice, c.stream));
+  EqTables eqt;
+  memset(&eqt, 0, sizeof(eqt));
+  eqt.count = 1, eqt.off[0] = 0, eqt.first[0] = 0, eqt.bits[0] = k;
+  const uint64_t total = (uint64_t)1 << k;
+  uint32_t grid = (uint32_t)((total + BLOCK - 1) / BLOCK);
+  if (D == 4)
+    hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors, d_out, total, nullptr,
+                       (uint64_t)0);
+  else
+    hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors, d_out, total, nullptr,
+                       (uint64_t)0);
+  EXH_HIP(hipGetLastError());
+  EXH_HIP(hipStreamSynchronize(c.stream));  // `factors` (pageable) and the pooled buffer are free to go after this
+  c.pool.release(d_factors);
+  return OK;
+}
+
 static uint64_t tail_pairs(int T, int D);
 
 int SumcheckSession::launch_setup() {

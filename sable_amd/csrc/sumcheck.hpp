@@ -20,6 +20,8 @@ struct KernelSet {  // the launchers generated for one statement and one degree 
   void (*launch_nodes)(const void *args, int pass, uint32_t grid, hipStream_t stream);
   int nodes_passes;  // launches of launch_nodes per round (0: not available)
 };
+// EQ-TABLE of k coordinates (canonical, host) into 2^k elements of device memory
+int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out);
 void register_kernels(const std::string &key, int D, KernelSet set);
 const KernelSet *find_kernels(const std::string &key, int D);
 

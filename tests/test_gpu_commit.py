@@ -194,3 +194,48 @@ def test_combine_columns_feeds_basefold_at_size():
     assert sa.basefold_verify(sa.Transcript("bf-combined", 4, proof=tr.proof()), nv, rr, v) == qs
     g.free()
     cols.free()
+
+
+@pytest.mark.parametrize("d,k", [(4, 0), (4, 1), (8, 5), (4, 12), (8, 9)])
+def test_eq_table_on_the_device(d, k):
+    rng = np.random.default_rng(k * 10 + d)
+    r = rng.integers(0, P, (k, d), dtype=np.uint32)
+    t = sa.eq_table_device(r, d)
+    assert same(t.download().reshape(1 << k, d), orc.eq_table(r, d))
+    t.free()
+
+
+def test_reduce_points_sumcheck_from_device_tables():
+    """The prover's side of reduce-points (src/pcs.lisp:333-362) from the entry points: per group of opening
+    points an eq table of the point and the columns combined with the group's F_p^4 coefficients, both built on
+    the device, then PROVE of (+ (* E0 G0) (* E1 G1)) with label "pcs-red" and degree 2.  Same proof bytes as the
+    oracle's composition of the same steps; the claim is the combination of the columns' evaluations, and the
+    verifier accepts it."""
+    c, ncols, d = 12, 3, 4
+    rng = np.random.default_rng(333)
+    cols = rng.integers(0, P, (ncols, 1 << c), dtype=np.uint32)
+    zs = [rng.integers(0, P, (c, d), dtype=np.uint32) for _ in range(2)]
+    cfs = [rng.integers(0, P, (ncols, d), dtype=np.uint32) for _ in range(2)]
+    form, names = "(+ (* e0 g0) (* e1 g1))", ["e0", "g0", "e1", "g1"]
+    dcols = sa.Table.upload(cols.reshape(-1))
+    dev, host = [], []
+    for z, cf in zip(zs, cfs):
+        dev += [sa.eq_table_device(z, d), sa.combine_columns(dcols, ncols, cf)]
+        host += [orc.eq_table(z, d), orc.combine_columns(cols, cf)]
+    tr, otr = sa.Transcript("red", d), orc.Transcript("red", d)
+    st, ost = sa.Statement(form, names), orc.Statement(form, names)
+    rho, finals, _ = sa.prove(tr, c, st, dev, label="pcs-red", degree=2)
+    want = orc.prove(otr, c, ost, host, label="pcs-red", degree=2)
+    assert tr.proof() == otr.proof() and same(rho, want[0]) and same(finals, want[1])
+    claim = np.zeros(d, np.uint32)
+    for z, cf in zip(zs, cfs):
+        for k in range(ncols):
+            lifted = np.zeros((1 << c, d), np.uint32)
+            lifted[:, 0] = cols[k]
+            claim = orc.ext_add(claim, orc.ext_mul(cf[k], orc.mle_eval(lifted, z, d)))
+    got_rho, reduced = sa.verify(sa.Transcript("red", d, proof=tr.proof()), c, st, claim, label="pcs-red", degree=2)
+    assert same(got_rho, rho)
+    assert sa.check_final(reduced, st, finals)
+    for t in dev:
+        t.free()
+    dcols.free()
