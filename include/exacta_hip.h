@@ -117,6 +117,11 @@ int exh_rs_fold(exh_table codeword, int degree_d, uint64_t m, int n_domain, int 
    takes them) and ncols coefficients of degree D (canonical, tower order); out: a new table of len elements */
 int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int degree_d, const uint32_t *coefficients,
                         exh_table *out);
+/* One class's share of a CROSS-ROUNDS round (src/pcs.lisp:485-512): DOT-PAIRS (:473-483) of its tables E and V
+   (EXT8s, the same even count) for the parities 0, 1, 2 at once -> out[3][8], and FOLD-TABLE (src/field.lisp:365-370)
+   of either by the round's challenge r (degree = the table's) -> a new table of half the length */
+int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out);
+int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out);
 /* EQ-TABLE (src/field.lisp:354-363) of the point r (k coordinates of degree D, canonical), as a device table of
    2^k elements: entry x = prod_b (x_b ? r_b : 1 - r_b).  What REDUCE-POINTS pairs with the combined columns
    (src/pcs.lisp:352) before it calls PROVE */

@@ -415,6 +415,15 @@ def rs_fold(codeword, twiddle_level, r):
     return out
 
 
+def dot_pairs(e, v):
+    """dot-pairs (src/pcs.lisp:473-483) of two tables of EXT8s for the parities 0, 1, 2: (3, 8)."""
+    e, v = _u32(e), _u32(v)
+    out = np.zeros((3, 8), np.uint32)
+    for parity in range(3):
+        lib().orc_dot_pairs(_p(e), _p(v), C.c_uint64(len(e)), parity, _p(out[parity]))
+    return out
+
+
 def combine_columns(columns, coefficients):
     """combine-columns (src/pcs.lisp:434-441): columns (ncols, len) base values, coefficients (ncols, D)."""
     cols, cf = _u32(columns), _u32(coefficients)

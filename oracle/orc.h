@@ -27,6 +27,8 @@
  *                                             every hash shape used, path checks against the cap,
  *                                             fold(encode(m)) = encode(fold(m)), final table = message
  *                                             folded at the challenges
+ *   dot-pairs, fold-table                     the BaseFold loop they serve (above); fold-table by the :mle vectors;
+ *                                             the round identity g(0) + g(1) of the folded tables = g(x)
  *   combine-columns                           the definition evaluated with big integers coordinate by
  *                                             coordinate (ext-scale is coordinate-wise, :ext vectors), unit
  *                                             coefficients, linearity; its output opening under BaseFold to
@@ -151,6 +153,9 @@ void orc_rs_brute_eval(const uint32_t *message, int n, uint32_t *out);
 /* fold a codeword of 2m elements of degree D (D = 1: base) on a twiddle level of m values */
 void orc_rs_fold(int D, uint64_t m, const uint32_t *codeword, const uint32_t *twiddle_level,
                  const uint32_t *r, uint32_t *out);
+/* DOT-PAIRS, src/pcs.lisp:473-483: sum over pairs of pick(e) pick(v) for two tables of len EXT8s; parity 0: even
+   entries, 1: odd entries, 2: 2 odd - even */
+void orc_dot_pairs(const uint32_t *e, const uint32_t *v, uint64_t len, int parity, uint32_t *out);
 /* COMBINE-COLUMNS, src/pcs.lisp:434-441 */
 void orc_combine_columns(int D, int ncols, uint64_t len, const uint32_t *columns, const uint32_t *coefficients,
                          uint32_t *out);

@@ -124,7 +124,7 @@ static void encode_ext(const uint32_t *table, int c, uint32_t *cw) {
 }
 
 /* DOT-PAIRS, src/pcs.lisp:473-483 */
-static void dot_pairs(const uint32_t *e, const uint32_t *v, uint64_t len, int parity, uint32_t *out) {
+void orc_dot_pairs(const uint32_t *e, const uint32_t *v, uint64_t len, int parity, uint32_t *out) {
   uint32_t acc[8] = {0}, a[8], b[8], t[8];
   for (uint64_t i = 0; i < len; i += 2) {
     const uint32_t *tabs[2] = {e, v};
@@ -182,7 +182,7 @@ int orc_basefold_prove(orc_tr *tr, int nv, const uint32_t *rr, const uint32_t *v
     uint64_t cur = len >> i;
     uint32_t ev[24];
     for (int parity = 0; parity < 3; parity++) /* a = prf * ysum = 0: every class has joined */
-      dot_pairs(tt, et, cur, parity, ev + 8 * parity);
+      orc_dot_pairs(tt, et, cur, parity, ev + 8 * parity);
     uint64_t dims[2] = {3, 8};
     if ((status = orc_tr_send(tr, ev, 2, dims, NULL))) goto done;
     uint32_t s[8];

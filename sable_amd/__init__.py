@@ -405,6 +405,21 @@ def combine_columns(columns, ncols, coefficients):
     return Table(h.value, length * d, d)
 
 
+def dot_pairs(e, v):
+    """dot-pairs of two Tables of EXT8s for the parities 0, 1, 2: (3, 8)."""
+    out = np.zeros((3, 8), np.uint32)
+    check(load().exh_dot_pairs(C.c_uint64(e.handle), C.c_uint64(v.handle), _p(out)))
+    return out
+
+
+def fold_table(table, r):
+    """fold-table of an extension Table by the challenge r -> Table of half the length."""
+    r = _u32(r)
+    h = C.c_uint64()
+    check(load().exh_fold_table(C.c_uint64(table.handle), _p(r), C.byref(h)))
+    return Table(h.value, table.n_u32 // 2, table.stride)
+
+
 def pcs_commit(tr, columns, ncols, c):
     """pcs-commit of one class: encode, leaf digests, Merkle levels; the cap is sent on the transcript."""
     hc, hl = C.c_uint64(), C.c_uint64()

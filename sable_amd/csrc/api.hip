@@ -598,6 +598,32 @@ int exh_rs_fold(exh_table codeword, int D, uint64_t m, int n_domain, int level, 
   return rs_fold_device(D, m, n_domain, level, cw->ptr, r, table_of(*out)->ptr);
 }
 
+int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out) {
+  DeviceTable *te = table_of(e), *tv = table_of(v);
+  if (!te || !tv) return E_PARAM;
+  if (!out || te->stride != 8 || tv->stride != 8 || te->n_u32 != tv->n_u32 || te->n_u32 < 16 || (te->n_u32 / 8) % 2) {
+    set_error("invalid-parameter: dot-pairs takes two tables of the same even number of EXT8s");
+    return E_PARAM;
+  }
+  return dot_pairs_device(te->ptr, tv->ptr, te->n_u32 / 8, out);
+}
+
+int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out) {
+  DeviceTable *t = table_of(table);
+  if (!t) return E_PARAM;
+  const int D = t->stride;
+  if (!r || !out || (D != 4 && D != 8) || t->n_u32 < (uint64_t)2 * D || (t->n_u32 / D) % 2) {
+    set_error("invalid-parameter: fold-table takes an even number of extension elements");
+    return E_PARAM;
+  }
+  const uint64_t len = t->n_u32 / D;
+  int status = exh_table_alloc(len / 2 * D, D, out);
+  if (status) return status;
+  status = fold_table_device(D, t->ptr, len, r, table_of(*out)->ptr);
+  if (status) exh_table_free(*out);
+  return status;
+}
+
 int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int D, const uint32_t *coefficients, exh_table *out) {
   DeviceTable *cols = table_of(columns);
   if (!cols) return E_PARAM;

@@ -584,15 +584,55 @@ __global__ __launch_bounds__(BLOCK) void sum_columns_kernel(const uint32_t *part
   }
 }
 
-// FOLD-TABLE (src/field.lisp:365-370) of EXT8 tables
-__global__ __launch_bounds__(BLOCK) void fold8_kernel(const uint32_t *in, uint32_t *out, uint64_t n_out,
-                                                      RoundArgs<8> args) {
+// DOT-PAIRS of two device tables of len EXT8s for the three parities: out[parity][8] on the host (one wait)
+int dot_pairs_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uint32_t *out) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  const uint64_t n_pairs = len / 2;
+  const uint32_t grid = (uint32_t)std::min<uint64_t>((n_pairs + BLOCK - 1) / BLOCK, 1024);
+  uint32_t *scratch = (uint32_t *)c.pool.alloc(((size_t)grid * 24 + 24) * 4);
+  if (!scratch) {
+    set_error("device-out-of-memory: dot-pairs partial sums");
+    return E_NOMEM;
+  }
+  uint32_t *sums = scratch + (size_t)grid * 24;
+  hipLaunchKernelGGL(dot_pairs_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, d_e, d_v, n_pairs, scratch);
+  hipLaunchKernelGGL(sum_columns_kernel, dim3(24), dim3(BLOCK), 0, c.stream, scratch, grid, 24u, sums);
+  EXH_HIP(hipMemcpyAsync(out, sums, 96, hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  c.pool.release(scratch);
+  return OK;
+}
+
+// FOLD-TABLE (src/field.lisp:365-370) of extension tables
+template <int D>
+__global__ __launch_bounds__(BLOCK) void fold_table_kernel(const uint32_t *in, uint32_t *out, uint64_t n_out,
+                                                           RoundArgs<D> args) {
   uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
   if (i >= n_out) return;
-  Ext<8> r;
+  Ext<D> r;
 #pragma unroll
-  for (int c = 0; c < 8; c++) r.c[c] = args.r_mont[c];
-  store_ext<8>(out + i * 8, fold_ext<8>(load_ext<8>(in + 2 * i * 8), load_ext<8>(in + (2 * i + 1) * 8), r));
+  for (int c = 0; c < D; c++) r.c[c] = args.r_mont[c];
+  store_ext<D>(out + i * D, fold_ext<D>(load_ext<D>(in + 2 * i * D), load_ext<D>(in + (2 * i + 1) * D), r));
+}
+template <int D>
+static void fold_table_launch(const uint32_t *in, uint32_t *out, uint64_t n_out, const uint32_t *r) {
+  RoundArgs<D> a;
+  memset(&a, 0, sizeof(a));
+  for (int k = 0; k < D; k++) a.r_mont[k] = to_mont(r[k] % P);
+  uint32_t grid = (uint32_t)((n_out + BLOCK - 1) / BLOCK);
+  hipLaunchKernelGGL(fold_table_kernel<D>, dim3(grid), dim3(BLOCK), 0, ctx().stream, in, out, n_out, a);
+}
+int fold_table_device(int D, const uint32_t *d_in, uint64_t len, const uint32_t *r, uint32_t *d_out) {
+  int status = ctx().require();
+  if (status) return status;
+  if (D == 4)
+    fold_table_launch<4>(d_in, d_out, len / 2, r);
+  else
+    fold_table_launch<8>(d_in, d_out, len / 2, r);
+  EXH_HIP(hipGetLastError());
+  return OK;
 }
 
 // EXT8 table (entries x 8) <-> 8 coordinate columns, for ENCODE-EXT (src/pcs.lisp:569-575)
@@ -740,8 +780,8 @@ int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v
     memset(&a, 0, sizeof(a));
     for (int k = 0; k < 8; k++) a.r_mont[k] = to_mont(x[k]);
     uint32_t gfold = (uint32_t)((n_pairs + BLOCK - 1) / BLOCK);
-    hipLaunchKernelGGL(fold8_kernel, dim3(gfold), dim3(BLOCK), 0, c.stream, tt, tt2, n_pairs, a);
-    hipLaunchKernelGGL(fold8_kernel, dim3(gfold), dim3(BLOCK), 0, c.stream, et, et2, n_pairs, a);
+    hipLaunchKernelGGL(fold_table_kernel<8>, dim3(gfold), dim3(BLOCK), 0, c.stream, tt, tt2, n_pairs, a);
+    hipLaunchKernelGGL(fold_table_kernel<8>, dim3(gfold), dim3(BLOCK), 0, c.stream, et, et2, n_pairs, a);
     std::swap(tt, tt2);
     std::swap(et, et2);
     if ((status = rs_fold_launch(8, cur, dom->tw_inv2 + dom->off[i], cw, x, cw2))) return status;

@@ -13,6 +13,10 @@ int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_
 // fold a codeword of 2m elements of degree D on level `level` of the 2^n_domain twiddle tables
 int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d_codeword, const uint32_t *r,
                    uint32_t *d_out);
+// DOT-PAIRS (src/pcs.lisp:473-483) of two device tables of len EXT8s, parities 0, 1, 2 -> out[3][8] (host)
+int dot_pairs_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uint32_t *out);
+// FOLD-TABLE (src/field.lisp:365-370): d_out[i] = in[2i] + r (in[2i+1] - in[2i]) for len extension elements
+int fold_table_device(int D, const uint32_t *d_in, uint64_t len, const uint32_t *r, uint32_t *d_out);
 // COMBINE-COLUMNS (src/pcs.lisp:434-441): d_out[x] = sum_k coef_k * column_k[x]; ncols base columns of len values,
 // coefficients canonical on the host (ncols * D words), d_out len * D words
 int combine_columns_device(int D, const uint32_t *d_cols, int ncols, uint64_t len, const uint32_t *coef,

@@ -239,3 +239,41 @@ def test_reduce_points_sumcheck_from_device_tables():
     for t in dev:
         t.free()
     dcols.free()
+
+
+@pytest.mark.parametrize("length", [2, 64, 1 << 12])
+def test_dot_pairs_and_fold_table_match_the_oracle(length):
+    """One class's share of a cross-rounds round (src/pcs.lisp:473-512): the three parity sums and the folds."""
+    rng = np.random.default_rng(length)
+    e = rng.integers(0, P, (length, 8), dtype=np.uint32)
+    v = rng.integers(0, P, (length, 8), dtype=np.uint32)
+    x = rng.integers(0, P, 8, dtype=np.uint32)
+    te, tv = sa.Table.upload(e), sa.Table.upload(v)
+    assert same(sa.dot_pairs(te, tv), orc.dot_pairs(e, v))
+    fe = sa.fold_table(te, x)
+    assert same(fe.download().reshape(-1, 8), orc.fold_table(e, x))
+    q = rng.integers(0, P, (length, 4), dtype=np.uint32)
+    x4 = rng.integers(0, P, 4, dtype=np.uint32)
+    tq = sa.Table.upload(q)
+    fq = sa.fold_table(tq, x4)
+    assert same(fq.download().reshape(-1, 4), orc.fold_table(q, x4))
+    for t in (te, tv, fe, tq, fq):
+        t.free()
+
+
+def test_cross_round_identity_at_size():
+    """At 2^20 entries per table, beyond what the oracle runs in seconds: the round's three sums are g(0), g(1), g(2)
+    of the quadratic g(X) = sum_i E_i(X) V_i(X), so after folding both tables by x the next round's g(0) + g(1) is
+    g(x) by Lagrange (the check of src/pcs.lisp:502-506), and two rounds chain."""
+    length = 1 << 20
+    rng = np.random.default_rng(20)
+    e, v = sa.Table.random(501, length, 8), sa.Table.random(502, length, 8)
+    for _ in range(2):
+        ev = sa.dot_pairs(e, v)
+        x = rng.integers(0, P, 8, dtype=np.uint32)
+        e2, v2 = sa.fold_table(e, x), sa.fold_table(v, x)
+        nxt = sa.dot_pairs(e2, v2)
+        assert same(orc.ext_add(nxt[0], nxt[1]), orc.lagrange(ev, x))
+        e.free(), v.free()
+        e, v = e2, v2
+    e.free(), v.free()
