@@ -27,7 +27,7 @@
  *                                             every hash shape used, path checks against the cap,
  *                                             fold(encode(m)) = encode(fold(m)), final table = message
  *                                             folded at the challenges
- *   dot-pairs, fold-table                     the BaseFold loop they serve (above); fold-table by the :mle vectors;
+ *   dot-pairs, fold-table                     their definitions in an independent pure-Python field on small tables;
  *                                             the round identity g(0) + g(1) of the folded tables = g(x)
  *   combine-columns                           the definition evaluated with big integers coordinate by
  *                                             coordinate (ext-scale is coordinate-wise, :ext vectors), unit

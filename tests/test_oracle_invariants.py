@@ -318,3 +318,25 @@ def test_combine_columns_from_the_definition():
         both = orc.combine_columns(cols, ((cf.astype(np.uint64) + cf2) % P).astype(np.uint32))
         apart = (got.astype(np.uint64) + orc.combine_columns(cols, cf2)) % P
         assert both.tolist() == apart.tolist()
+
+
+def test_dot_pairs_and_fold_table_from_the_definition():
+    """dot-pairs (src/pcs.lisp:473-483) and fold-table (src/field.lisp:365-370) against the independent
+    pure-Python field: the three picks (even, odd, 2 odd - even) and entry + r (next - entry)."""
+    rng = np.random.default_rng(473)
+    for length in (2, 6):
+        e = rng.integers(0, P, (length, 8), dtype=np.uint32)
+        v = rng.integers(0, P, (length, 8), dtype=np.uint32)
+        picks = [lambda t, i: t[i], lambda t, i: t[i + 1],
+                 lambda t, i: pf.sub(pf.scale(t[i + 1], 2), t[i])]
+        el, vl = [list(map(int, row)) for row in e], [list(map(int, row)) for row in v]
+        want = []
+        for pick in picks:
+            total = [0] * 8
+            for i in range(0, length, 2):
+                total = pf.add(total, pf.mul(pick(el, i), pick(vl, i)))
+            want.append(total)
+        assert orc.dot_pairs(e, v).tolist() == want
+        r = [int(x) for x in rng.integers(0, P, 8, dtype=np.uint32)]
+        folded = [pf.add(el[i], pf.mul(r, pf.sub(el[i + 1], el[i]))) for i in range(0, length, 2)]
+        assert orc.fold_table(e, np.array(r, np.uint32)).tolist() == folded
