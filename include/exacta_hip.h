@@ -122,6 +122,9 @@ int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int degree_d
    of either by the round's challenge r (degree = the table's) -> a new table of half the length */
 int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out);
 int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out);
+/* The opening's table per class (src/pcs.lisp:709-716), one unit at a time: out[x] = h[x] + scale * column[x]
+   over extension tables of one shape; h = 0 stands for the table of zeros the sum starts from */
+int exh_table_scale_add(exh_table h, const uint32_t *scale, exh_table column, exh_table *out);
 /* EQ-TABLE (src/field.lisp:354-363) of the point r (k coordinates of degree D, canonical), as a device table of
    2^k elements: entry x = prod_b (x_b ? r_b : 1 - r_b).  What REDUCE-POINTS pairs with the combined columns
    (src/pcs.lisp:352) before it calls PROVE */

@@ -424,6 +424,13 @@ def dot_pairs(e, v):
     return out
 
 
+def scale_add(h, scale, column):
+    """h + scale * column over extension tables (src/pcs.lisp:709-716): a new array."""
+    h, scale, column = _u32(h).copy(), _u32(scale), _u32(column)
+    lib().orc_scale_add(len(scale), C.c_uint64(len(h)), _p(scale), _p(column), _p(h))
+    return h
+
+
 def combine_columns(columns, coefficients):
     """combine-columns (src/pcs.lisp:434-441): columns (ncols, len) base values, coefficients (ncols, D)."""
     cols, cf = _u32(columns), _u32(coefficients)

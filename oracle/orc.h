@@ -27,7 +27,7 @@
  *                                             every hash shape used, path checks against the cap,
  *                                             fold(encode(m)) = encode(fold(m)), final table = message
  *                                             folded at the challenges
- *   dot-pairs, fold-table                     their definitions in an independent pure-Python field on small tables;
+ *   dot-pairs, fold-table, scale-add          their definitions in an independent pure-Python field on small tables;
  *                                             the round identity g(0) + g(1) of the folded tables = g(x)
  *   combine-columns                           the definition evaluated with big integers coordinate by
  *                                             coordinate (ext-scale is coordinate-wise, :ext vectors), unit
@@ -156,6 +156,8 @@ void orc_rs_fold(int D, uint64_t m, const uint32_t *codeword, const uint32_t *tw
 /* DOT-PAIRS, src/pcs.lisp:473-483: sum over pairs of pick(e) pick(v) for two tables of len EXT8s; parity 0: even
    entries, 1: odd entries, 2: 2 odd - even */
 void orc_dot_pairs(const uint32_t *e, const uint32_t *v, uint64_t len, int parity, uint32_t *out);
+/* h[x] += scale * column[x], the per-class table of the opening (src/pcs.lisp:709-716) */
+void orc_scale_add(int D, uint64_t len, const uint32_t *scale, const uint32_t *column, uint32_t *h);
 /* COMBINE-COLUMNS, src/pcs.lisp:434-441 */
 void orc_combine_columns(int D, int ncols, uint64_t len, const uint32_t *columns, const uint32_t *coefficients,
                          uint32_t *out);

@@ -348,3 +348,13 @@ void orc_combine_columns(int D, int ncols, uint64_t len, const uint32_t *columns
     memcpy(out + x * D, g, D * sizeof(uint32_t));
   }
 }
+
+/* the opening's table per class, src/pcs.lisp:709-716: h[x] <- h[x] + scale * column[x] over EXT8s (one call
+   per unit or pulled unit of the class, starting from zeros) */
+void orc_scale_add(int D, uint64_t len, const uint32_t *scale, const uint32_t *column, uint32_t *h) {
+  for (uint64_t x = 0; x < len; x++) {
+    uint32_t t[ORC_MAXD];
+    orc_ext_mul(D, scale, column + x * D, t);
+    orc_ext_add(D, h + x * D, t, h + x * D);
+  }
+}

@@ -405,6 +405,14 @@ def combine_columns(columns, ncols, coefficients):
     return Table(h.value, length * d, d)
 
 
+def scale_add(h, scale, column):
+    """h + scale * column over extension Tables of one shape (h None: zeros) -> a new Table."""
+    out = C.c_uint64()
+    check(load().exh_table_scale_add(C.c_uint64(h.handle if h is not None else 0), _p(_u32(scale)),
+                                     C.c_uint64(column.handle), C.byref(out)))
+    return Table(out.value, column.n_u32, column.stride)
+
+
 def dot_pairs(e, v):
     """dot-pairs of two Tables of EXT8s for the parities 0, 1, 2: (3, 8)."""
     out = np.zeros((3, 8), np.uint32)

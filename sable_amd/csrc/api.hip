@@ -598,6 +598,21 @@ int exh_rs_fold(exh_table codeword, int D, uint64_t m, int n_domain, int level, 
   return rs_fold_device(D, m, n_domain, level, cw->ptr, r, table_of(*out)->ptr);
 }
 
+int exh_table_scale_add(exh_table h, const uint32_t *scale, exh_table column, exh_table *out) {
+  DeviceTable *tc = table_of(column), *th = h ? table_of(h) : nullptr;
+  if (!tc || (h && !th)) return E_PARAM;
+  const int D = tc->stride;
+  if (!scale || !out || (D != 4 && D != 8) || tc->n_u32 < (uint64_t)D || (th && (th->stride != D || th->n_u32 != tc->n_u32))) {
+    set_error("invalid-parameter: scale-add takes extension tables of one shape");
+    return E_PARAM;
+  }
+  int status = exh_table_alloc(tc->n_u32, D, out);
+  if (status) return status;
+  status = scale_add_device(D, th ? th->ptr : nullptr, tc->ptr, tc->n_u32 / D, scale, table_of(*out)->ptr);
+  if (status) exh_table_free(*out);
+  return status;
+}
+
 int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out) {
   DeviceTable *te = table_of(e), *tv = table_of(v);
   if (!te || !tv) return E_PARAM;

@@ -584,6 +584,41 @@ __global__ __launch_bounds__(BLOCK) void sum_columns_kernel(const uint32_t *part
   }
 }
 
+// out[x] = h[x] + scale * column[x] over extension tables (h null: zero): the opening's table per class is the
+// sum of its units' columns, each times the unit's scalar (src/pcs.lisp:709-716)
+template <int D>
+__global__ __launch_bounds__(BLOCK) void scale_add_kernel(const uint32_t *h, const uint32_t *column, uint32_t *out,
+                                                          uint64_t len, RoundArgs<D> args) {
+  uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (i >= len) return;
+  Ext<D> sc;
+#pragma unroll
+  for (int c = 0; c < D; c++) sc.c[c] = args.r_mont[c];
+  Ext<D> v = ext_mul_mont<D>(sc, load_ext<D>(column + i * D));
+  if (h) v = ext_add<D>(v, load_ext<D>(h + i * D));
+  store_ext<D>(out + i * D, v);
+}
+template <int D>
+static void scale_add_launch(const uint32_t *h, const uint32_t *column, uint32_t *out, uint64_t len,
+                             const uint32_t *scale) {
+  RoundArgs<D> a;
+  memset(&a, 0, sizeof(a));
+  for (int k = 0; k < D; k++) a.r_mont[k] = to_mont(scale[k] % P);
+  uint32_t grid = (uint32_t)((len + BLOCK - 1) / BLOCK);
+  hipLaunchKernelGGL(scale_add_kernel<D>, dim3(grid), dim3(BLOCK), 0, ctx().stream, h, column, out, len, a);
+}
+int scale_add_device(int D, const uint32_t *d_h, const uint32_t *d_column, uint64_t len, const uint32_t *scale,
+                     uint32_t *d_out) {
+  int status = ctx().require();
+  if (status) return status;
+  if (D == 4)
+    scale_add_launch<4>(d_h, d_column, d_out, len, scale);
+  else
+    scale_add_launch<8>(d_h, d_column, d_out, len, scale);
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
 // DOT-PAIRS of two device tables of len EXT8s for the three parities: out[parity][8] on the host (one wait)
 int dot_pairs_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uint32_t *out) {
   Context &c = ctx();

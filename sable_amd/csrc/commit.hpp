@@ -17,6 +17,9 @@ int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d
 int dot_pairs_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uint32_t *out);
 // FOLD-TABLE (src/field.lisp:365-370): d_out[i] = in[2i] + r (in[2i+1] - in[2i]) for len extension elements
 int fold_table_device(int D, const uint32_t *d_in, uint64_t len, const uint32_t *r, uint32_t *d_out);
+// d_out[x] = d_h[x] (null: zero) + scale * d_column[x] over len extension elements (src/pcs.lisp:709-716)
+int scale_add_device(int D, const uint32_t *d_h, const uint32_t *d_column, uint64_t len, const uint32_t *scale,
+                     uint32_t *d_out);
 // COMBINE-COLUMNS (src/pcs.lisp:434-441): d_out[x] = sum_k coef_k * column_k[x]; ncols base columns of len values,
 // coefficients canonical on the host (ncols * D words), d_out len * D words
 int combine_columns_device(int D, const uint32_t *d_cols, int ncols, uint64_t len, const uint32_t *coef,

@@ -277,3 +277,23 @@ def test_cross_round_identity_at_size():
         e.free(), v.free()
         e, v = e2, v2
     e.free(), v.free()
+
+
+@pytest.mark.parametrize("d,length", [(8, 1), (8, 1000), (4, 4096)])
+def test_scale_add_builds_the_class_table(d, length):
+    """src/pcs.lisp:709-716: the class's table is the sum over its units of scalar * column, from zeros."""
+    rng = np.random.default_rng(709 + length)
+    cols = [rng.integers(0, P, (length, d), dtype=np.uint32) for _ in range(3)]
+    scs = [rng.integers(0, P, d, dtype=np.uint32) for _ in range(3)]
+    want = np.zeros((length, d), np.uint32)
+    h = None
+    for col, sc in zip(cols, scs):
+        want = orc.scale_add(want, sc, col)
+        t = sa.Table.upload(col)
+        nxt = sa.scale_add(h, sc, t)
+        t.free()
+        if h is not None:
+            h.free()
+        h = nxt
+    assert same(h.download().reshape(length, d), want)
+    h.free()

@@ -340,3 +340,12 @@ def test_dot_pairs_and_fold_table_from_the_definition():
         r = [int(x) for x in rng.integers(0, P, 8, dtype=np.uint32)]
         folded = [pf.add(el[i], pf.mul(r, pf.sub(el[i + 1], el[i]))) for i in range(0, length, 2)]
         assert orc.fold_table(e, np.array(r, np.uint32)).tolist() == folded
+
+
+def test_scale_add_from_the_definition():
+    rng = np.random.default_rng(709)
+    h = rng.integers(0, P, (5, 8), dtype=np.uint32)
+    col = rng.integers(0, P, (5, 8), dtype=np.uint32)
+    sc = rng.integers(0, P, 8, dtype=np.uint32)
+    want = [pf.add(list(map(int, h[x])), pf.mul(list(map(int, sc)), list(map(int, col[x])))) for x in range(5)]
+    assert orc.scale_add(h, sc, col).tolist() == want
