@@ -16,6 +16,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <stddef.h>
 #include <type_traits>
 
 #include "dev_transcript.cuh"
@@ -915,10 +916,19 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   }
   if (args.host_log && G == 1) {
     __syncthreads();
-    // every word through the L2 (this workgroup wrote some of them a moment ago, other launches the rest)
+    // every word through the L2 (this workgroup wrote some of them a moment ago, other launches the rest); of
+    // the logs only what the rounds filled: the head, points * D words of a round's message, D of its challenge
     const uint32_t *words = reinterpret_cast<const uint32_t *>(args.ctrl);
-    for (uint32_t u = tid; u < sizeof(Ctrl) / 4; u += BLOCK)
-      args.host_log[u] = __hip_atomic_load(words + u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    auto deliver = [&](uint32_t at) {
+      args.host_log[at] = __hip_atomic_load(words + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    const uint32_t all_rounds = args.first_round + args.rounds, mw = args.points * D;
+    for (uint32_t u = tid; u < offsetof(Ctrl, msg) / 4; u += BLOCK) deliver(u);
+    for (uint32_t u = tid; u < all_rounds * mw; u += BLOCK)
+      deliver((uint32_t)(offsetof(Ctrl, msg) / 4) + (u / mw) * (MAXPTS * 8) + u % mw);
+    for (uint32_t u = tid; u < all_rounds * D; u += BLOCK)
+      deliver((uint32_t)(offsetof(Ctrl, chal) / 4) + (u / D) * 8 + u % D);
+    for (uint32_t u = tid; u < (uint32_t)d.T * D; u += BLOCK) deliver((uint32_t)(offsetof(Ctrl, finals) / 4) + u);
     __threadfence_system();
     __syncthreads();
     if (tid == 0) {
