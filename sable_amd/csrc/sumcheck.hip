@@ -885,7 +885,8 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     // itself delivers the control block to pinned host memory
     const bool deliver = !c.profiling && (size >> ((folds_due > 0 ? 1 : 0) + (n - j))) == 1;
     if (deliver) {
-      host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = ++c.log_seq;
+      if (++c.log_seq == 0) ++c.log_seq;  // 0 is what the flag is reset to
+      host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = c.log_seq;
       reinterpret_cast<volatile uint32_t *>(down)[ctrl_words] = 0;
     }
     status = launch_tail(j, n - j, 1, folds_due > 0);
