@@ -25,10 +25,16 @@ struct EqTables {
 // (both set-up kernels also clear the totals of the grid launch of LDS-resident slices: the first launch of a
 // session is the one place that comes before every use)
 template <int D>
-__global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const uint32_t *factors, uint32_t *out,
-                                                          uint64_t total, uint32_t *zero, uint64_t zero_words) {
+__global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const uint32_t *factors,
+                                                          uint32_t n_factor_words, uint32_t *out, uint64_t total,
+                                                          uint32_t *zero, uint64_t zero_words) {
   uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
   for (uint64_t z = gid; z < zero_words; z += (uint64_t)gridDim.x * BLOCK) zero[z] = 0;
+  // every variable's two factors into LDS first: an entry is a chain of up to `bits` products, and a load from
+  // memory inside each link is most of the kernel's time
+  __shared__ uint32_t lds_factors[2 * MAXROUNDS * 8];
+  for (uint32_t u = threadIdx.x; u < n_factor_words; u += BLOCK) lds_factors[u] = factors[u];
+  __syncthreads();
   if (gid >= total) return;
   int k = 0;
   uint64_t start = 0;
@@ -39,8 +45,11 @@ __global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const u
   uint64_t x = gid - start;
   Ext<D> e = ext_lift<D>(1);
   for (int b = 0; b < tabs.bits[k]; b++) {
-    const uint32_t *f = factors + ((size_t)(tabs.first[k] + b) * 2 + (((x >> b) & 1) ? 0 : 1)) * D;
-    e = ext_mul_mont<D>(e, load_ext<D>(f));
+    const uint32_t *f = lds_factors + ((size_t)(tabs.first[k] + b) * 2 + (((x >> b) & 1) ? 0 : 1)) * D;
+    Ext<D> fe;
+#pragma unroll
+    for (int c = 0; c < D; c++) fe.c[c] = f[c];
+    e = ext_mul_mont<D>(e, fe);
   }
   store_ext<D>(out + (tabs.off[k] + x) * D, e);
 }
@@ -366,11 +375,11 @@ int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out) {
   const uint64_t total = (uint64_t)1 << k;
   uint32_t grid = (uint32_t)((total + BLOCK - 1) / BLOCK);
   if (D == 4)
-    hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors, d_out, total, nullptr,
-                       (uint64_t)0);
+    hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors,
+                       (uint32_t)factors.size(), d_out, total, nullptr, (uint64_t)0);
   else
-    hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors, d_out, total, nullptr,
-                       (uint64_t)0);
+    hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors,
+                       (uint32_t)factors.size(), d_out, total, nullptr, (uint64_t)0);
   EXH_HIP(hipGetLastError());
   EXH_HIP(hipStreamSynchronize(c.stream));  // `factors` (pageable) and the pooled buffer are free to go after this
   c.pool.release(d_factors);
@@ -394,11 +403,11 @@ int SumcheckSession::launch_setup() {
     // tables are laid out in launch order, so thread gid maps to table k by running sums; the
     // offsets themselves may skip other regions, so they are taken from eqt.off
     if (D == 4)
-      hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq,
-                         zero, zero_words);
+      hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, (uint32_t)(2 * n * D), base,
+                         setup.total_eq, zero, zero_words);
     else
-      hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, base, setup.total_eq,
-                         zero, zero_words);
+      hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, (uint32_t)(2 * n * D), base,
+                         setup.total_eq, zero, zero_words);
     cleared = zero_words > 0;
     zero_words = 0;
   }
