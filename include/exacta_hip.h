@@ -108,6 +108,13 @@ int exh_rs_encode(exh_table messages, int ncols, int c, exh_table *codewords);
    symbols 4l..4l+3 of every column; levels (optional handle out) holds all levels, leaves first, as
    8-word digests; cap: 32 * cap_rows bytes */
 int exh_merkle_commit(exh_table codewords, int ncols, int c, exh_table *levels, uint8_t *cap, uint64_t *cap_rows);
+/* OPEN-QUERIES' gathers for one (unit, class) (src/pcs.lisp:721-734): out_leaves[count][ncols][4] = LEAF-ROWS
+   (src/pcs.lisp:275-277) of leaf leaves[q] < 2^(c-1), the array FIELD-ARRAY-OF-LEAVES (:659-665) records; with
+   levels (else 0), out_paths[count][depth][32 bytes] = PATH (src/pcs.lisp:79-84) of the same leaves up to the
+   cap level depth = CAP-LEVEL(2^(c-1)) (src/pcs.lisp:57-59), written to out_depth.  The caller derives leaves[q]
+   from the query index as (ash q (- c nv)) and records both in the transcript. */
+int exh_open_queries(exh_table codewords, int ncols, int c, exh_table levels, const uint64_t *leaves, int count,
+                     uint32_t *out_leaves, uint8_t *out_paths, int *out_depth);
 /* RS:FOLD of an extension codeword of 2m elements of degree D on twiddle level `level` of the
    2^n_domain tables (src/rs.lisp:93-101) */
 int exh_rs_fold(exh_table codeword, int degree_d, uint64_t m, int n_domain, int level, const uint32_t *r,

@@ -431,6 +431,25 @@ def scale_add(h, scale, column):
     return h
 
 
+def open_queries(codewords, c, levels, leaves):
+    """open-queries' data for one (unit, class) (src/pcs.lisp:721-734): codewords (ncols, 2^(c+1)); levels: the
+    bytes of all levels, leaves first, or None -> (leaves (Q, ncols, 4), paths (Q, depth, 32) bytes)."""
+    cw = _u32(codewords)
+    ncols = cw.shape[0]
+    idx = np.ascontiguousarray(leaves, np.uint64)
+    depth = cap_level(1 << (c - 1)) if levels is not None else 0
+    out = np.zeros((len(idx), ncols, 4), np.uint32)
+    paths = np.zeros((len(idx), depth, 32), np.uint8)
+    lv = None
+    if levels is not None:  # a list of levels (as commit_columns returns them) or their bytes
+        lv = (np.concatenate([np.ascontiguousarray(l, np.uint8).reshape(-1) for l in levels])
+              if isinstance(levels, (list, tuple)) else np.frombuffer(bytes(levels), np.uint8).copy())
+    got = lib().orc_open_queries(_p(cw), ncols, c, lv.ctypes.data_as(C.c_void_p) if lv is not None else None,
+                                 idx.ctypes.data_as(C.c_void_p), len(idx), _p(out), paths.ctypes.data_as(C.c_void_p))
+    assert got == depth
+    return out, paths
+
+
 def combine_columns(columns, coefficients):
     """combine-columns (src/pcs.lisp:434-441): columns (ncols, len) base values, coefficients (ncols, D)."""
     cols, cf = _u32(columns), _u32(coefficients)

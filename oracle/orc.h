@@ -29,6 +29,8 @@
  *                                             folded at the challenges
  *   dot-pairs, fold-table, scale-add          their definitions in an independent pure-Python field on small tables;
  *                                             the round identity g(0) + g(1) of the folded tables = g(x)
+ *   open-queries (leaves, paths)              numpy indexing of the codewords by the definition; every opened leaf,
+ *                                             hashed and walked up its path, lands on the committed cap
  *   combine-columns                           the definition evaluated with big integers coordinate by
  *                                             coordinate (ext-scale is coordinate-wise, :ext vectors), unit
  *                                             coefficients, linearity; its output opening under BaseFold to
@@ -219,6 +221,9 @@ int orc_cap_level(uint64_t leaves);
 void orc_merkle_levels(const uint8_t *leaves, uint64_t nleaves, uint8_t *out);
 int orc_check_path(const uint8_t h[32], const uint8_t *path, int depth, uint64_t i,
                    const uint8_t *cap);
+/* OPEN-QUERIES' leaves and paths of one (unit, class), src/pcs.lisp:721-734; returns the paths' depth */
+int orc_open_queries(const uint32_t *codewords, int ncols, int c, const uint8_t *levels, const uint64_t *leaves,
+                     int count, uint32_t *out_leaves, uint8_t *out_paths);
 /* commit NCOLS columns of 2^c base values: codewords (ncols * 2^(c+1)), leaf digests (2^(c-1) * 32
    bytes), all tree levels, and the cap; returns the cap's row count */
 uint64_t orc_commit_columns(const uint32_t *const *columns, int ncols, int c, uint32_t *codewords,

@@ -358,3 +358,26 @@ void orc_scale_add(int D, uint64_t len, const uint32_t *scale, const uint32_t *c
     orc_ext_add(D, h + x * D, t, h + x * D);
   }
 }
+
+/* OPEN-QUERIES' recorded data for one (unit, class), src/pcs.lisp:721-734: the (Q, rows, 4) array of the queried
+   leaves (LEAF-ROWS :275-277 through FIELD-ARRAY-OF-LEAVES :659-665) and, with LEVELS (all levels, leaves
+   first, as orc_merkle_levels lays them out), each leaf's PATH (:79-84) up to the cap level.  Returns that depth. */
+int orc_open_queries(const uint32_t *codewords, int ncols, int c, const uint8_t *levels, const uint64_t *leaves,
+                     int count, uint32_t *out_leaves, uint8_t *out_paths) {
+  const uint64_t nleaves = (uint64_t)1 << (c - 1), cw_len = (uint64_t)1 << (c + 1);
+  const int depth = levels ? orc_cap_level(nleaves) : 0;
+  for (int q = 0; q < count; q++) {
+    for (int k = 0; k < ncols; k++)
+      for (int sym = 0; sym < 4; sym++)
+        out_leaves[((size_t)q * ncols + k) * 4 + sym] = codewords[(uint64_t)k * cw_len + 4 * leaves[q] + sym];
+    uint64_t i = leaves[q], level_size = nleaves;
+    const uint8_t *level = levels;
+    for (int l = 0; l < depth; l++) {
+      memcpy(out_paths + ((size_t)q * depth + l) * 32, level + (i ^ 1) * 32, 32);
+      level += level_size * 32;
+      level_size >>= 1;
+      i >>= 1;
+    }
+  }
+  return depth;
+}

@@ -386,6 +386,21 @@ def merkle_commit(codewords, ncols, c, want_levels=True):
     return levels, cap[:rows.value].copy()
 
 
+def open_queries(codewords, ncols, c, levels, leaves):
+    """open-queries' gathers for one (unit, class): the queried leaves' rows (Q, ncols, 4) and, with the levels
+    Table of merkle_commit, their paths up to the cap level (Q, depth, 32) bytes (else depth 0)."""
+    idx = np.ascontiguousarray(leaves, np.uint64)
+    nleaves = 1 << (c - 1)
+    max_depth = max(0, nleaves.bit_length() - 1)
+    out = np.zeros((len(idx), ncols, 4), np.uint32)
+    paths = np.zeros((len(idx), max_depth, 32), np.uint8)
+    depth = C.c_int()
+    check(load().exh_open_queries(C.c_uint64(codewords.handle), ncols, c, C.c_uint64(levels.handle if levels else 0),
+                                  idx.ctypes.data_as(C.POINTER(C.c_uint64)), len(idx), _p(out),
+                                  paths.ctypes.data_as(u8p), C.byref(depth)))
+    return out, paths.reshape(-1)[:len(idx) * depth.value * 32].reshape(len(idx), depth.value, 32).copy()
+
+
 def rs_fold(codeword, d, n_domain, level, r):
     m = codeword.entries // 2
     r = _u32(r)

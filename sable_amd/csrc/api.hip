@@ -585,6 +585,37 @@ int exh_merkle_commit(exh_table codewords, int ncols, int c, exh_table *levels, 
   return status;
 }
 
+int exh_open_queries(exh_table codewords, int ncols, int c, exh_table levels, const uint64_t *leaves, int count,
+                     uint32_t *out_leaves, uint8_t *out_paths, int *out_depth) {
+  DeviceTable *cw = table_of(codewords);
+  if (!cw) return E_PARAM;
+  if (ncols < 1 || c < 1 || c > 23 || cw->n_u32 != ((uint64_t)ncols << (c + 1))) {
+    set_error("invalid-parameter: codewords must hold ncols * 2^(c+1) symbols, 1 <= c <= 23");
+    return E_PARAM;
+  }
+  const uint64_t nleaves = (uint64_t)1 << (c - 1);
+  const uint32_t *d_levels = nullptr;
+  if (levels) {
+    DeviceTable *lv = table_of(levels);
+    if (!lv) return E_PARAM;
+    if (lv->n_u32 != (2 * nleaves - 1) * 8 || !out_paths) {
+      set_error("invalid-parameter: levels must hold 2 * 2^(c-1) - 1 digests, and the paths need a buffer");
+      return E_PARAM;
+    }
+    d_levels = lv->ptr;
+  }
+  if (count < 0 || count > (1 << 20) || (count > 0 && (!leaves || !out_leaves))) {
+    set_error("invalid-parameter: 0 <= count <= 2^20 leaf indices and a buffer for their rows");
+    return E_PARAM;
+  }
+  for (int q = 0; q < count; q++)
+    if (leaves[q] >= nleaves) {
+      set_error("invalid-parameter: leaf index beyond the tree's 2^(c-1) leaves");
+      return E_PARAM;
+    }
+  return open_queries_device(cw->ptr, ncols, c, d_levels, leaves, count, out_leaves, out_paths, out_depth);
+}
+
 int exh_rs_fold(exh_table codeword, int D, uint64_t m, int n_domain, int level, const uint32_t *r, exh_table *out) {
   DeviceTable *cw = table_of(codeword);
   if (!cw) return E_PARAM;

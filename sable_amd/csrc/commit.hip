@@ -753,6 +753,66 @@ static int gather_to_host(const uint32_t *src, const std::vector<uint64_t> &offs
   return OK;
 }
 
+// OPEN-QUERIES' two gathers for one (unit, class) (src/pcs.lisp:721-734).  Leaves: out[(q * ncols + k) * 4 + s] =
+// symbol 4 * leaf_q + s of column k (LEAF-ROWS, src/pcs.lisp:275-277, as the (Q, rows, 4) array of
+// FIELD-ARRAY-OF-LEAVES, :659-665): one thread per (q, k), one 16-byte load.
+__global__ __launch_bounds__(BLOCK) void open_leaves_kernel(const uint32_t *cw, uint64_t cw_len, uint32_t ncols,
+                                                            const uint64_t *leaf, uint32_t count, uint32_t *out) {
+  uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid >= (uint64_t)count * ncols) return;
+  uint32_t q = (uint32_t)(gid / ncols), k = (uint32_t)(gid % ncols);
+  const uint4 v = *(const uint4 *)(cw + (uint64_t)k * cw_len + 4 * leaf[q]);
+  *(uint4 *)(out + gid * 4) = v;
+}
+
+// Paths: out[(q * depth + d) * 8 ..] = the sibling of leaf_q's ancestor on level d (PATH, src/pcs.lisp:79-84); the
+// levels lie leaves first, level d at digest 2 * nleaves - 2 * (nleaves >> d).  One thread per digest word.
+__global__ __launch_bounds__(BLOCK) void open_paths_kernel(const uint32_t *levels, uint64_t nleaves, uint32_t depth,
+                                                           const uint64_t *leaf, uint32_t count, uint32_t *out) {
+  uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid >= (uint64_t)count * depth * 8) return;
+  uint32_t w = (uint32_t)(gid % 8), d = (uint32_t)((gid / 8) % depth), q = (uint32_t)(gid / 8 / depth);
+  uint64_t start = 2 * nleaves - 2 * (nleaves >> d);
+  out[gid] = levels[(start + ((leaf[q] >> d) ^ 1)) * 8 + w];
+}
+
+int open_queries_device(const uint32_t *d_codewords, int ncols, int c, const uint32_t *d_levels, const uint64_t *leaves,
+                        int count, uint32_t *out_leaves, uint8_t *out_paths, int *out_depth) {
+  Context &cx = ctx();
+  int status = cx.require();
+  if (status) return status;
+  const uint64_t nleaves = (uint64_t)1 << (c - 1), cw_len = (uint64_t)1 << (c + 1);
+  const uint32_t depth = d_levels ? (uint32_t)cap_level_of(nleaves) : 0;
+  if (out_depth) *out_depth = (int)depth;
+  if (count == 0) return OK;
+  const uint64_t leaf_words = (uint64_t)count * ncols * 4, path_words = (uint64_t)count * depth * 8;
+  // one pooled buffer: the indices (padded to 16 bytes: the leaves are stored as uint4), the leaves, the paths
+  const size_t idx_slots = ((size_t)count + 1) & ~(size_t)1;
+  uint64_t *d_idx = (uint64_t *)cx.pool.alloc(idx_slots * 8 + (leaf_words + path_words) * 4);
+  if (!d_idx) {
+    set_error("device-out-of-memory: query openings");
+    return E_NOMEM;
+  }
+  uint32_t *d_leaf_out = (uint32_t *)(d_idx + idx_slots), *d_path_out = d_leaf_out + leaf_words;
+  hipError_t e = hipMemcpyAsync(d_idx, leaves, (size_t)count * 8, hipMemcpyHostToDevice, cx.stream);
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL(open_leaves_kernel, dim3((uint32_t)(((uint64_t)count * ncols + BLOCK - 1) / BLOCK)), dim3(BLOCK),
+                       0, cx.stream, d_codewords, cw_len, (uint32_t)ncols, d_idx, (uint32_t)count, d_leaf_out);
+    if (path_words)
+      hipLaunchKernelGGL(open_paths_kernel, dim3((uint32_t)((path_words + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0,
+                         cx.stream, d_levels, nleaves, depth, d_idx, (uint32_t)count, d_path_out);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess) e = hipMemcpyAsync(out_leaves, d_leaf_out, leaf_words * 4, hipMemcpyDeviceToHost, cx.stream);
+  if (e == hipSuccess && path_words)
+    e = hipMemcpyAsync(out_paths, d_path_out, path_words * 4, hipMemcpyDeviceToHost, cx.stream);
+  hipError_t e2 = hipStreamSynchronize(cx.stream);  // the indices (pageable) and the pooled buffer are free after this
+  cx.pool.release(d_idx);
+  EXH_HIP(e);
+  EXH_HIP(e2);
+  return OK;
+}
+
 int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
                    int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final) {
   Context &c = ctx();

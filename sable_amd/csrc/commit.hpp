@@ -28,6 +28,11 @@ int combine_columns_device(int D, const uint32_t *d_cols, int ncols, uint64_t le
 // 2^(c+1) symbols; cap: the level max(0, log2(leaves) - 7), as bytes
 int merkle_commit_columns(const uint32_t *d_codewords, int ncols, int c, uint32_t *d_levels, uint8_t *cap,
                           uint64_t *cap_rows);
+// OPEN-QUERIES' gathers for one (unit, class) (src/pcs.lisp:721-734): the queried leaves' rows of a class's ncols
+// codewords of 2^(c+1) symbols (out_leaves: count * ncols * 4 words) and, when d_levels is given, each leaf's
+// siblings up to the cap level (out_paths: count * depth * 32 bytes); leaves: count leaf indices below 2^(c-1)
+int open_queries_device(const uint32_t *d_codewords, int ncols, int c, const uint32_t *d_levels, const uint64_t *leaves,
+                        int count, uint32_t *out_leaves, uint8_t *out_paths, int *out_depth);
 int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
                    int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final);
 int basefold_verify(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,

@@ -297,3 +297,46 @@ def test_scale_add_builds_the_class_table(d, length):
         h = nxt
     assert same(h.download().reshape(length, d), want)
     h.free()
+
+
+@pytest.mark.parametrize("c,ncols,count", [(1, 1, 3), (6, 5, 7), (12, 3, 40), (9, 70, 1)])
+def test_open_queries_match_the_oracle(c, ncols, count):
+    """src/pcs.lisp:721-734: the queried leaves' rows and their paths, as the prover records them."""
+    rng = np.random.default_rng(c * 100 + ncols)
+    cols = [rng.integers(0, P, 1 << c, dtype=np.uint32) for _ in range(ncols)]
+    ocw, olevels, ocap = orc.commit_columns(cols, c)
+    nleaves = 1 << (c - 1)
+    idx = rng.integers(0, nleaves, count).astype(np.uint64)
+    idx[0], idx[-1] = 0, nleaves - 1
+    want_leaves, want_paths = orc.open_queries(ocw, c, olevels, idx)
+    t = sa.Table.upload(np.concatenate(cols))
+    cw = sa.encode(t, ncols, c)
+    levels, cap = sa.merkle_commit(cw, ncols, c)
+    got_leaves, got_paths = sa.open_queries(cw, ncols, c, levels, idx)
+    assert same(got_leaves, want_leaves)
+    assert got_paths.shape == want_paths.shape and same(got_paths, want_paths)
+    only_leaves, none = sa.open_queries(cw, ncols, c, None, idx)
+    assert same(only_leaves, want_leaves) and none.shape == (count, 0, 32)
+    empty = sa.open_queries(cw, ncols, c, levels, np.zeros(0, np.uint64))
+    assert empty[0].shape == (0, ncols, 4)
+    with pytest.raises(sa.ExactaError):
+        sa.open_queries(cw, ncols, c, levels, np.array([nleaves], np.uint64))
+    for x in (t, cw, levels):
+        x.free()
+
+
+def test_open_queries_full_size_open_to_the_cap():
+    """Config 5's commitment: 64 queried leaves of the 2^22-leaf tree, each hashed and walked up its path to the cap."""
+    c, ncols = 23, 2
+    t = sa.Table.random(12, ncols << c)
+    cw = sa.encode(t, ncols, c)
+    levels, cap = sa.merkle_commit(cw, ncols, c)
+    nleaves = 1 << (c - 1)
+    idx = np.random.default_rng(5).integers(0, nleaves, 64).astype(np.uint64)
+    leaves, paths = sa.open_queries(cw, ncols, c, levels, idx)
+    assert paths.shape == (64, orc.cap_level(nleaves), 32)
+    for q, l in enumerate(int(x) for x in idx):
+        assert orc.check_path(orc.leaf_digest(leaves[q]), paths[q], l, cap)
+    assert not orc.check_path(orc.leaf_digest(leaves[0]), paths[1], int(idx[0]), cap)
+    for x in (t, cw, levels):
+        x.free()

@@ -349,3 +349,28 @@ def test_scale_add_from_the_definition():
     sc = rng.integers(0, P, 8, dtype=np.uint32)
     want = [pf.add(list(map(int, h[x])), pf.mul(list(map(int, sc)), list(map(int, col[x])))) for x in range(5)]
     assert orc.scale_add(h, sc, col).tolist() == want
+
+
+@pytest.mark.parametrize("c,ncols", [(1, 1), (4, 3), (10, 2)])
+def test_open_queries_from_the_definition(c, ncols):
+    """src/pcs.lisp:721-734: the opened leaves are symbols 4l..4l+3 of every codeword (:275-277), the paths the
+    siblings up to the cap level (:79-84): numpy indexing, and every opening hashes up to the committed cap."""
+    rng = np.random.default_rng(721 + c)
+    cols = [rng.integers(0, pf.P, 1 << c, dtype=np.uint32) for _ in range(ncols)]
+    cw, levels, cap = orc.commit_columns(cols, c)
+    nleaves = 1 << (c - 1)
+    idx = np.concatenate([[0, nleaves - 1], rng.integers(0, nleaves, 9)]).astype(np.uint64)
+    leaves, paths = orc.open_queries(cw, c, levels, idx)
+    depth = orc.cap_level(nleaves)
+    assert leaves.shape == (len(idx), ncols, 4) and paths.shape == (len(idx), depth, 32)
+    for q, l in enumerate(int(x) for x in idx):
+        assert np.array_equal(leaves[q], cw[:, 4 * l:4 * l + 4])
+        for lev in range(depth):
+            assert np.array_equal(paths[q, lev], levels[lev][(l >> lev) ^ 1])
+        assert orc.check_path(orc.leaf_digest(leaves[q]), paths[q], l, cap)
+        if depth:  # a path of another leaf does not open this one
+            other = (q + 1) % len(idx)
+            if (int(idx[other]) >> 1) != (l >> 1):
+                assert not orc.check_path(orc.leaf_digest(leaves[q]), paths[other], l, cap)
+    no_paths = orc.open_queries(cw, c, None, idx)
+    assert np.array_equal(no_paths[0], leaves) and no_paths[1].shape == (len(idx), 0, 32)
