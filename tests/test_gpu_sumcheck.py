@@ -110,6 +110,13 @@ def test_config3_product_constraint_over_fp8(n):
     assert st.degree == 4 and len(proof) == 12 + n * (18 + 4 * 4 * 8)
 
 
+DOMAIN_FORM = ("(+ (* A0 (+ (* m0 (- Z g1 (* BETA0 v1))) (* m1 (- Z g0 (* BETA0 v0)))))"
+               " (* AL0 (- Z g0 (* BETA0 v0)) (- Z g1 (* BETA0 v1)))"
+               " (* GAM0 c0) (* GETA0 c1))")
+DOMAIN_TABLES = ["g0", "g1", "v0", "v1", "m0", "m1", "c0", "c1"]
+DOMAIN_CONSTANTS = ["Z", "BETA0", "A0", "AL0", "GAM0", "GETA0"]
+
+
 @pytest.mark.parametrize("form,names,cnames,d,base,with_eq", [
     ("(* t0 t1 t2)", ["t0", "t1", "t2"], [], 4, True, True),
     ("(* t0 t1 t2)", ["t0", "t1", "t2"], [], 8, False, False),
@@ -126,6 +133,10 @@ def test_config3_product_constraint_over_fp8(n):
     ("(+ (* alpha (+ t0 1) (- t1 t0) t2) (* 3 t0) 9)", ["t0", "t1", "t2"], ["alpha"], 4, False, True),
     ("(- (* (expt (- t0 1) 2) (+ t1 t0)) (* beta (- t1 4) t0))", ["t0", "t1"], ["beta"], 4, True, False),
     ("(* (- t0) (+ t1 -3) (+ t0 t1 t2 t3 1) t3)", ["t0", "t1", "t2", "t3"], [], 8, True, True),
+    # the shape of DOMAIN-STATEMENT (src/domain.lisp:95-114): a lookup with a numerator, its denominators
+    # q = Z - tag - BETA0 * value at both halves, and a constraint's two halves
+    (DOMAIN_FORM, DOMAIN_TABLES, DOMAIN_CONSTANTS, 8, True, True),
+    (DOMAIN_FORM, DOMAIN_TABLES, DOMAIN_CONSTANTS, 4, False, True),
 ])
 def test_any_statement_on_the_interpreter_or_generated_kernels(form, names, cnames, d, base, with_eq):
     """tests.lisp:311-395: statements that are not plain products, constants, base or extension tables."""
@@ -247,6 +258,7 @@ def test_device_loop_entry_point_from_a_host_transcript_state():
     ("(* t0 t1)", ["t0", "t1"], [], 8, False, False, 16),
     ("(+ (* t0 t1 t2) (* 7 t1) -1)", ["t0", "t1", "t2"], [], 4, True, True, 19),
     ("(* (+ (* 5 t0) (* -3 t1) 7) (- t2 (* 2 t0)))", ["t0", "t1", "t2"], [], 4, True, True, 16),
+    (DOMAIN_FORM, DOMAIN_TABLES, DOMAIN_CONSTANTS, 8, True, True, 17),  # eight columns, six constants, interpreter
 ])
 def test_rounds_on_a_grid_of_lds_resident_slices(form, names, cnames, d, base, with_eq, n):
     """Sizes at which the rounds between the large kernels and the last workgroup run as one launch of
