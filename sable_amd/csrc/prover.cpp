@@ -43,17 +43,25 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
     state.used = tr.state.used;
     state.counter_lo = (uint32_t)tr.state.counter, state.counter_hi = (uint32_t)(tr.state.counter >> 32);
     std::vector<uint32_t> messages((size_t)n * points * D), challenges((size_t)n * D);
-    if ((status = s.run_device(state, messages.data(), challenges.data()))) return status;
-    for (int j = 0; j < n; j++) {
-      uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
-      if ((status = tr.send(&messages[(size_t)j * points * D], 2, dims, nullptr))) return status;
-      uint32_t *r = out_chal + (size_t)j * D;
-      tr.challenge(D, r);
-      if (memcmp(r, &challenges[(size_t)j * D], 4 * D) != 0) {
-        set_error("device-error: the device transcript drew a different challenge in round " + std::to_string(j));
-        return E_DEVICE;
+    int replayed = 0;
+    auto replay = [&](int upto) -> int {
+      for (; replayed < upto; replayed++) {
+        const int j = replayed;
+        uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
+        int st_send = tr.send(&messages[(size_t)j * points * D], 2, dims, nullptr);
+        if (st_send) return st_send;
+        uint32_t *r = out_chal + (size_t)j * D;
+        tr.challenge(D, r);
+        if (memcmp(r, &challenges[(size_t)j * D], 4 * D) != 0) {
+          set_error("device-error: the device transcript drew a different challenge in round " + std::to_string(j));
+          return E_DEVICE;
+        }
       }
-    }
+      return OK;
+    };
+    // the leading rounds are replayed while the device still works on the last ones
+    if ((status = s.run_device(state, messages.data(), challenges.data(), replay))) return status;
+    if ((status = replay(n))) return status;
     return s.finish(out_finals, out_folded);
   }
   uint32_t sums[16 * 8];

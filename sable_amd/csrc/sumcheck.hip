@@ -738,7 +738,8 @@ static uint64_t tail_pairs(int T, int D) {
   return p;
 }
 
-int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges) {
+int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges,
+                                const std::function<int(int)> &early) {
   Context &c = ctx();
   if (int owned = owns_arenas()) return owned;
   if (round != 0 || pending_fold || claim_mode || !device_capable()) {
@@ -889,6 +890,8 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   uint32_t *down = c.host_pinned + PIN_DOWN;
   const size_t ctrl_words = (sizeof(Ctrl) + 3) / 4;
   bool logged_to_host = false;
+  int early_rounds = 0;  // leading rounds already handed to `early`
+  bool early_on = false;
   if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
     // when a single entry per table is left at the end (the finals travel in the control block), the launch
     // itself delivers the control block to pinned host memory
@@ -896,10 +899,13 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     if (deliver) {
       if (++c.log_seq == 0) ++c.log_seq;  // 0 is what the flag is reset to
       host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = c.log_seq;
+      host_early = (early && j > 0) ? 1 : 0;
+      early_on = host_early != 0;
       reinterpret_cast<volatile uint32_t *>(down)[ctrl_words] = 0;
+      reinterpret_cast<volatile uint32_t *>(down)[ctrl_words + 1] = 0;
     }
     status = launch_tail(j, n - j, 1, folds_due > 0);
-    host_log = nullptr;
+    host_log = nullptr, host_early = 0;
     folds_due = 0;
     tail_done = status == OK;
     logged_to_host = deliver && tail_done;
@@ -917,6 +923,24 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     volatile uint32_t *flag = reinterpret_cast<volatile uint32_t *>(down) + ctrl_words;
     uint32_t spins = 0;
     while (*flag != c.log_seq) {
+      const uint32_t word = flag[1];
+      if (early_on && (word >> 6) == (c.log_seq & 0x03ffffffu) && (int)(word & 63) > early_rounds) {
+        // more leading rounds are in: hand them on meanwhile
+        std::atomic_thread_fence(std::memory_order_acquire);
+        const int upto = std::min<int>((int)(word & 63), n);
+        const Ctrl *rc = reinterpret_cast<const Ctrl *>(down);
+        for (int r = early_rounds; r < upto; r++) {
+          memcpy(messages + (size_t)r * points * D, rc->msg[r], (size_t)points * D * 4);
+          memcpy(challenges + (size_t)r * D, rc->chal[r], (size_t)D * 4);
+        }
+        early_rounds = upto;
+        const int early_status = early(upto);
+        if (early_status) {
+          (void)hipStreamSynchronize(c.stream);  // nothing of this session is left running
+          return early_status;
+        }
+        continue;
+      }
       if ((++spins & 1023) == 0 && hipStreamQuery(c.stream) == hipSuccess) break;
     }
     if (*flag != c.log_seq) {
@@ -986,7 +1010,7 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
     a.pstride = pstride;
     a.groups = groups;
     a.spin_limit = 200000;
-    a.host_log = host_log, a.host_flag_at = host_flag_at, a.host_seq = host_seq;
+    a.host_log = host_log, a.host_flag_at = host_flag_at, a.host_seq = host_seq, a.host_early = host_early;
     for (int jj = 0; jj < rounds; jj++) {
       a.low_off[jj] = low_off[j + jj];
       a.high_off[jj] = high_off[j + jj];

@@ -26,7 +26,8 @@
 namespace exh {
 
 // StmtDesc and the limits MAXT, MAXG, ... come from stmtdesc.hpp
-constexpr int MAXROUNDS = 48;  // rounds of one device-driven sumcheck
+constexpr int MAXROUNDS = 48;  // rounds of one device-driven sumcheck (a count of them fits six bits)
+constexpr uint32_t COURIER_STEP = 1;  // the last launch sends finished rounds to the host every so many rounds
 constexpr int MAXPTS = 7;      // wire points of a device-driven round message
 constexpr int MAXTAIL = 16;    // rounds the tail kernel can take
 
@@ -94,6 +95,9 @@ struct TailArgs {
   // on the stream to read the logs (null: it does both)
   uint32_t *host_log;
   uint32_t host_flag_at, host_seq;
+  // host_early: the launch also delivers finished rounds' messages and challenges as it goes, counting them in
+  // host_log[host_flag_at + 1] as (host_seq << 6) | rounds, so the host can work on them while this one runs
+  uint32_t host_early;
 };
 
 template <int D>
@@ -768,6 +772,35 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   const uint32_t tid = threadIdx.x, cap = args.capacity, G = gridDim.x, wg = blockIdx.x;
   const uint32_t width = (uint32_t)d.nacc * D;
   if (args.ctrl->round != args.first_round) return;  // an earlier launch gave up: leave the count as it is
+  // The courier: with host_early, the last wavefront carries finished rounds' rows (message, challenge) to the
+  // host log while the launch runs, and publishes in host_log[host_flag_at + 1] how many leading rounds are
+  // there (with the delivery's sequence number above the count's six bits).  The rounds before this launch go
+  // out at once; a round of this launch goes out at the start of a later one, and is published a delivery after
+  // that, when its stores have long landed and the release costs no wait.
+  const bool courier = args.host_log && args.host_early && G == 1;
+  uint32_t carried = courier ? args.first_round : 0;  // rounds whose rows have been stored to the host log
+  auto carry_rows = [&](uint32_t from, uint32_t upto) {
+    const uint32_t lane = tid - (BLOCK - 64), mw = args.points * D;
+    const uint32_t *words = reinterpret_cast<const uint32_t *>(args.ctrl);
+    for (uint32_t u = from * mw + lane; u < upto * mw; u += 64) {
+      const uint32_t at = (uint32_t)(offsetof(Ctrl, msg) / 4) + (u / mw) * (MAXPTS * 8) + u % mw;
+      args.host_log[at] = __hip_atomic_load(words + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    for (uint32_t u = from * D + lane; u < upto * D; u += 64) {
+      const uint32_t at = (uint32_t)(offsetof(Ctrl, chal) / 4) + (u / D) * 8 + u % D;
+      args.host_log[at] = __hip_atomic_load(words + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+  auto publish = [&](uint32_t count) {
+    __threadfence_system();
+    if (tid == BLOCK - 64)
+      __hip_atomic_store(args.host_log + args.host_flag_at + 1, (args.host_seq << 6) | count, __ATOMIC_RELEASE,
+                         __HIP_MEMORY_SCOPE_SYSTEM);
+  };
+  if (courier && tid >= BLOCK - 64) {
+    carry_rows(0, args.first_round);
+    publish(args.first_round);
+  }
   RunB3S tr;
   if (tid < 64) rb3s_load(tr, epi.ring, &args.ctrl->tr);
   uint32_t entries = (args.first_fold ? args.entries / 2 : args.entries) / G;  // of this workgroup's slice
@@ -817,6 +850,13 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   __syncthreads();
   for (uint32_t jj = 0; jj < args.rounds; jj++) {
     const uint32_t pairs = entries / 2;
+    if (courier && jj > 0 && jj % COURIER_STEP == 0) {
+      if (tid >= BLOCK - 64) {
+        if (carried > args.first_round) publish(carried);
+        carry_rows(carried, args.first_round + jj);
+      }
+      carried = args.first_round + jj;
+    }
     Acc96 acc[MAXACC][D];
 #pragma unroll
     for (int a = 0; a < MAXACC; a++)
@@ -923,10 +963,11 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
       args.host_log[at] = __hip_atomic_load(words + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
     const uint32_t all_rounds = args.first_round + args.rounds, mw = args.points * D;
+    const uint32_t from = carried;  // the rounds before have gone out already
     for (uint32_t u = tid; u < offsetof(Ctrl, msg) / 4; u += BLOCK) deliver(u);
-    for (uint32_t u = tid; u < all_rounds * mw; u += BLOCK)
+    for (uint32_t u = from * mw + tid; u < all_rounds * mw; u += BLOCK)
       deliver((uint32_t)(offsetof(Ctrl, msg) / 4) + (u / mw) * (MAXPTS * 8) + u % mw);
-    for (uint32_t u = tid; u < all_rounds * D; u += BLOCK)
+    for (uint32_t u = from * D + tid; u < all_rounds * D; u += BLOCK)
       deliver((uint32_t)(offsetof(Ctrl, chal) / 4) + (u / D) * 8 + u % D);
     for (uint32_t u = tid; u < (uint32_t)d.T * D; u += BLOCK) deliver((uint32_t)(offsetof(Ctrl, finals) / 4) + u);
     __threadfence_system();
