@@ -899,7 +899,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     if (deliver) {
       if (++c.log_seq == 0) ++c.log_seq;  // 0 is what the flag is reset to
       host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = c.log_seq;
-      host_early = (early && j > 0) ? 1 : 0;
+      host_early = early ? 1 : 0;
       early_on = host_early != 0;
       reinterpret_cast<volatile uint32_t *>(down)[ctrl_words] = 0;
       reinterpret_cast<volatile uint32_t *>(down)[ctrl_words + 1] = 0;

@@ -797,7 +797,7 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
       __hip_atomic_store(args.host_log + args.host_flag_at + 1, (args.host_seq << 6) | count, __ATOMIC_RELEASE,
                          __HIP_MEMORY_SCOPE_SYSTEM);
   };
-  if (courier && tid >= BLOCK - 64) {
+  if (courier && args.first_round > 0 && tid >= BLOCK - 64) {
     carry_rows(0, args.first_round);
     publish(args.first_round);
   }
