@@ -226,10 +226,12 @@ def test_linearity_and_fold_consistency_at_scale():
         t.free()
 
 
-def test_device_loop_entry_point_from_a_host_transcript_state():
-    """exh_sumcheck_run: the host absorbs the header, hands over its hash state, and replays the messages."""
-    n, d = 11, 4
-    rng = np.random.default_rng(6)
+@pytest.mark.parametrize("n", [4, 11, 17])
+def test_device_loop_entry_point_from_a_host_transcript_state(n):
+    """exh_sumcheck_run: the host absorbs the header, hands over its hash state, and replays the messages (every
+    round in one launch, slices and last launch, streaming rounds before them)."""
+    d = 4
+    rng = np.random.default_rng(6 + n)
     tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in range(3)]
     eq, alpha = rand_ext(rng, (n,), d), rand_ext(rng, (1,), d)
     st, ost = both(CONFIG2, ["t0", "t1", "t2"], ["alpha"])
