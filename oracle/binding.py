@@ -68,7 +68,7 @@ i32p = C.POINTER(C.c_int32)
 
 class Stmt(C.Structure):
     _fields_ = [("T", C.c_int), ("C", C.c_int), ("nterms", C.c_int), ("coeff", u32p), ("start", i32p),
-                ("vars", i32p)]
+                ("vars", i32p), ("nops", C.c_int), ("ops", i32p), ("args", i32p)]
 
 
 class Msg(C.Structure):
@@ -103,6 +103,8 @@ def _declare(l):
 
 
 def _u32(a):
+    if isinstance(a, np.ndarray) and a.dtype == np.uint32 and a.flags.c_contiguous and a.size > (1 << 16):
+        return a  # a large table already in the wire type (its values are residues by construction)
     a = np.asarray(a, dtype=np.uint64)
     out = np.empty(a.shape, np.uint32)  # keeps rank 0 (ascontiguousarray would not)
     out[...] = a % P
@@ -461,6 +463,94 @@ def combine_columns(columns, coefficients):
 
 
 # ------------------------------------------------------------------ statements and sumcheck
+def _postfix(form, index, n_tables):
+    """The form as written, as the postfix program of orc.h's orc_stmt: what ARITHMETIC-FORM emits
+    (src/forms.lisp:113-141), n-ary chains reduced left to right, (expt b k) as k - 1 products of b."""
+    ops, args = [], []
+
+    def emit(op, arg=0):
+        ops.append(op)
+        args.append(arg)
+
+    def chain(op, arguments, empty):
+        if not arguments:
+            emit(2, empty)
+            return
+        walk(arguments[0])
+        for a in arguments[1:]:
+            walk(a)
+            emit(op)
+
+    def walk(f):
+        if isinstance(f, bool):
+            raise ValueError("malformed form")
+        if isinstance(f, int):
+            emit(2, f % P)
+        elif isinstance(f, str):
+            v = index[f.upper()]
+            emit(0, v) if v < n_tables else emit(1, v - n_tables)
+        elif isinstance(f, (list, tuple)) and f:
+            op, arguments = f[0], list(f[1:])
+            if op == "+":
+                chain(3, arguments, 0)
+            elif op == "*":
+                chain(5, arguments, 1)
+            elif op == "-":
+                if not arguments:
+                    raise ValueError("malformed form")
+                if len(arguments) == 1:
+                    walk(arguments[0])
+                    emit(6)
+                else:
+                    chain(4, arguments, 0)
+            elif op in ("expt", "EXPT"):
+                base, k = arguments
+                if not isinstance(k, int) or k < 0:
+                    raise ValueError("malformed form")
+                chain(5, [base] * k, 1)
+            else:
+                raise ValueError("malformed form")
+        else:
+            raise ValueError("malformed form: %r" % (f,))
+
+    walk(form)
+    return ops, args
+
+
+def set_fast(threads):
+    """threads > 0: orc_sumcheck_prove (and the provers built on it) run the threaded straight-line path of
+    orc_fast.c; 0: the plain restatement (the default, the one the golden proofs pin).  Same bytes either way."""
+    lib().orc_set_fast(int(threads))
+
+
+def host_threads():
+    return lib().orc_host_threads()
+
+
+def splitmix_field(seed, count):
+    """The seeded synthetic field elements of the benchmarks (exh_table_random's rule) on the host."""
+    out = np.empty(count, np.uint32)
+    lib().orc_splitmix_field(C.c_uint64(seed), C.c_uint64(count), _p(out))
+    return out
+
+
+def ext_mul_plain(a, b):
+    a, b = _u32(a), _u32(b)
+    out = np.zeros_like(a)
+    lib().orc_ext_mul_plain(len(a), _p(a), _p(b), _p(out))
+    return out
+
+
+def round_sums_fast(st, d, points, tables, low, high, constants=None, threads=1):
+    arrs, strides, ptrs = _tables(tables, d)
+    low, high = _u32(low).reshape(-1, d), _u32(high).reshape(-1, d)
+    ca = _u32(constants).reshape(-1, d) if constants is not None and len(constants) else np.zeros((1, d), np.uint32)
+    out = np.zeros((points, d), np.uint32)
+    _check(lib().orc_round_sums_fast(C.byref(st.c), d, points, C.c_uint64(len(low)), C.c_uint64(len(high)), ptrs,
+                                     strides.ctypes.data_as(i32p), _p(low), _p(high), _p(ca), threads, _p(out)))
+    return out
+
+
 class Statement:
     """A statement form with its table and constant variables fixed: the oracle's monomial IR."""
 
@@ -479,8 +569,11 @@ class Statement:
         self._coeff = np.array(coeff, np.uint32)
         self._start = np.array(start, np.int32)
         self._vars = np.array(vs if vs else [0], np.int32)
+        ops, args = _postfix(self.form, index, len(self.tables))
+        self._ops, self._args = np.array(ops, np.int32), np.array(args, np.int32)
         self.c = Stmt(len(self.tables), len(self.constants), len(coeff), _p(self._coeff),
-                      self._start.ctypes.data_as(i32p), self._vars.ctypes.data_as(i32p))
+                      self._start.ctypes.data_as(i32p), self._vars.ctypes.data_as(i32p), len(ops),
+                      self._ops.ctypes.data_as(i32p), self._args.ctypes.data_as(i32p))
         self.degree = lib().orc_stmt_degree(C.byref(self.c))
 
     def evaluate(self, table_values, constants, d):

@@ -74,6 +74,11 @@ void orc_ext_sub(int D, const uint32_t *a, const uint32_t *b, uint32_t *out);
 void orc_ext_neg(int D, const uint32_t *a, uint32_t *out);
 void orc_ext_scale(int D, const uint32_t *a, uint32_t s, uint32_t *out);
 void orc_ext_mul(int D, const uint32_t *a, const uint32_t *b, uint32_t *out);
+/* MUL* as the loops of src/field.lisp:213-234 for any power-of-two D <= 8 (orc_ext_mul runs the unrolled
+   orc_ext_mul4 / orc_ext_mul8 at D = 4, 8: the same residues) */
+void orc_ext_mul_plain(int D, const uint32_t *a, const uint32_t *b, uint32_t *out);
+void orc_ext_mul4(const uint32_t *a, const uint32_t *b, uint32_t *out);
+void orc_ext_mul8(const uint32_t *a, const uint32_t *b, uint32_t *out);
 int orc_ext_inv(int D, const uint32_t *a, uint32_t *out);
 void orc_ext_eq1(int D, const uint32_t *a, const uint32_t *b, uint32_t *out);
 void orc_ext_eq(int D, int k, const uint32_t *as, const uint32_t *bs, uint32_t *out);
@@ -171,6 +176,11 @@ typedef struct {
   const uint32_t *coeff;  /* nterms */
   const int32_t *start;   /* nterms + 1 offsets into vars */
   const int32_t *vars;
+  /* optionally the form as written, as a postfix program (ARITHMETIC-FORM, src/forms.lisp:113-141): op 0 table,
+     1 constant, 2 integer (arg = its residue), 3 +, 4 -, 5 *, 6 unary -; chains reduced left to right.  Only the
+     fast path (orc_set_fast) runs it; nops = 0: it evaluates the monomials instead. */
+  int nops;
+  const int32_t *ops, *args;
 } orc_stmt;
 int orc_stmt_degree(const orc_stmt *st); /* degree in the tables */
 void orc_stmt_eval(const orc_stmt *st, int D, const uint32_t *table_vals /* T*D */,
@@ -199,6 +209,19 @@ void orc_round_sums(const orc_stmt *st, int D, int points, uint64_t pairs_low, u
                     const uint32_t *high, const uint32_t *consts, uint32_t *out /* points*D */);
 void orc_fold_flat(int D, uint64_t len, const uint32_t *entries, int stride, const uint32_t *r,
                    uint32_t *out /* D * len/2 */);
+/* The same two functions organised for speed (orc_fast.c): the written form as straight-line code, base-field
+   lines when the reference would use them, unrolled products, OpenMP threads.  Same words out.
+   orc_set_fast(t > 0) makes orc_sumcheck_prove use them with t threads (0: the plain path, the default). */
+int orc_round_sums_fast(const orc_stmt *st, int D, int points, uint64_t n_low, uint64_t n_high,
+                        const uint32_t *const *tables, const int32_t *strides, const uint32_t *low,
+                        const uint32_t *high, const uint32_t *consts, int threads, uint32_t *out);
+int orc_fold_flat_fast(int D, uint64_t len, const uint32_t *entries, int stride, const uint32_t *r, int threads,
+                       uint32_t *out);
+void orc_set_fast(int threads);
+int orc_fast_threads(void);
+int orc_host_threads(void); /* what OpenMP would use by default */
+/* SplitMix64(seed) -> 31-bit words, kept when below p: the seeded synthetic inputs of the benchmarks */
+void orc_splitmix_field(uint64_t seed, uint64_t count, uint32_t *out);
 
 /* ---- LogUp-GKR (src/gkr.lisp) */
 /* leaves: per lookup l, p = leaves[2l], q = leaves[2l+1], each K*2^n EXTs block-major */

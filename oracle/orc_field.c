@@ -96,7 +96,15 @@ static void mul_star(int d, const uint32_t *a_t, const uint32_t *b_t, uint32_t *
   for (int e = 0; e < d; e++) out_t[e] = c[bit_reverse(e, bits)];
 }
 
-void orc_ext_mul(int D, const uint32_t *a, const uint32_t *b, uint32_t *out) { mul_star(D, a, b, out); }
+void orc_ext_mul_plain(int D, const uint32_t *a, const uint32_t *b, uint32_t *out) { mul_star(D, a, b, out); }
+void orc_ext_mul(int D, const uint32_t *a, const uint32_t *b, uint32_t *out) {
+  if (D == 4)
+    orc_ext_mul4(a, b, out);
+  else if (D == 8)
+    orc_ext_mul8(a, b, out);
+  else
+    mul_star(D, a, b, out);
+}
 
 /* A w for the generator w of A's level, src/field.lisp:206-211 */
 static void mul_by_generator(int d, const uint32_t *a, uint32_t *out) {

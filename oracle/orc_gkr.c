@@ -35,6 +35,7 @@ static void layer_stmt_make(layer_stmt *ls, int lookups, int extra) {
     }
   }
   ls->start[nterms] = k;
+  memset(&ls->st, 0, sizeof(ls->st));
   ls->st.T = T;
   ls->st.C = 2 * lookups;
   ls->st.nterms = nterms;

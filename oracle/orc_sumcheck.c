@@ -173,7 +173,11 @@ int orc_sumcheck_prove(orc_tr *tr, int n, const orc_stmt *st, const uint32_t *co
       n_high = (uint64_t)1 << (n - middle);
     }
     uint32_t sums[16 * ORC_MAXD];
-    orc_round_sums(st, D, points, n_low, n_high, cur, stride, low, high, consts, sums);
+    const int fast = orc_fast_threads();
+    if (fast > 0)
+      orc_round_sums_fast(st, D, points, n_low, n_high, cur, stride, low, high, consts, fast, sums);
+    else
+      orc_round_sums(st, D, points, n_low, n_high, cur, stride, low, high, consts, sums);
     free(low);
     free(high);
     uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
@@ -183,7 +187,10 @@ int orc_sumcheck_prove(orc_tr *tr, int n, const orc_stmt *st, const uint32_t *co
     orc_tr_challenge(tr, D, r);
     for (int t = 0; t < T; t++) {
       uint32_t *next = (uint32_t *)malloc((size / 2) * D * sizeof(uint32_t) + 4);
-      orc_fold_flat(D, size, cur[t], stride[t], r, next);
+      if (fast > 0)
+        orc_fold_flat_fast(D, size, cur[t], stride[t], r, fast, next);
+      else
+        orc_fold_flat(D, size, cur[t], stride[t], r, next);
       free(flat[t]);
       flat[t] = next;
       cur[t] = next;
