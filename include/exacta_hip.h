@@ -129,6 +129,13 @@ int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int degree_d
    of either by the round's challenge r (degree = the table's) -> a new table of half the length */
 int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out);
 int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out);
+/* exh_dot_pairs for callers that cannot allocate device memory while they run (code under HIP graph capture,
+   tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+   arguments and result as exh_dot_pairs; the workgroups' partial sums live in a static 48 KiB device array that
+   each GPU holds until the process ends, and the call makes no hipMalloc, hipFree or other allocating call.
+   Tables of more than 2^26 EXT8s are refused (invalid-parameter).  Calls on one GPU share that GPU's array:
+   calls that overlap on one GPU race. */
+int exh_dot_pairs_static(exh_table e, exh_table v, uint32_t *out);
 /* The opening's table per class (src/pcs.lisp:709-716), one unit at a time: out[x] = h[x] + scale * column[x]
    over extension tables of one shape; h = 0 stands for the table of zeros the sum starts from */
 int exh_table_scale_add(exh_table h, const uint32_t *scale, exh_table column, exh_table *out);

@@ -435,6 +435,13 @@ def dot_pairs(e, v):
     return out
 
 
+def dot_pairs_static(e, v):
+    """dot_pairs through the entry point that allocates nothing (static device scratch): (3, 8)."""
+    out = np.zeros((3, 8), np.uint32)
+    check(load().exh_dot_pairs_static(C.c_uint64(e.handle), C.c_uint64(v.handle), _p(out)))
+    return out
+
+
 def fold_table(table, r):
     """fold-table of an extension Table by the challenge r -> Table of half the length."""
     r = _u32(r)

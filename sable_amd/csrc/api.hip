@@ -654,6 +654,16 @@ int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out) {
   return dot_pairs_device(te->ptr, tv->ptr, te->n_u32 / 8, out);
 }
 
+int exh_dot_pairs_static(exh_table e, exh_table v, uint32_t *out) {
+  DeviceTable *te = table_of(e), *tv = table_of(v);
+  if (!te || !tv) return E_PARAM;
+  if (!out || te->stride != 8 || tv->stride != 8 || te->n_u32 != tv->n_u32 || te->n_u32 < 16 || (te->n_u32 / 8) % 2) {
+    set_error("invalid-parameter: dot-pairs takes two tables of the same even number of EXT8s");
+    return E_PARAM;
+  }
+  return dot_pairs_static_device(te->ptr, tv->ptr, te->n_u32 / 8, out);
+}
+
 int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out) {
   DeviceTable *t = table_of(table);
   if (!t) return E_PARAM;

@@ -640,6 +640,70 @@ int dot_pairs_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uin
   return OK;
 }
 
+// ---- DOT-PAIRS once more for callers that must not allocate: the workgroups' partial sums live in a static
+// device array instead of a pooled buffer, and the 24 words of the result come back through the pinned host
+// buffer the context has held since exh_init.  The array's name is a host-side stand-in: the address kernels
+// can use comes from hipGetSymbolAddress, once per device, with that device current (each GPU holds its own
+// copy of the array at its own address).  Every call on a GPU shares that GPU's array: calls that overlap on one
+// GPU race.  A launch writes every word it later reads, so nothing has to be cleared between calls.
+constexpr uint32_t STATIC_DOT_GRID = 512;                    // workgroups of the launch
+constexpr uint64_t STATIC_DOT_MAX_LEN = (uint64_t)1 << 26;   // EXT8s per table: 2 GiB each
+constexpr size_t STATIC_DOT_RESULT_AT = 4096;                // word of the pinned buffer the result lands at
+static __device__ __align__(256) uint32_t scratch[STATIC_DOT_GRID * 24];  // 48 KiB per GPU until the process ends
+constexpr int STATIC_MAX_DEVICES = 64;
+static uint32_t *g_scratch_ptr[STATIC_MAX_DEVICES];
+
+// the sums of the partial rows, written where `sums` points (mapped host memory here)
+__global__ __launch_bounds__(BLOCK) void sum_columns_to_host_kernel(const uint32_t *partials, uint32_t nblocks,
+                                                                    uint32_t width, uint32_t *sums) {
+  __shared__ uint32_t lds[BLOCK / 64];
+  uint32_t o = blockIdx.x, v = 0;
+  for (uint32_t b = threadIdx.x; b < nblocks; b += BLOCK) v = fadd(v, partials[(uint64_t)b * width + o]);
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < BLOCK / 64; w++) v = fadd(v, lds[w]);
+    __hip_atomic_store(sums + o, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+int dot_pairs_static_setup(int device) {
+  if (device < 0 || device >= STATIC_MAX_DEVICES) {
+    set_error("invalid-parameter: device index beyond the static scratch table");
+    return E_PARAM;
+  }
+  if (g_scratch_ptr[device]) return OK;
+  uint32_t *ptr = nullptr;
+  EXH_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+  g_scratch_ptr[device] = ptr;
+  return OK;
+}
+
+int dot_pairs_static_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uint32_t *out) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  if (len > STATIC_DOT_MAX_LEN) {
+    set_error("invalid-parameter: dot-pairs without allocation takes tables of at most 2^26 EXT8s");
+    return E_PARAM;
+  }
+  uint32_t *partials = c.device >= 0 && c.device < STATIC_MAX_DEVICES ? g_scratch_ptr[c.device] : nullptr;
+  if (!partials) {
+    set_error("device-error: the static scratch array was not set up on this device");
+    return E_DEVICE;
+  }
+  const uint64_t n_pairs = len / 2;
+  const uint32_t grid = (uint32_t)std::min<uint64_t>((n_pairs + BLOCK - 1) / BLOCK, STATIC_DOT_GRID);
+  hipLaunchKernelGGL(dot_pairs_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, d_e, d_v, n_pairs, partials);
+  hipLaunchKernelGGL(sum_columns_to_host_kernel, dim3(24), dim3(BLOCK), 0, c.stream, partials, grid, 24u,
+                     c.host_pinned_dev + STATIC_DOT_RESULT_AT);
+  EXH_HIP(hipGetLastError());
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  memcpy(out, c.host_pinned + STATIC_DOT_RESULT_AT, 96);
+  return OK;
+}
+
 // FOLD-TABLE (src/field.lisp:365-370) of extension tables
 template <int D>
 __global__ __launch_bounds__(BLOCK) void fold_table_kernel(const uint32_t *in, uint32_t *out, uint64_t n_out,

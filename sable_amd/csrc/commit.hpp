@@ -15,6 +15,9 @@ int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d
                    uint32_t *d_out);
 // DOT-PAIRS (src/pcs.lisp:473-483) of two device tables of len EXT8s, parities 0, 1, 2 -> out[3][8] (host)
 int dot_pairs_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uint32_t *out);
+// the same without any allocation (a static device array holds the partial sums); setup: once per device, at init
+int dot_pairs_static_setup(int device);
+int dot_pairs_static_device(const uint32_t *d_e, const uint32_t *d_v, uint64_t len, uint32_t *out);
 // FOLD-TABLE (src/field.lisp:365-370): d_out[i] = in[2i] + r (in[2i+1] - in[2i]) for len extension elements
 int fold_table_device(int D, const uint32_t *d_in, uint64_t len, const uint32_t *r, uint32_t *d_out);
 // d_out[x] = d_h[x] (null: zero) + scale * d_column[x] over len extension elements (src/pcs.lisp:709-716)

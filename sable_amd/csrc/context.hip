@@ -1,6 +1,8 @@
 // context.hip -- see context.hpp.
 #include "context.hpp"
 
+#include "commit.hpp"
+
 namespace exh {
 
 static Context g_ctx;
@@ -136,6 +138,10 @@ int ctx_init(int device) {
   // coherent and mapped: a kernel writes a sumcheck's logs into it directly and the host polls for them
   EXH_HIP(hipHostMalloc((void **)&c.host_pinned, c.host_pinned_words * 4, hipHostMallocMapped | hipHostMallocCoherent));
   EXH_HIP(hipHostGetDevicePointer((void **)&c.host_pinned_dev, c.host_pinned, 0));
+  {  // the device address of the static scratch array, with this device current
+    int scratch_status = dot_pairs_static_setup(device);
+    if (scratch_status) return scratch_status;
+  }
   c.device = device;
   c.compute_units = prop.multiProcessorCount;
   c.ready = true;
