@@ -33,9 +33,11 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
   if (status) return status;
   absorb_header(tr, label, n, degree, bw ? K : 1);
   if (device_rounds && s.device_capable()) {
-    // the rounds run back to back on the device, transcript included; the messages are then replayed
-    // into this transcript, which must draw the same challenges
-    DevB3S state;
+    // the rounds run back to back on the device, transcript included.  This transcript then takes the messages
+    // as they were sent and the hash state the device's transcript ended in; with EXACTA_HIP_REPLAY=1 it absorbs
+    // the messages itself instead and checks that it draws the same challenges (a diagnostic: the two
+    // transcripts are the same function, and the tests hold the device's to the oracle's bytes)
+    DevB3S state, final_state;
     memcpy(state.cv, tr.state.cv, 32);
     for (int i = 0; i < 16; i++)
       state.block[i] = (uint32_t)tr.state.block[4 * i] | (uint32_t)tr.state.block[4 * i + 1] << 8 |
@@ -43,25 +45,34 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
     state.used = tr.state.used;
     state.counter_lo = (uint32_t)tr.state.counter, state.counter_hi = (uint32_t)(tr.state.counter >> 32);
     std::vector<uint32_t> messages((size_t)n * points * D), challenges((size_t)n * D);
-    int replayed = 0;
-    auto replay = [&](int upto) -> int {
-      for (; replayed < upto; replayed++) {
-        const int j = replayed;
-        uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
-        int st_send = tr.send(&messages[(size_t)j * points * D], 2, dims, nullptr);
-        if (st_send) return st_send;
-        uint32_t *r = out_chal + (size_t)j * D;
+    if ((status = s.run_device(state, messages.data(), challenges.data(), &final_state))) return status;
+    const char *replay = getenv("EXACTA_HIP_REPLAY");
+    const bool replaying = replay && replay[0] == '1';
+    for (int j = 0; j < n; j++) {
+      uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
+      int st_send = tr.send(&messages[(size_t)j * points * D], 2, dims, nullptr, replaying);
+      if (st_send) return st_send;
+      uint32_t *r = out_chal + (size_t)j * D;
+      if (replaying) {
         tr.challenge(D, r);
         if (memcmp(r, &challenges[(size_t)j * D], 4 * D) != 0) {
           set_error("device-error: the device transcript drew a different challenge in round " + std::to_string(j));
           return E_DEVICE;
         }
+      } else {
+        memcpy(r, &challenges[(size_t)j * D], 4 * D);
       }
-      return OK;
-    };
-    // the leading rounds are replayed while the device still works on the last ones
-    if ((status = s.run_device(state, messages.data(), challenges.data(), replay))) return status;
-    if ((status = replay(n))) return status;
+    }
+    if (!replaying) {
+      if (final_state.used > 64) {
+        set_error("device-error: the device transcript's final state is malformed");
+        return E_DEVICE;
+      }
+      memcpy(tr.state.cv, final_state.cv, 32);
+      for (int i = 0; i < 64; i++) tr.state.block[i] = (uint8_t)(final_state.block[i / 4] >> (8 * (i % 4)));
+      tr.state.used = final_state.used;
+      tr.state.counter = ((uint64_t)final_state.counter_hi << 32) | final_state.counter_lo;
+    }
     return s.finish(out_finals, out_folded);
   }
   uint32_t sums[16 * 8];

@@ -492,6 +492,18 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   return OK;
 }
 
+// [deg][m] = 1 / prod_{q != m, q <= deg} (m - q), in Montgomery form: the denominators of the Lagrange basis
+// over the nodes 0..deg
+static void fill_inv_den(uint32_t *out) {
+  for (int deg = 1; deg <= MAXDEG; deg++)
+    for (int m = 0; m <= deg; m++) {
+      uint32_t den = 1;
+      for (int q = 0; q <= deg; q++)
+        if (q != m) den = fmul(den, m > q ? (uint32_t)(m - q) : P - (uint32_t)(q - m));
+      out[deg * (MAXDEG + 1) + m] = to_mont(finv(den));
+    }
+}
+
 // Rounds 0 and 1 from one sweep of the base tables (nothing folded): the slot sums in as many launches as the
 // generated kernels need, then the epilogue that sends both rounds' messages.
 template <int D>
@@ -530,13 +542,7 @@ static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs) {
     e.deg[g] = (uint32_t)s.desc.deg[g], e.nev[g] = (uint32_t)s.desc.nev[g];
     for (int k = 0; k < s.desc.nev[g]; k++) e.ev[g][k] = (uint8_t)s.desc.ev[g][k];
   }
-  for (int deg = 1; deg <= MAXDEG; deg++)
-    for (int m = 0; m <= deg; m++) {
-      uint32_t den = 1;
-      for (int q = 0; q <= deg; q++)
-        if (q != m) den = fmul(den, m > q ? (uint32_t)(m - q) : P - (uint32_t)(q - m));
-      e.inv_den[deg * (MAXDEG + 1) + m] = to_mont(finv(den));
-    }
+  fill_inv_den(e.inv_den);
   c.prof_begin("epilogue", 0, 0);
   if (D == 4)
     hipLaunchKernelGGL(nodes_epilogue_kernel<4>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
@@ -738,8 +744,7 @@ static uint64_t tail_pairs(int T, int D) {
   return p;
 }
 
-int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges,
-                                const std::function<int(int)> &early) {
+int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges, DevB3S *final_state) {
   Context &c = ctx();
   if (int owned = owns_arenas()) return owned;
   if (round != 0 || pending_fold || claim_mode || !device_capable()) {
@@ -890,8 +895,6 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   uint32_t *down = c.host_pinned + PIN_DOWN;
   const size_t ctrl_words = (sizeof(Ctrl) + 3) / 4;
   bool logged_to_host = false;
-  int early_rounds = 0;  // leading rounds already handed to `early`
-  bool early_on = false;
   if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
     // when a single entry per table is left at the end (the finals travel in the control block), the launch
     // itself delivers the control block to pinned host memory
@@ -899,13 +902,11 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     if (deliver) {
       if (++c.log_seq == 0) ++c.log_seq;  // 0 is what the flag is reset to
       host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = c.log_seq;
-      host_early = early ? 1 : 0;
-      early_on = host_early != 0;
       reinterpret_cast<volatile uint32_t *>(down)[ctrl_words] = 0;
       reinterpret_cast<volatile uint32_t *>(down)[ctrl_words + 1] = 0;
     }
     status = launch_tail(j, n - j, 1, folds_due > 0);
-    host_log = nullptr, host_early = 0;
+    host_log = nullptr;
     folds_due = 0;
     tail_done = status == OK;
     logged_to_host = deliver && tail_done;
@@ -923,24 +924,6 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     volatile uint32_t *flag = reinterpret_cast<volatile uint32_t *>(down) + ctrl_words;
     uint32_t spins = 0;
     while (*flag != c.log_seq) {
-      const uint32_t word = flag[1];
-      if (early_on && (word >> 6) == (c.log_seq & 0x03ffffffu) && (int)(word & 63) > early_rounds) {
-        // more leading rounds are in: hand them on meanwhile
-        std::atomic_thread_fence(std::memory_order_acquire);
-        const int upto = std::min<int>((int)(word & 63), n);
-        const Ctrl *rc = reinterpret_cast<const Ctrl *>(down);
-        for (int r = early_rounds; r < upto; r++) {
-          memcpy(messages + (size_t)r * points * D, rc->msg[r], (size_t)points * D * 4);
-          memcpy(challenges + (size_t)r * D, rc->chal[r], (size_t)D * 4);
-        }
-        early_rounds = upto;
-        const int early_status = early(upto);
-        if (early_status) {
-          (void)hipStreamSynchronize(c.stream);  // nothing of this session is left running
-          return early_status;
-        }
-        continue;
-      }
       if ((++spins & 1023) == 0 && hipStreamQuery(c.stream) == hipSuccess) break;
     }
     if (*flag != c.log_seq) {
@@ -969,6 +952,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     memcpy(messages + (size_t)r * points * D, rc->msg[r], (size_t)points * D * 4);
     memcpy(challenges + (size_t)r * D, rc->chal[r], (size_t)D * 4);
   }
+  if (final_state) *final_state = rc->tr;
   round = n;
   pending_fold = folds_due > 0;  // after a round kernel the last challenge's fold is still to do
   if (pending_fold) memcpy(pending_r, rc->chal[n - 1], (size_t)D * 4);
@@ -1010,7 +994,7 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
     a.pstride = pstride;
     a.groups = groups;
     a.spin_limit = 200000;
-    a.host_log = host_log, a.host_flag_at = host_flag_at, a.host_seq = host_seq, a.host_early = host_early;
+    a.host_log = host_log, a.host_flag_at = host_flag_at, a.host_seq = host_seq;
     for (int jj = 0; jj < rounds; jj++) {
       a.low_off[jj] = low_off[j + jj];
       a.high_off[jj] = high_off[j + jj];

@@ -48,7 +48,7 @@ struct SumcheckSession {
   unsigned long long *d_slice_totals = nullptr;  // the totals of the grid launch of slices
   bool slice_totals_clear = false;               // cleared by the session's set-up kernel and not used since
   uint32_t *host_log = nullptr;                  // set around the loop's last launch: where it delivers the logs
-  uint32_t host_flag_at = 0, host_seq = 0, host_early = 0;
+  uint32_t host_flag_at = 0, host_seq = 0;
   uint64_t max_grid = 0;
   uint32_t pstride = 0;  // words per workgroup partial
   int node_slots_n = 0;  // slot sums of the base-field sweep that serves rounds 0 and 1
@@ -84,11 +84,9 @@ struct SumcheckSession {
   int round_sums(uint32_t *out /* points * D */);
   // All rounds on the device without a host round trip: the transcript runs on the device from the
   // given B3S state; afterwards messages[j] (points * D words) and challenges[j] (D words) hold what
-  // was sent and drawn, and the session is ready for finish().  Needs points <= MAXPTS.
-  // early (optional): called once, while the last launch still runs, with the count of leading rounds whose
-  // messages and challenges are already in place; a non-zero return ends the call with that status
-  int run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges,
-                 const std::function<int(int)> &early = nullptr);
+  // was sent and drawn, final_state (optional) the transcript's hash state after the last challenge, and the
+  // session is ready for finish().  Needs points <= MAXPTS.
+  int run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges, DevB3S *final_state = nullptr);
   // rounds first_round .. first_round + rounds - 1 with the tables in LDS, over `grid` workgroups
   int launch_tail(int first_round, int rounds, uint32_t grid, bool first_fold);
   bool device_capable() const { return points <= MAXPTS && n <= MAXROUNDS; }

@@ -27,7 +27,6 @@ namespace exh {
 
 // StmtDesc and the limits MAXT, MAXG, ... come from stmtdesc.hpp
 constexpr int MAXROUNDS = 48;  // rounds of one device-driven sumcheck (a count of them fits six bits)
-constexpr uint32_t COURIER_STEP = 1;  // the last launch sends finished rounds to the host every so many rounds
 constexpr int MAXPTS = 7;      // wire points of a device-driven round message
 constexpr int MAXTAIL = 16;    // rounds the tail kernel can take
 
@@ -95,9 +94,6 @@ struct TailArgs {
   // on the stream to read the logs (null: it does both)
   uint32_t *host_log;
   uint32_t host_flag_at, host_seq;
-  // host_early: the launch also delivers finished rounds' messages and challenges as it goes, counting them in
-  // host_log[host_flag_at + 1] as (host_seq << 6) | rounds, so the host can work on them while this one runs
-  uint32_t host_early;
 };
 
 template <int D>
@@ -185,9 +181,12 @@ __device__ __forceinline__ void v_mul_acc(Acc96 *acc, uint32_t a, uint32_t b) { 
 template <int D>
 __device__ __forceinline__ void v_mul_acc(Acc96 *acc, const Ext<D> &a, const Ext<D> &b) { ext_mul_acc<D>(acc, a, b); }
 
-template <int D, class V, class Desc>
+// With PARTS > 1 only the accumulators a with a % PARTS == part are computed (part is uniform over the
+// wavefront): the last rounds, with a pair per lane and lanes to spare, give each of a workgroup's wavefronts a
+// share of a pair's accumulators, so that a round waits for a quarter of the products.
+template <int D, class V, class Desc, int PARTS = 1>
 __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, const V *hi, const Ext<D> &w,
-                                                Acc96 (*acc)[D]) {
+                                                Acc96 (*acc)[D], uint32_t part = 0) {
   V cur[MAXT], slope[MAXT];
 #pragma unroll
   for (int t = 0; t < MAXT; t++)
@@ -244,7 +243,7 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
 #pragma unroll
           for (int k = 0; k < MAXEV; k++) {
             if (k < d.nev[g]) {
-              if (d.ev[g][k] == x) {
+              if (d.ev[g][k] == x && (PARTS == 1 || (uint32_t)(a % PARTS) == part)) {
                 // the product of the factors but the last; the last goes with the accumulation
                 const bool pre = EXT && d.nev[g] >= 3 && d.deg[g] >= 2;
                 V prod = pre ? wcur[g] : cur[d.tab[g][0]];
@@ -264,6 +263,11 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
     }
   }
 }
+
+// A workgroup barrier that orders LDS traffic only: what the threads of a workgroup hand each other in these
+// kernels lives in LDS, and a full barrier would also wait for every global access in flight (the weights fetched
+// a round ahead, the rows on their way to the host).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // cross-lane sum of a canonical value over the 64 lanes of a wavefront: four DPP butterfly steps inside
 // each row of 16 lanes (no LDS traffic), then the four row sums through read-lane
@@ -507,14 +511,46 @@ __device__ __forceinline__ void block_sums(const Desc &d, Acc96 (*acc)[D], uint3
       }
     }
   }
-  __syncthreads();
+  lds_barrier();
   for (uint32_t o = tid; o < (uint32_t)d.nacc * D; o += BLOCK) {
     uint32_t v = lds[0][o];
 #pragma unroll
     for (int wv = 1; wv < BLOCK / 64; wv++) v = fadd(v, lds[wv][o]);
     sums[o] = v;
   }
-  __syncthreads();
+  lds_barrier();
+}
+
+// The wavefront's sums of the accumulators a = PART, PART + PARTS, ... (the ones accumulate_pair<.., PARTS> fills
+// on the wavefront that has this part), reduced mod p, into sums[a * D ..] (LDS).  Every word of sums is written
+// by one wavefront.
+template <int D, int PART, int PARTS, int W, class Desc>
+__device__ __forceinline__ void part_chunk_sums(const Desc &d, Acc96 (*acc)[D], int first, int count, uint32_t *sums) {
+  const uint32_t total = wave_sums_transposed<W>([&](int k) -> uint32_t {
+    const int o = first + k, q = o / D;
+    return PARTS * q + PART < MAXACC && q < count ? acc_reduce(acc[(PARTS * q + PART) % MAXACC][o % D]) : 0u;
+  });
+  const uint32_t l = threadIdx.x & 63;
+  constexpr int BITS = W == 32 ? 5 : W == 16 ? 4 : 3;
+  uint32_t idx = 0;
+#pragma unroll
+  for (int b = 0; b < BITS; b++) idx |= ((l >> b) & 1u) << (BITS - 1 - b);
+  const uint32_t o = first + idx;
+  if (l < W && o < (uint32_t)count * D) sums[(PARTS * (o / D) + PART) * D + o % D] = total;
+}
+template <int D, int PART, int PARTS, class Desc>
+__device__ __forceinline__ void part_wave_sums(const Desc &d, Acc96 (*acc)[D], uint32_t *sums) {
+  const int count = (d.nacc - PART + PARTS - 1) / PARTS;  // accumulators of this part
+  if (count <= 0) return;
+  if (count * D <= 8)
+    part_chunk_sums<D, PART, PARTS, 8>(d, acc, 0, count, sums);
+  else if (count * D <= 16)
+    part_chunk_sums<D, PART, PARTS, 16>(d, acc, 0, count, sums);
+  else {
+#pragma unroll
+    for (int first = 0; first < ((MAXACC + PARTS - 1) / PARTS) * D; first += 32)
+      if (first < count * D) part_chunk_sums<D, PART, PARTS, 32>(d, acc, first, count, sums);
+  }
 }
 
 // From the round's accumulator sums (LDS, nacc * D words, scaled as the kernels leave them) to the round
@@ -547,13 +583,13 @@ __device__ __forceinline__ void round_message(const uint32_t *sums, uint32_t nac
 #pragma unroll
     for (int c = 0; c < D; c++) e->prod[u * D + c] = pr.c[c];
   }
-  __syncthreads();
+  lds_barrier();
   for (uint32_t o = tid; o < points * D; o += nthreads) {
     uint32_t k = o / D, c = o % D, v = c0[o];
     for (uint32_t a = 0; a < nacc; a++) v = fadd(v, e->prod[(k * nacc + a) * D + c]);
     e->msg[o] = v;
   }
-  __syncthreads();
+  lds_barrier();
 }
 
 // the first wavefront's part: send the message, draw the challenge, log both (every lane the same steps)
@@ -772,35 +808,6 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   const uint32_t tid = threadIdx.x, cap = args.capacity, G = gridDim.x, wg = blockIdx.x;
   const uint32_t width = (uint32_t)d.nacc * D;
   if (args.ctrl->round != args.first_round) return;  // an earlier launch gave up: leave the count as it is
-  // The courier: with host_early, the last wavefront carries finished rounds' rows (message, challenge) to the
-  // host log while the launch runs, and publishes in host_log[host_flag_at + 1] how many leading rounds are
-  // there (with the delivery's sequence number above the count's six bits).  The rounds before this launch go
-  // out at once; a round of this launch goes out at the start of a later one, and is published a delivery after
-  // that, when its stores have long landed and the release costs no wait.
-  const bool courier = args.host_log && args.host_early && G == 1;
-  uint32_t carried = courier ? args.first_round : 0;  // rounds whose rows have been stored to the host log
-  auto carry_rows = [&](uint32_t from, uint32_t upto) {
-    const uint32_t lane = tid - (BLOCK - 64), mw = args.points * D;
-    const uint32_t *words = reinterpret_cast<const uint32_t *>(args.ctrl);
-    for (uint32_t u = from * mw + lane; u < upto * mw; u += 64) {
-      const uint32_t at = (uint32_t)(offsetof(Ctrl, msg) / 4) + (u / mw) * (MAXPTS * 8) + u % mw;
-      args.host_log[at] = __hip_atomic_load(words + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    for (uint32_t u = from * D + lane; u < upto * D; u += 64) {
-      const uint32_t at = (uint32_t)(offsetof(Ctrl, chal) / 4) + (u / D) * 8 + u % D;
-      args.host_log[at] = __hip_atomic_load(words + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  };
-  auto publish = [&](uint32_t count) {
-    __threadfence_system();
-    if (tid == BLOCK - 64)
-      __hip_atomic_store(args.host_log + args.host_flag_at + 1, (args.host_seq << 6) | count, __ATOMIC_RELEASE,
-                         __HIP_MEMORY_SCOPE_SYSTEM);
-  };
-  if (courier && args.first_round > 0 && tid >= BLOCK - 64) {
-    carry_rows(0, args.first_round);
-    publish(args.first_round);
-  }
   RunB3S tr;
   if (tid < 64) rb3s_load(tr, epi.ring, &args.ctrl->tr);
   uint32_t entries = (args.first_fold ? args.entries / 2 : args.entries) / G;  // of this workgroup's slice
@@ -839,106 +846,148 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   }
   // the weight factors of this thread's first pair of a round, fetched one round ahead
   Ext<D> wl = ext_zero<D>(), wh = ext_zero<D>();
+  // (a round of at most 64 pairs runs with a pair per lane on all four wavefronts, each computing a share of the
+  // pair's accumulators)
+  const uint32_t lane = tid & 63, wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+  // (every thread loads, from a clamped index: a load under a condition has to be merged with the old value as soon
+  // as it is issued, which turns the prefetch into a wait for memory at the end of every round)
   auto fetch_weight = [&](uint32_t jj, uint32_t pairs) {
-    if (tid < pairs) {
-      const uint64_t i = (uint64_t)wg * pairs + tid;
-      wl = load_ext<D>(args.weights + (args.low_off[jj] + (i & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
-      wh = load_ext<D>(args.weights + (args.high_off[jj] + (i >> args.low_bits[jj])) * D);
-    }
+    const uint32_t me = pairs <= 64 ? lane : tid;
+    const uint64_t i = (uint64_t)wg * pairs + (me < pairs ? me : pairs - 1);
+    wl = load_ext<D>(args.weights + (args.low_off[jj] + (i & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
+    wh = load_ext<D>(args.weights + (args.high_off[jj] + (i >> args.low_bits[jj])) * D);
+  };
+  // a fold of `count` outputs by r, a table per wavefront, in place: the lanes run in lockstep, so every read of
+  // a chunk of 64 comes before its writes, and those land below what later chunks read
+  auto fold_small = [&](const Ext<D> &r, uint32_t count) {
+#pragma unroll
+    for (int t = 0; t < MAXT; t++)
+      if (t < d.T && (uint32_t)(t & 3) == wave) {
+        for (uint32_t x = lane; x < count; x += 64) {
+          const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * x) * D;
+          const Ext<D> folded = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
+          store_ext<D>(tail_tables + ((size_t)t * cap + x) * D, folded);
+        }
+      }
   };
   fetch_weight(0, entries / 2);
   __syncthreads();
   for (uint32_t jj = 0; jj < args.rounds; jj++) {
     const uint32_t pairs = entries / 2;
-    if (courier && jj > 0 && jj % COURIER_STEP == 0) {
-      if (tid >= BLOCK - 64) {
-        if (carried > args.first_round) publish(carried);
-        carry_rows(carried, args.first_round + jj);
-      }
-      carried = args.first_round + jj;
-    }
-    Acc96 acc[MAXACC][D];
+    const bool small = pairs <= 64 && BLOCK == 256;
+    {  // the round's sums
+      Acc96 acc[MAXACC][D];
 #pragma unroll
-    for (int a = 0; a < MAXACC; a++)
+      for (int a = 0; a < MAXACC; a++)
 #pragma unroll
-      for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
-    for (uint32_t i = tid; i < pairs; i += BLOCK) {
-      Ext<D> lo[MAXT], hi[MAXT];
-#pragma unroll
-      for (int t = 0; t < MAXT; t++)
-        if (t < d.T) {
-          const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * i) * D;
-          lo[t] = load_ext<D>(p);
-          hi[t] = load_ext<D>(p + D);
-        }
-      if (i >= BLOCK) {  // beyond the prefetched pair
-        const uint64_t gi = (uint64_t)wg * pairs + i;
-        wl = load_ext<D>(args.weights + (args.low_off[jj] + (gi & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
-        wh = load_ext<D>(args.weights + (args.high_off[jj] + (gi >> args.low_bits[jj])) * D);
-      }
-      accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
-    }
-    if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
-    block_sums<D, true>(d, acc, lds, sums);
-    if (G > 1) {
-      // The round's sums over all workgroups.  Each workgroup adds its sums into its group's totals,
-      // one integer atomic per word that also counts the contribution in the word's top 16 bits; a
-      // word whose count equals the group's size is complete, so readers poll the words themselves:
-      // nothing else is exchanged (the tables live in LDS), and no fence or separate barrier is needed.
-      // Groups keep the atomics on one address few.
-      const uint32_t NG = args.groups, gsize = G / NG;
-      unsigned long long *totals = args.totals + (size_t)jj * NG * args.pstride;
-      for (uint32_t o = tid; o < width; o += BLOCK)
-        __hip_atomic_fetch_add(totals + (size_t)(wg % NG) * args.pstride + o, ((unsigned long long)1 << 48) + sums[o],
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      int complete = 1;
-      for (uint32_t u = tid; u < NG * width; u += BLOCK) {
-        const unsigned long long *word = totals + (size_t)(u / width) * args.pstride + u % width;
-        unsigned long long v;
-        uint32_t polls = 0;
-        while (((v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 48) != gsize) {
-          if (++polls > args.spin_limit) {  // the grid is not all there: give up, the host sees the round count
-            complete = 0;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(1);
-        }
-        epi.prod[u] = f_canonical((double)(v & (((unsigned long long)1 << 48) - 1)));  // exact below 2^53
-      }
-      if (!__syncthreads_and(complete)) return;
-      for (uint32_t o = tid; o < width; o += BLOCK) {
-        uint32_t v = 0;
-        for (uint32_t g = 0; g < NG; g++) v = fadd(v, epi.prod[g * width + o]);
-        sums[o] = v;
-      }
-      __syncthreads();
-    }
-    round_message<D>(sums, (uint32_t)d.nacc, args.points, epi.mtilde, c0s + (size_t)jj * args.points * D, &epi);
-    if (tid < 64) transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi, wg == 0);
-    __syncthreads();
-    Ext<D> r;
-#pragma unroll
-    for (int c = 0; c < D; c++) r.c[c] = epi.r_mont[c];
-    // fold in place, 256 entries at a time in ascending order: a chunk's reads come before its writes,
-    // and its writes land below everything a later chunk reads
-    for (uint32_t base = 0; base < pairs; base += BLOCK) {
-      const uint32_t x = base + tid;
-      Ext<D> folded[MAXT];
-      if (x < pairs) {
+        for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
+      if (small && lane < pairs) {
+        Ext<D> lo[MAXT], hi[MAXT];
 #pragma unroll
         for (int t = 0; t < MAXT; t++)
           if (t < d.T) {
-            const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * x) * D;
-            folded[t] = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
+            const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * lane) * D;
+            lo[t] = load_ext<D>(p);
+            hi[t] = load_ext<D>(p + D);
           }
+        accumulate_pair<D, Ext<D>, Desc, 4>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc, wave);
       }
-      __syncthreads();
-      if (x < pairs) {
+      for (uint32_t i = tid; i < pairs && !small; i += BLOCK) {
+        Ext<D> lo[MAXT], hi[MAXT];
 #pragma unroll
         for (int t = 0; t < MAXT; t++)
-          if (t < d.T) store_ext<D>(tail_tables + ((size_t)t * cap + x) * D, folded[t]);
+          if (t < d.T) {
+            const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * i) * D;
+            lo[t] = load_ext<D>(p);
+            hi[t] = load_ext<D>(p + D);
+          }
+        if (i >= BLOCK) {  // beyond the prefetched pair
+          const uint64_t gi = (uint64_t)wg * pairs + i;
+          wl = load_ext<D>(args.weights + (args.low_off[jj] + (gi & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
+          wh = load_ext<D>(args.weights + (args.high_off[jj] + (gi >> args.low_bits[jj])) * D);
+        }
+        accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
       }
-      __syncthreads();
+      if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
+      if (small) {
+        if (wave == 0)
+          part_wave_sums<D, 0, 4>(d, acc, sums);
+        else if (wave == 1)
+          part_wave_sums<D, 1, 4>(d, acc, sums);
+        else if (wave == 2)
+          part_wave_sums<D, 2, 4>(d, acc, sums);
+        else
+          part_wave_sums<D, 3, 4>(d, acc, sums);
+        lds_barrier();
+      } else {
+        block_sums<D, true>(d, acc, lds, sums);
+      }
+      if (G > 1) {
+        // The round's sums over all workgroups.  Each workgroup adds its sums into its group's totals,
+        // one integer atomic per word that also counts the contribution in the word's top 16 bits; a
+        // word whose count equals the group's size is complete, so readers poll the words themselves:
+        // nothing else is exchanged (the tables live in LDS), and no fence or separate barrier is needed.
+        // Groups keep the atomics on one address few.
+        const uint32_t NG = args.groups, gsize = G / NG;
+        unsigned long long *totals = args.totals + (size_t)jj * NG * args.pstride;
+        for (uint32_t o = tid; o < width; o += BLOCK)
+          __hip_atomic_fetch_add(totals + (size_t)(wg % NG) * args.pstride + o, ((unsigned long long)1 << 48) + sums[o],
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int complete = 1;
+        for (uint32_t u = tid; u < NG * width; u += BLOCK) {
+          const unsigned long long *word = totals + (size_t)(u / width) * args.pstride + u % width;
+          unsigned long long v;
+          uint32_t polls = 0;
+          while (((v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 48) != gsize) {
+            if (++polls > args.spin_limit) {  // the grid is not all there: give up, the host sees the round count
+              complete = 0;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+          }
+          epi.prod[u] = f_canonical((double)(v & (((unsigned long long)1 << 48) - 1)));  // exact below 2^53
+        }
+        if (!__syncthreads_and(complete)) return;
+        for (uint32_t o = tid; o < width; o += BLOCK) {
+          uint32_t v = 0;
+          for (uint32_t g = 0; g < NG; g++) v = fadd(v, epi.prod[g * width + o]);
+          sums[o] = v;
+        }
+        lds_barrier();
+      }
+    }
+    {  // the message, the challenge, the fold
+      round_message<D>(sums, (uint32_t)d.nacc, args.points, epi.mtilde, c0s + (size_t)jj * args.points * D, &epi);
+      if (tid < 64) transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi, wg == 0);
+      lds_barrier();
+      Ext<D> r;
+#pragma unroll
+      for (int c = 0; c < D; c++) r.c[c] = epi.r_mont[c];
+      if (small) {
+        fold_small(r, pairs);
+        lds_barrier();
+      }
+      // fold in place, 256 entries at a time in ascending order: a chunk's reads come before its writes,
+      // and its writes land below everything a later chunk reads
+      for (uint32_t base = 0; base < pairs && !small; base += BLOCK) {
+        const uint32_t x = base + tid;
+        Ext<D> folded[MAXT];
+        if (x < pairs) {
+#pragma unroll
+          for (int t = 0; t < MAXT; t++)
+            if (t < d.T) {
+              const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * x) * D;
+              folded[t] = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
+            }
+        }
+        lds_barrier();
+        if (x < pairs) {
+#pragma unroll
+          for (int t = 0; t < MAXT; t++)
+            if (t < d.T) store_ext<D>(tail_tables + ((size_t)t * cap + x) * D, folded[t]);
+        }
+        lds_barrier();
+      }
     }
     entries = pairs;
   }
@@ -963,11 +1012,10 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
       args.host_log[at] = __hip_atomic_load(words + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
     const uint32_t all_rounds = args.first_round + args.rounds, mw = args.points * D;
-    const uint32_t from = carried;  // the rounds before have gone out already
     for (uint32_t u = tid; u < offsetof(Ctrl, msg) / 4; u += BLOCK) deliver(u);
-    for (uint32_t u = from * mw + tid; u < all_rounds * mw; u += BLOCK)
+    for (uint32_t u = tid; u < all_rounds * mw; u += BLOCK)
       deliver((uint32_t)(offsetof(Ctrl, msg) / 4) + (u / mw) * (MAXPTS * 8) + u % mw);
-    for (uint32_t u = from * D + tid; u < all_rounds * D; u += BLOCK)
+    for (uint32_t u = tid; u < all_rounds * D; u += BLOCK)
       deliver((uint32_t)(offsetof(Ctrl, chal) / 4) + (u / D) * 8 + u % D);
     for (uint32_t u = tid; u < (uint32_t)d.T * D; u += BLOCK) deliver((uint32_t)(offsetof(Ctrl, finals) / 4) + u);
     __threadfence_system();

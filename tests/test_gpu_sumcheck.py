@@ -319,3 +319,29 @@ def test_base_field_sweep_with_block_weights(K, n, d, with_eq, monkeypatch):
     consts = rand_ext(rng, (1,), d)
     prove_both("nodes-bw", d, n, CONFIG2, ["t0", "t1", "t2"], tables, eq=eq, constants=consts, cnames=["alpha"],
                block_weights=bw)
+
+
+@pytest.mark.parametrize("n", [6, 19])
+def test_host_replay_of_the_device_transcript(n, monkeypatch):
+    """By default the host transcript takes the device transcript's final hash state; with EXACTA_HIP_REPLAY=1 it
+    absorbs the logged messages itself and must draw the same challenges.  Same proof bytes, and the transcript
+    goes on identically afterwards, either way."""
+    rng = np.random.default_rng(77 + n)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in range(3)]
+    eq, alpha = rand_ext(rng, (n,), 4), rand_ext(rng, (1,), 4)
+    st = sa.Statement(CONFIG2, ["t0", "t1", "t2"], ["alpha"])
+    dev = [sa.Table.upload(t) for t in tables]
+    outs = []
+    for replay in ("0", "1"):
+        monkeypatch.setenv("EXACTA_HIP_REPLAY", replay)
+        tr = sa.Transcript("replay", 4)
+        chal, finals, _ = sa.prove(tr, n, st, dev, eq=eq, constants=alpha)
+        outs.append((tr.proof(), chal.copy(), finals.copy(), tr.challenge().copy(), tr.state_digest()))
+    assert outs[0][0] == outs[1][0] and outs[0][4] == outs[1][4]
+    for a, b in zip(outs[0][1:4], outs[1][1:4]):
+        assert same(a, b)
+    otr = orc.Transcript("replay", 4)
+    orc.prove(otr, n, orc.Statement(CONFIG2, ["t0", "t1", "t2"], ["alpha"]), tables, eq=eq, constants=alpha)
+    assert same(otr.challenge(), outs[0][3])
+    for t in dev:
+        t.free()
