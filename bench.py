@@ -1,13 +1,17 @@
 #!/usr/bin/env python3
-"""Benchmark of the sumcheck proving path on one MI355X.
+"""Benchmark of the proving path on one MI355X.
 
-A step is one whole sumcheck `prove` of the headline workload: statement (+ (* alpha t0 t1 t2) (* 3 t1)) in
-eq mode over three base-field tables of 2^24 seeded uniform KoalaBear elements, F_p^4 challenges, degree-3
-round messages, BLAKE3 transcript -- header absorb to last challenge, finals read back.  The tables are
-resident in HBM before the timed region.  value = 3 * 2^24 table entries / time per step.
+A step is one whole sumcheck `prove` of the headline workload (config 2): statement
+(+ (* alpha t0 t1 t2) (* 3 t1)) in eq mode over three base-field tables of 2^24 seeded uniform KoalaBear elements,
+F_p^4 challenges, degree-3 round messages, BLAKE3 transcript -- header absorb to last challenge, finals read back.
+The tables are resident in HBM before the timed region.  value = 3 * 2^24 table entries / time per step.
 
-Prints one JSON line with the metric, the roofline of the dominant kernel (measured live with HIP events on
-the library's stream) and the CPU oracle timed on a bounded sample of the same workload.
+One JSON line: the metric; `roofline` for the streaming launch with the largest time (HIP events on the library's
+stream) and `roofline_by_time` for every launch of a prove; `int32_mul`, the integer-multiply roofline;
+`cpu_baseline`, the CPU oracle's threaded path on a bounded sample of the same workload (one thread and all host
+threads, best of 7); `other_configs`, the other four configured workloads timed the same way in the same run.
+The timed proof is checked before it is reported: the library's verifier accepts it and its SHA-256 is the one the
+CPU oracle's proof of the same seeded inputs has (tests/golden/config_hashes.json).
 """
 import argparse
 import ctypes as C
@@ -22,24 +26,62 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-FORM, TABLES, CONSTS = "(+ (* alpha t0 t1 t2) (* 3 t1))", ["t0", "t1", "t2"], ["alpha"]
+from sable_amd import workloads as wl  # noqa: E402
+
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# The integer-multiply roofline's peak: one 32-bit multiply (v_mad_u64_u32, v_mul_lo_u32, v_mul_hi_u32) per lane
+# every 4.7 cycles of a SIMD's 16 lanes x 4, as measured with independent chains on this part at 2.4 GHz:
+# 256 CUs x 4 SIMDs x 64 lanes / 4.7 cycles x 2.4e9
+INT32_MUL_PEAK_PER_S = 256 * 4 * 64 / 4.7 * 2.4e9
+
+# Figures that were measured on one version of the kernels and are only reported while the kernels' sources are
+# that version: HBM bytes per launch from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE, each scaled by what
+# the same counter reads for the plain copy kernel of `--workload copy`), and 32-bit integer multiply instructions
+# per lane and prove from the kernels' instruction streams times their trip counts (profiles/ holds both summaries).
+MEASURED = {
+    "kernel_sources_sha256": "",
+    "traffic": {("round_nodes_base", 24): 203495288, ("round_fold2_base", 24): 403802364},
+    "int32_mul_per_prove": None,
+}
+KERNEL_SOURCES = ["sumcheck_kernels.cuh", "field.cuh", "dev_transcript.cuh", "blake3.cuh", "stmtdesc.hpp"]
+
+
+def kernel_sources_sha256():
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "sable_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def sha(b):
+    return hashlib.sha256(bytes(b)).hexdigest()
+
+
+def golden():
+    with open(os.path.join(ROOT, "tests", "golden", "config_hashes.json")) as f:
+        return json.load(f)
 
 
 def splitmix_field(seed, count):
-    """SplitMix64(seed) -> 31-bit words, rejected when >= p: the rule the library's seeded tables use."""
-    P = 2130706433
-    out, x, mask = [], seed, (1 << 64) - 1
+    """SplitMix64(seed) -> 31-bit words, kept when below p: the rule the library's seeded tables use."""
+    P = wl.P
+    out = np.empty(0, np.uint32)
+    mask = (1 << 64) - 1
+    x0 = seed
     while len(out) < count:
-        x = (x + 0x9E3779B97F4A7C15) & mask
-        z = x
-        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
-        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
-        z ^= z >> 31
-        w = z >> 33
-        if w < P:
-            out.append(w)
-    return np.array(out, np.uint32)
+        m = max(64, int((count - len(out)) * 1.02) + 16)
+        idx = np.arange(1, m + 1, dtype=np.uint64)
+        with np.errstate(over="ignore"):
+            x = (np.uint64(x0) + idx * np.uint64(0x9E3779B97F4A7C15)) & np.uint64(mask)
+            z = x
+            z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+            z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+            z = z ^ (z >> np.uint64(31))
+        w = (z >> np.uint64(33)).astype(np.uint32)
+        out = np.concatenate([out, w[w < P]])
+        x0 = int(x[-1])
+    return out[:count].copy()
 
 
 def profile_entries(sa):
@@ -53,257 +95,275 @@ def profile_entries(sa):
     return out
 
 
-def cpu_baseline(sa, n_sample, d, seed):
-    """The CPU oracle (a C restatement of the reference's prover, single thread) on the same statement and
-    seeds at a smaller n, sized for roughly 10-30 s.  The same sample then goes through the GPU path as the
-    checker of this run: the proof bytes must be the oracle's."""
-    from oracle import binding as orc
-    st = orc.Statement(FORM, TABLES, CONSTS)
-    tables = [splitmix_field(seed * 1000 + k, 1 << n_sample) for k in range(3)]
-    eq = splitmix_field(seed + 900, n_sample * d).reshape(n_sample, d)
-    alpha = splitmix_field(seed + 901, d).reshape(1, d)
-    t0 = time.perf_counter()
-    otr = orc.Transcript("config2", d)
-    orc.prove(otr, n_sample, st, tables, eq=eq, constants=alpha)
-    dt = time.perf_counter() - t0
-    dev = [sa.Table.upload(t) for t in tables]
-    tr = sa.Transcript("config2", d)
-    sa.prove(tr, n_sample, sa.Statement(FORM, TABLES, CONSTS), dev, eq=eq, constants=alpha)
-    for t in dev:
-        t.free()
-    if tr.proof() != otr.proof():
-        sys.exit(f"bench.py: the GPU proof at n={n_sample} differs from the CPU oracle's")
-    return {"value": 3 * (1 << n_sample) / dt, "unit": "table entries/s", "cores": 1, "kind": "port",
-            "sample": f"same statement, seeds and transcript at n={n_sample} (3*2^{n_sample} entries, "
-                      f"{dt:.1f} s); the GPU proof of the same sample is byte-identical; the reference's Lisp "
-                      f"prover cannot run here (no SBCL)"}
-
-
-def run_sumcheck_config(sa, name, form, tables, consts, n, d, seed, steps, warmup, cpu_n):
-    """A sumcheck workload other than the headline one: same timing rules, one JSON line."""
-    st = sa.Statement(form, tables, consts)
-    T = len(tables)
-    dev = [sa.Table.random(seed * 1000 + k, 1 << n) for k in range(T)]
-    eq = splitmix_field(seed + 900, n * d).reshape(n, d)
-    cv = splitmix_field(seed + 901, d * max(len(consts), 1)).reshape(-1, d) if consts else None
-
-    def step():
-        tr = sa.Transcript(name, d)
-        sa.prove(tr, n, st, dev, eq=eq, constants=cv)
-        return tr
-
+def timed(sa, step, steps, warmup):
+    """W untimed steps, then exactly K steps between two device-wide waits: seconds per step, last result."""
+    out = None
     for _ in range(warmup):
-        step()
+        out = step()
     sa.check(sa.load().exh_synchronize())
     t0 = time.perf_counter()
     for _ in range(steps):
-        tr = step()
+        out = step()
     sa.check(sa.load().exh_synchronize())
-    dt = (time.perf_counter() - t0) / steps
+    return (time.perf_counter() - t0) / steps, out
+
+
+def launches(sa, step, steps):
+    """Every launch of `steps` more steps, timed with HIP events on the library's stream: per (kernel, round)
+    [average ms, launches per step, algorithmic bytes per launch], and the same summed per kernel name."""
     sa.check(sa.load().exh_profile_enable(1))
     for _ in range(steps):
         step()
-    by_kernel = {}
-    for kname, rnd, ms, nbytes in profile_entries(sa):
-        k = by_kernel.setdefault((kname, rnd), [0.0, 0, nbytes])
+    by = {}
+    for name, rnd, ms, nbytes in profile_entries(sa):
+        k = by.setdefault((name, rnd), [0.0, 0, nbytes])
         k[0] += ms
         k[1] += 1
     sa.check(sa.load().exh_profile_enable(0))
-    (kname, kround), (ktotal, kcalls, kbytes) = max(by_kernel.items(), key=lambda kv: kv[1][0])
-    avg_ms = ktotal / kcalls
-    achieved = kbytes / (avg_ms * 1e-3) / 1e9
-    points = max(st.degree, 1)
-    out = {"metric": f"sumcheck table entries/s ({name})", "value": T * (1 << n) / dt, "unit": "table entries/s",
-           "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": 1e3 * dt, "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": f"u32 (Montgomery KoalaBear, F_p^{d} tower)",
-           "data": "synthetic (SplitMix64-seeded uniform field elements)",
-           "config": {"workload": f"sumcheck prove of {form}, eq mode, n={n}, {T} base tables, F_p^{d}",
-                      "generated_kernel": st.has_generated_kernel(d), "proof_bytes": len(tr.proof()),
-                      "proof_sha256": hashlib.sha256(tr.proof()).hexdigest()},
-           "loop_hbm_fraction": T * (1 << n) * (8 + 8 * d) / dt / (HBM_PEAK_GBS * 1e9),
-           "roofline": {"bound": "hbm", "kernel": f"{kname} (round {kround})", "achieved": achieved,
-                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                        "avg_launch_ms": avg_ms, "alg_bytes_per_launch": kbytes, "traffic": None}}
-    assert len(tr.proof()) == 12 + n * (18 + 4 * points * d)
-    if cpu_n > 0:
-        from oracle import binding as orc
-        ost = orc.Statement(form, tables, consts)
-        ht = [splitmix_field(seed * 1000 + k, 1 << cpu_n) for k in range(T)]
-        heq = splitmix_field(seed + 900, cpu_n * d).reshape(cpu_n, d)
-        t0 = time.perf_counter()
-        orc.prove(orc.Transcript(name, d), cpu_n, ost, ht, eq=heq, constants=cv)
-        cdt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": T * (1 << cpu_n) / cdt, "unit": "table entries/s", "cores": 1, "kind": "port",
-                               "sample": f"same statement at n={cpu_n} ({cdt:.1f} s)"}
-    for t in dev:
-        t.free()
-    return out
+    return {k: (v[0] / v[1], v[1] / steps, v[2]) for k, v in by.items()}
 
 
-def run_gkr(sa, steps, warmup, cpu_n):
-    """Config 4: LogUp-GKR of 2^22 int8-range lookups into a 2^16-entry range table.  The witness tree has
-    leaves (1, Z - v_i), n = 22; the table tree leaves (m_j, Z - t_j), n = 16, t_j = j - 32768, m_j the exact
-    multiplicities; both roots are equal as fractions.  A step = prove-upper of both trees (fraction trees +
-    every layer's sumcheck)."""
-    d, nw, nt, seed = 4, 22, 16, 4
-    rng = np.random.default_rng(seed)
-    values = rng.integers(-128, 128, 1 << nw)
-    table = np.arange(1 << nt) - 32768
-    mult = np.bincount(values + 32768, minlength=1 << nt)
-    z = sa.Transcript("config4-z", d).challenge()
+def by_time(by):
+    total = sum(avg * per for avg, per, _ in by.values())
+    rows = []
+    for (name, rnd), (avg, per, nbytes) in sorted(by.items(), key=lambda kv: -kv[1][0] * kv[1][1]):
+        row = {"kernel": name, "round": rnd, "avg_launch_ms": avg, "launches_per_step": per,
+               "share_of_kernel_time": avg * per / total if total else 0.0, "alg_bytes_per_launch": nbytes}
+        if nbytes:
+            row["hbm_frac"] = nbytes / (avg * 1e-3) / 1e9 / HBM_PEAK_GBS
+        rows.append(row)
+    return rows
 
-    def leaves(num, val):
-        P = sa.P
-        p = np.zeros((len(num), d), np.uint32)
-        p[:, 0] = np.asarray(num, np.int64) % P
-        q = np.tile(z.astype(np.int64), (len(val), 1))
-        q[:, 0] = (q[:, 0] - np.asarray(val, np.int64)) % P
-        return p, q.astype(np.uint32)
 
-    wit = [sa.Table.upload(a) for a in leaves(np.ones(1 << nw, np.int64), values)]
-    tab = [sa.Table.upload(a) for a in leaves(mult, table)]
+# ------------------------------------------------------------------ sumcheck configurations
+def sumcheck_setup(sa, name, n=None):
+    cfg = wl.SUMCHECK[name]
+    n, d, T = n or cfg["n"], cfg["d"], len(cfg["tables"])
+    st = sa.Statement(cfg["form"], cfg["tables"], cfg["constants"])
+    dev = [sa.Table.random(wl.table_seed(cfg, k), 1 << n) for k in range(T)]
+    eq = splitmix_field(wl.eq_seed(cfg), n * d).reshape(n, d)
+    cv = splitmix_field(wl.constants_seed(cfg), d * len(cfg["constants"])).reshape(-1, d) if cfg["constants"] else None
 
     def step():
-        tw, tt = sa.Transcript("config4-w", d), sa.Transcript("config4-t", d)
+        tr = sa.Transcript(name, d)
+        chal, finals, _ = sa.prove(tr, n, st, dev, eq=eq, constants=cv)
+        return tr, finals
+
+    return cfg, n, d, T, st, dev, eq, cv, step
+
+
+def sumcheck_checked(sa, name, n, d, st, dev, eq, cv, tr, finals, gold):
+    """The timed proof before it is reported: the verifier accepts it; at the configured size its digest is the
+    CPU oracle's."""
+    proof = tr.proof()
+    claim = sa.hypercube_sum(st, n, dev, d, eq=eq, constants=cv)
+    vtr = sa.Transcript(name, d, proof=proof)
+    _, reduced = sa.verify(vtr, n, st, claim, eq=eq, constants=cv)
+    if not (vtr.finished() and sa.check_final(reduced, st, finals, constants=cv)):
+        sys.exit(f"bench.py: the verifier rejects the timed {name} proof")
+    want = gold.get(name, {}).get("proof_sha256") if n == wl.SUMCHECK[name]["n"] else None
+    if want is not None and sha(proof) != want:
+        sys.exit(f"bench.py: the timed {name} proof differs from the CPU oracle's")
+    return proof, want is not None
+
+
+def run_sumcheck(sa, name, steps, warmup, gold, n=None):
+    cfg, n, d, T, st, dev, eq, cv, step = sumcheck_setup(sa, name, n)
+    dt, (tr, finals) = timed(sa, step, steps, warmup)
+    proof, pinned = sumcheck_checked(sa, name, n, d, st, dev, eq, cv, tr, finals, gold)
+    by = launches(sa, step, max(2, min(steps, 10)))
+    for t in dev:
+        t.free()
+    streaming = {k: v for k, v in by.items() if k[0].startswith("round_")} or by
+    (kname, kround), (avg_ms, per, kbytes) = max(streaming.items(), key=lambda kv: kv[1][0] * kv[1][1])
+    achieved = kbytes / (avg_ms * 1e-3) / 1e9
+    return {"workload": f"sumcheck prove of {cfg['form']}, eq mode, n={n}, {T} base tables of 2^{n}, F_p^{d}, BLAKE3 "
+                        "transcript", "n": n, "tables": T, "extension": d, "degree": st.degree,
+            "ms_per_step": 1e3 * dt, "entries_per_s": T * (1 << n) / dt, "proof_bytes": len(proof),
+            "proof_sha256": sha(proof), "proof_is_the_cpu_oracles": pinned, "verifier_accepts": True,
+            "generated_kernel": st.has_generated_kernel(d),
+            "loop_hbm_fraction": T * (1 << n) * (8 + 8 * d) / dt / (HBM_PEAK_GBS * 1e9),
+            "roofline": {"bound": "hbm", "kernel": f"{kname} (round {kround})", "achieved": achieved,
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "avg_launch_ms": avg_ms,
+                         "launches_per_step": per, "alg_bytes_per_launch": kbytes, "traffic": None},
+            "roofline_by_time": by_time(by)}
+
+
+# ------------------------------------------------------------------ config 4: LogUp-GKR
+def run_gkr(sa, steps, warmup, gold):
+    g = wl.GKR
+    d, nw, nt = g["d"], g["n_witness"], g["n_table"]
+    z = sa.Transcript(g["z_label"], d).challenge()
+    seeded = sa.Table.random(g["seed"], 1 << nw)
+    words = seeded.download()
+    seeded.free()
+    wit_h, tab_h = wl.gkr_leaves(np, words, z, nw, nt, d)
+    wit = [sa.Table.upload(a) for a in wit_h]
+    tab = [sa.Table.upload(a) for a in tab_h]
+
+    def step():
+        tw, tt = sa.Transcript(g["witness_label"], d), sa.Transcript(g["table_label"], d)
         sa.prove_upper(tw, nw, 1, [tuple(wit)])
         sa.prove_upper(tt, nt, 1, [tuple(tab)])
         return tw, tt
 
-    for _ in range(warmup):
-        step()
-    sa.check(sa.load().exh_synchronize())
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        tw, tt = step()
-    sa.check(sa.load().exh_synchronize())
-    dt = (time.perf_counter() - t0) / steps
-    from oracle import binding as orc
-    rw, rt = orc.decode_proof(tw.proof())[0], orc.decode_proof(tt.proof())[0]
-    same_fraction = np.array_equal(orc.ext_mul(rw[0], rt[1]), orc.ext_mul(rt[0], rw[1]))
-    # algorithmic bytes of prove-upper per tree (16 B entries): tree build 3 * 2 * 2^n * 16 - ..., layer sumchecks
-    def alg(n):
+    dt, (tw, tt) = timed(sa, step, steps, warmup)
+    pinned = True
+    for key, tr, n in (("witness", tw, nw), ("table", tt, nt)):
+        vtr = sa.Transcript(g[key + "_label"], d, proof=tr.proof())
+        sa.verify_upper(vtr, n, 1, 1)
+        if not vtr.finished():
+            sys.exit("bench.py: the verifier rejects the timed GKR proof")
+        want = gold.get("config4", {}).get(key, {}).get("proof_sha256")
+        if want is None:
+            pinned = False
+        elif sha(tr.proof()) != want:
+            sys.exit(f"bench.py: the timed GKR proof ({key} tree) differs from the CPU oracle's")
+    by = launches(sa, step, max(2, min(steps, 5)))
+    for t in wit + tab:
+        t.free()
+
+    def alg(n):  # fraction trees (2 x 16-byte entries read per parent pair, one written) + the layers' sumchecks
         build = sum(2 * (2 << m) * 16 + 2 * (1 << m) * 16 for m in range(n))
         layers = sum(4 * (4 * (1 << l) * 16) for l in range(n - 1))
         return build + layers
+
     nbytes = alg(nw) + alg(nt)
-    out = {"metric": "LogUp-GKR prove-upper lookups/s (config 4)", "value": (1 << nw) / dt, "unit": "lookups/s",
-           "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": 1e3 * dt, "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": "u32 (Montgomery KoalaBear, F_p^4 tower)",
-           "data": "synthetic (seeded uniform int8 lookups, exact multiplicities)",
-           "config": {"workload": "LogUp-GKR: 2^22 int8-range lookups into a 2^16-entry table, witness tree n=22 + "
-                                  "table tree n=16, F_p^4, prove-upper of both", "roots_equal_as_fractions": bool(same_fraction),
-                      "proof_bytes": len(tw.proof()) + len(tt.proof())},
-           "roofline": {"bound": "hbm", "kernel": "prove-upper (whole: tree build + 36 layer sumchecks)",
-                        "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "alg_bytes": nbytes, "traffic": None}}
-    if cpu_n > 0:
-        rng = np.random.default_rng(1)
-        p = rng.integers(0, sa.P, (1 << cpu_n, d), dtype=np.uint32)
-        q = rng.integers(1, sa.P, (1 << cpu_n, d), dtype=np.uint32)
-        t0 = time.perf_counter()
-        orc.gkr_prove_upper(orc.Transcript("config4-w", d), cpu_n, 1, [(p, q)])
-        cdt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": (1 << cpu_n) / cdt, "unit": "lookups/s", "cores": 1, "kind": "port",
-                               "sample": f"prove-upper of one tree of 2^{cpu_n} leaves ({cdt:.1f} s)"}
-    return out
+    return {"workload": "LogUp-GKR: 2^22 int8-range lookups into a 2^16-entry table, witness tree n=22 + table tree "
+                        "n=16, F_p^4, prove-upper of both", "ms_per_step": 1e3 * dt, "lookups_per_s": (1 << nw) / dt,
+            "proof_bytes": len(tw.proof()) + len(tt.proof()), "proof_sha256": [sha(tw.proof()), sha(tt.proof())],
+            "proof_is_the_cpu_oracles": pinned, "verifier_accepts": True,
+            "timed_launches_per_step": sum(per for _, per, _ in by.values()),
+            "roofline": {"bound": "hbm", "kernel": "prove-upper (whole: tree build + 36 layer sumchecks)",
+                         "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "alg_bytes": nbytes, "traffic": None},
+            "roofline_by_time": by_time(by)[:8]}
 
 
-def run_commit(sa, steps, warmup, cpu_c):
-    """Config 5 as the reference runs it: 2^24 coefficients = two columns of 2^23 (the code's domain is capped
-    at 2^24 points), rate-1/2 encode to two codewords of 2^24, 2^22 BLAKE3 leaves, Merkle levels, cap of 128."""
-    c, ncols = 23, 2
-    cols = sa.Table.random(5005, ncols << c)
+# ------------------------------------------------------------------ config 5: commitment
+def run_commit(sa, steps, warmup, gold):
+    cm = wl.COMMIT
+    c, ncols = cm["c"], cm["ncols"]
+    cols = sa.Table.random(cm["seed"], ncols << c)
 
     def step():
-        tr = sa.Transcript("config5", 4)
+        tr = sa.Transcript(cm["label"], 4)
         cw, levels = sa.pcs_commit(tr, cols, ncols, c)
         cw.free(), levels.free()
         return tr
 
-    for _ in range(warmup):
-        step()
-    sa.check(sa.load().exh_synchronize())
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        tr = step()
-    sa.check(sa.load().exh_synchronize())
-    dt = (time.perf_counter() - t0) / steps
+    dt, tr = timed(sa, step, steps, warmup)
+    from_proof = tr.proof()
+    cap = from_proof[-128 * 32:]
+    want = gold.get("config5", {}).get("cap_sha256")
+    if want is not None and sha(cap) != want:
+        sys.exit("bench.py: the timed commitment's cap differs from the CPU oracle's")
+    by = launches(sa, step, max(2, min(steps, 10)))
+    cols.free()
     nleaves = 1 << (c - 1)
-    nbytes = ncols * (4 << c) + ncols * (4 << (c + 1)) + ncols * (4 << (c + 1)) + 32 * nleaves + 64 * (nleaves - 1) + 32 * (nleaves - 1)
-    out = {"metric": "BaseFold commit ms (config 5)", "value": 1e3 * dt, "unit": "ms", "n_gpus": 1, "steps": steps,
-           "warmup": warmup, "ms_per_step": 1e3 * dt, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-           "dtype": "u32 (Montgomery KoalaBear) + BLAKE3", "data": "synthetic (SplitMix64-seeded uniform field elements)",
-           "config": {"workload": "pcs-commit: 2 columns of 2^23 coefficients -> 2 codewords of 2^24, 2^22 leaves, "
-                                  "Merkle levels, cap of 128 digests", "cap_sha256": hashlib.sha256(tr.proof()).hexdigest(),
-                      "leaf_hashes_per_s": nleaves / dt, "butterflies_per_s": ncols * 23 * (1 << 23) / dt},
-           "roofline": {"bound": "hbm", "kernel": "encode + leaves + Merkle (whole commit)", "achieved": nbytes / dt / 1e9,
-                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS,
-                        "alg_bytes": nbytes, "traffic": None}}
-    if cpu_c > 0:
-        from oracle import binding as orc
-        hc = [splitmix_field(77 + k, 1 << cpu_c) for k in range(ncols)]
-        t0 = time.perf_counter()
-        orc.commit_columns(hc, cpu_c)
-        cdt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": 1e3 * cdt * (1 << (c - cpu_c)), "unit": "ms", "cores": 1, "kind": "port",
-                               "sample": f"commit of 2 columns of 2^{cpu_c} ({cdt:.1f} s), scaled linearly by 2^{c - cpu_c} "
-                                         "(ignores the log factor of the encoder, so it flatters the CPU)"}
-    return out
+    nbytes = (ncols * (4 << c) + ncols * (4 << (c + 1)) + ncols * (4 << (c + 1)) + 32 * nleaves + 64 * (nleaves - 1)
+              + 32 * (nleaves - 1))
+    return {"workload": "pcs-commit: 2 columns of 2^23 coefficients -> 2 codewords of 2^24, 2^22 leaves, Merkle levels, "
+                        "cap of 128 digests", "ms_per_step": 1e3 * dt, "cap_sha256": sha(cap),
+            "cap_is_the_cpu_oracles": want is not None, "leaf_hashes_per_s": nleaves / dt,
+            "butterflies_per_s": ncols * 23 * (1 << 23) / dt,
+            "roofline": {"bound": "hbm", "kernel": "encode + leaves + Merkle (whole commit)", "achieved": nbytes / dt / 1e9,
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS,
+                         "alg_bytes": nbytes, "traffic": None},
+            "roofline_by_time": by_time(by)[:8]}
 
 
-def run_combine(sa, steps, warmup, cpu_c):
-    """combine-columns at config 5's shape: the two committed columns of 2^23 base values into the table of
-    2^23 EXT8s that BaseFold opens (src/pcs.lisp:434-441)."""
-    c, ncols, d = 23, 2, 8
+def run_combine(sa, steps, warmup, ncols=2):
+    """combine-columns at config 5's shape: the committed columns of 2^23 base values into the table of 2^23
+    EXT8s that BaseFold opens (src/pcs.lisp:434-441)."""
+    c, d = 23, 8
     cols = sa.Table.random(5005, ncols << c)
     cf = splitmix_field(5006, ncols * d).reshape(ncols, d)
-    lib = sa.load()
 
     def step():
         sa.combine_columns(cols, ncols, cf).free()
 
-    for _ in range(warmup):
-        step()
-    sa.check(lib.exh_synchronize())
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    sa.check(lib.exh_synchronize())
-    dt = (time.perf_counter() - t0) / steps
-    sa.check(lib.exh_profile_enable(1))
-    for _ in range(steps):
-        step()
-    entries = [e for e in profile_entries(sa) if e[0] == "combine_columns"]
-    sa.check(lib.exh_profile_enable(0))
-    avg_ms = sum(e[2] for e in entries) / len(entries)
-    nbytes = (1 << c) * (4 * ncols + 4 * d)
-    out = {"metric": "combine-columns entries/s (config 5's columns)", "value": ncols * (1 << c) / dt,
-           "unit": "column entries/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": 1e3 * dt,
-           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32 (Montgomery KoalaBear, F_p^8)",
-           "data": "synthetic (SplitMix64-seeded uniform field elements)",
-           "config": {"workload": "combine-columns: 2 base columns of 2^23 with F_p^8 coefficients -> 2^23 EXT8s"},
-           "roofline": {"bound": "hbm", "kernel": "combine_columns", "achieved": nbytes / (avg_ms * 1e-3) / 1e9,
-                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                        "avg_launch_ms": avg_ms, "alg_bytes_per_launch": nbytes, "traffic": None}}
-    if cpu_c > 0:
-        from oracle import binding as orc
-        hc = np.stack([splitmix_field(77 + k, 1 << cpu_c) for k in range(ncols)])
-        t0 = time.perf_counter()
-        orc.combine_columns(hc, cf)
-        cdt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": ncols * (1 << cpu_c) / cdt, "unit": "column entries/s", "cores": 1, "kind": "port",
-                               "sample": f"2 columns of 2^{cpu_c} ({cdt:.2f} s)"}
+    dt, _ = timed(sa, step, steps, warmup)
+    by = launches(sa, step, max(2, min(steps, 10)))
     cols.free()
-    return out
+    nbytes = (1 << c) * (4 * ncols + 4 * d)
+    total_ms = sum(avg * per for avg, per, _ in by.values())
+    return {"workload": f"combine-columns: {ncols} base columns of 2^23 with F_p^8 coefficients -> 2^23 EXT8s",
+            "ms_per_step": 1e3 * dt, "column_entries_per_s": ncols * (1 << c) / dt,
+            "roofline": {"bound": "hbm", "kernel": "combine_columns (all launches of a call)",
+                         "achieved": nbytes / (total_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": nbytes / (total_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "kernel_ms_per_call": total_ms,
+                         "alg_bytes_per_call": nbytes, "traffic": None}}
 
 
-# HBM bytes per launch of the dominant kernel at the headline workload, from two rocprofv3 --pmc runs of this
-# file (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the plain
-# copy kernel of `--workload copy`, whose traffic is known (the summary of those runs is kept with the profiles)
-MEASURED_TRAFFIC = {
-    ("round_nodes_base", 24): 203495288,  # per launch of the sweep for rounds 0 and 1: the base tables read once
-    ("round_fold2_base", 24): 403802364,  # round 2: 2.024e8 read (base tables) + 2.014e8 written (generation 2)
-}
+# ------------------------------------------------------------------ the CPU baseline
+def cpu_info():
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return model, os.cpu_count()
+
+
+def cpu_baseline(sa, n_one, n_all, best_of=7):
+    """The CPU oracle (a C restatement of the reference's prover: the statement as straight-line code, lines by
+    addition, one reduction per four products, split eq weights; oracle/orc_fast.c) on the headline statement, seeds
+    and transcript at smaller n: one thread (the reference is single-threaded) and all host threads (OpenMP over
+    the HIGH blocks), best of `best_of` warm runs each.  The one-thread sample then goes through the GPU path as a
+    checker of this run: the proof bytes must be the oracle's."""
+    from oracle import binding as orc
+    cfg = wl.SUMCHECK["config2"]
+    d = cfg["d"]
+    st = orc.Statement(cfg["form"], cfg["tables"], cfg["constants"])
+
+    def inputs(n):
+        tables = [orc.splitmix_field(wl.table_seed(cfg, k), 1 << n) for k in range(3)]
+        eq = orc.splitmix_field(wl.eq_seed(cfg), n * d).reshape(n, d)
+        alpha = orc.splitmix_field(wl.constants_seed(cfg), d).reshape(1, d)
+        return tables, eq, alpha
+
+    def best(n, threads):
+        tables, eq, alpha = inputs(n)
+        orc.set_fast(threads)
+        times = []
+        for _ in range(best_of + 1):  # the first run warms the caches and the allocator
+            otr = orc.Transcript("config2", d)
+            t0 = time.perf_counter()
+            orc.prove(otr, n, st, tables, eq=eq, constants=alpha)
+            times.append(time.perf_counter() - t0)
+        orc.set_fast(0)
+        return min(times[1:]), otr.proof(), (tables, eq, alpha)
+
+    threads = orc.host_threads()
+    one_s, proof, (tables, eq, alpha) = best(n_one, 1)
+    dev = [sa.Table.upload(t) for t in tables]
+    tr = sa.Transcript("config2", d)
+    sa.prove(tr, n_one, sa.Statement(cfg["form"], cfg["tables"], cfg["constants"]), dev, eq=eq, constants=alpha)
+    for t in dev:
+        t.free()
+    if tr.proof() != proof:
+        sys.exit(f"bench.py: the GPU proof at n={n_one} differs from the CPU oracle's")
+    all_s, _, _ = best(n_all, threads)
+    model, cores = cpu_info()
+    return {"value": 3 * (1 << n_one) / one_s, "unit": "table entries/s", "cores": 1, "kind": "port",
+            "best_of": best_of, "cpu_model": model, "host_cores": cores,
+            "all_threads": {"value": 3 * (1 << n_all) / all_s, "threads": threads,
+                            "sample": f"n={n_all}, {all_s:.3f} s"},
+            "sample": f"same statement, seeds and transcript at n={n_one} (3*2^{n_one} entries, {one_s:.2f} s on one "
+                      f"thread); the GPU proof of the same sample is byte-identical; the reference's Lisp prover "
+                      f"cannot run here (no SBCL)",
+            "reference_published": {
+                "source": "the reference's README.md:114-149: SBCL 2.2.9, one thread, 4-vCPU Xeon 2.1 GHz VM; none at n=24",
+                "3 base tables n=18 F_p^4, small values vs folding": "0.104 s vs 0.120 s = 7.6e6 / 6.6e6 table entries/s",
+                "3 base tables n=18 F_p^8, split eq": "0.244 s = 3.2e6 table entries/s",
+                "3 extension tables n=18 F_p^8, split eq": "0.424 s = 1.9e6 table entries/s",
+                "extrapolated to config 2 (3*2^24 entries at 7.6e6/s; an extrapolation, and the constant alpha keeps the "
+                "reference off its base-field kernel, so its real time is higher)": "6.6 s"}}
 
 
 def run_copy(steps):
@@ -317,108 +377,99 @@ def run_copy(steps):
     print(json.dumps({"workload": "copy", "read_bytes": a.numel() * 4, "written_bytes": b.numel() * 4, "steps": steps}))
 
 
+def line(metric, value, unit, higher, dtype, data, res, steps, warmup):
+    out = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+           "ms_per_step": res["ms_per_step"], "higher_is_better": higher, "scaling": "weak", "vs_baseline": None,
+           "dtype": dtype, "data": data, "config": {"workload": res["workload"]}}
+    for k, v in res.items():
+        if k in ("roofline", "roofline_by_time", "loop_hbm_fraction"):
+            out[k] = v
+        elif k not in ("workload", "ms_per_step"):
+            out["config"][k] = v
+    return out
+
+
+SEEDED = "synthetic (SplitMix64-seeded uniform field elements)"
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "combine", "copy"],
+    ap.add_argument("--workload", default="config2",
+                    choices=["config1", "config2", "config3", "config4", "config5", "combine", "combine128", "copy"],
                     help="config2 (default) is the headline; the others are the remaining configured workloads; "
                          "copy is the known-size kernel the traffic counters are calibrated on")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--n", type=int, default=24, help="variables (24 is the headline workload)")
-    ap.add_argument("--cpu-n", type=int, default=22, help="variables of the CPU baseline's sample (0: skip)")
+    ap.add_argument("--n", type=int, default=0, help="variables, when not the configured size")
+    ap.add_argument("--cpu-n", type=int, default=20, help="variables of the one-thread CPU baseline's sample (0: skip)")
+    ap.add_argument("--others", type=int, default=1, help="0: leave the other configured workloads out of the headline's line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus above 1 is not supported (nothing here uses a "
                  "second device)")
-
     if args.workload == "copy":
         run_copy(args.steps)
         return
     import sable_amd as sa
     sa.init(0)
-    if args.workload == "config1":
-        print(json.dumps(run_sumcheck_config(sa, "config1", "(* t0 t1)", ["t0", "t1"], [], 16, 4, 1, args.steps,
-                                             args.warmup, 16 if args.cpu_n else 0)))
-        return
-    if args.workload == "config3":
-        print(json.dumps(run_sumcheck_config(sa, "config3", "(* (+ c0 3) (- c1 c0) c2 c3)", ["c0", "c1", "c2", "c3"], [],
-                                             26 if args.n == 24 else args.n, 8, 3, args.steps, args.warmup,
-                                             18 if args.cpu_n else 0)))
+    gold = golden()
+    steps, warmup, n = args.steps, args.warmup, args.n or None
+    if args.workload in ("config1", "config3"):
+        res = run_sumcheck(sa, args.workload, steps, warmup, gold, n)
+        d = res["extension"]
+        print(json.dumps(line(f"sumcheck table entries/s ({args.workload})", res["entries_per_s"], "table entries/s", True,
+                              f"u32 (Montgomery KoalaBear, F_p^{d} tower)", SEEDED, res, steps, warmup)))
         return
     if args.workload == "config4":
-        print(json.dumps(run_gkr(sa, args.steps, args.warmup, 18 if args.cpu_n else 0)))
+        res = run_gkr(sa, steps, warmup, gold)
+        print(json.dumps(line("LogUp-GKR prove-upper lookups/s (config 4)", res["lookups_per_s"], "lookups/s", True,
+                              "u32 (Montgomery KoalaBear, F_p^4 tower)",
+                              "synthetic (seeded uniform int8 lookups, exact multiplicities)", res, steps, warmup)))
         return
     if args.workload == "config5":
-        print(json.dumps(run_commit(sa, args.steps, args.warmup, 18 if args.cpu_n else 0)))
+        res = run_commit(sa, steps, warmup, gold)
+        print(json.dumps(line("BaseFold commit ms (config 5)", res["ms_per_step"], "ms", False,
+                              "u32 (Montgomery KoalaBear) + BLAKE3", SEEDED, res, steps, warmup)))
         return
-    if args.workload == "combine":
-        print(json.dumps(run_combine(sa, args.steps, args.warmup, 20 if args.cpu_n else 0)))
+    if args.workload in ("combine", "combine128"):
+        res = run_combine(sa, steps, warmup, 128 if args.workload == "combine128" else 2)
+        print(json.dumps(line("combine-columns entries/s (config 5's columns)", res["column_entries_per_s"],
+                              "column entries/s", True, "u32 (Montgomery KoalaBear, F_p^8)", SEEDED, res, steps, warmup)))
         return
-    n, d, seed = args.n, 4, 2
-    st = sa.Statement(FORM, TABLES, CONSTS)
-    tables = [sa.Table.random(seed * 1000 + k, 1 << n) for k in range(3)]
-    eq = splitmix_field(seed + 900, n * d).reshape(n, d)
-    alpha = splitmix_field(seed + 901, d).reshape(1, d)
 
-    def step():
-        tr = sa.Transcript("config2", d)
-        sa.prove(tr, n, st, tables, eq=eq, constants=alpha)
-        return tr
-
-    for _ in range(args.warmup):
-        step()
-    # the library runs on its own HIP stream (not torch's): exh_synchronize is the device-wide barrier
-    sa.check(sa.load().exh_synchronize())
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        tr = step()  # every prove ends with its finals on the host: the stream is drained
-    sa.check(sa.load().exh_synchronize())
-    elapsed = time.perf_counter() - t0
-    ms_per_step = 1e3 * elapsed / args.steps
-    entries = 3 * (1 << n)
-    proof = tr.proof()
-
-    # the dominant kernel, timed live with HIP events on the library's stream over `steps` more proves
-    sa.check(sa.load().exh_profile_enable(1))
-    for _ in range(args.steps):
-        step()
-    by_kernel = {}
-    for name, rnd, ms, nbytes in profile_entries(sa):
-        k = by_kernel.setdefault((name, rnd), [0.0, 0, nbytes])
-        k[0] += ms
-        k[1] += 1
-    sa.check(sa.load().exh_profile_enable(0))
-    # The roofline figure is for the streaming launch (the ones that read the tables from HBM: round_*) with the
-    # largest total time per prove; the launch with the largest time of all may be one of the LDS-resident ones
-    # (slices, tail), which are latency-bound by construction and move a few MB: it is named beside it.
-    streaming = {k: v for k, v in by_kernel.items() if k[0].startswith("round_")}
-    (kname, kround), (ktotal, kcalls, kbytes) = max(streaming.items(), key=lambda kv: kv[1][0])
-    (tname, tround), (ttotal, tcalls, _) = max(by_kernel.items(), key=lambda kv: kv[1][0])
-    avg_ms = ktotal / kcalls
-    achieved = kbytes / (avg_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC.get((kname, n))
-    loop_alg_bytes = 3 * (1 << n) * (8 + 8 * d)
-
-    result = {
-        "metric": "sumcheck table entries/s at n=24 deg-3", "value": entries / (elapsed / args.steps),
-        "unit": "table entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u32 (Montgomery KoalaBear, F_p^4 tower; exact integers in f64 for the first sweep's products)",
-        "data": "synthetic (SplitMix64-seeded uniform field elements)",
-        "config": {"workload": f"sumcheck prove of {FORM}, eq mode, n={n}, three base tables of 2^{n}, F_p^4, "
-                               "BLAKE3 transcript", "tables": 3, "n": n, "degree": 3, "extension": 4,
-                   "proof_sha256": hashlib.sha256(proof).hexdigest(), "proof_bytes": len(proof)},
-        "loop_hbm_fraction": loop_alg_bytes / (elapsed / args.steps) / (HBM_PEAK_GBS * 1e9),
-        "roofline": {"bound": "hbm", "kernel": f"{kname} (round {kround})", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "avg_launch_ms": avg_ms, "launches_per_step": kcalls // args.steps,
-                     "alg_bytes_per_launch": kbytes, "traffic": traffic,
-                     "longest_launch": {"kernel": f"{tname} (round {tround})", "avg_launch_ms": ttotal / tcalls,
-                                        "note": "LDS-resident rounds are latency-bound" if not tname.startswith("round_") else ""}},
-    }
-    result["cpu_baseline"] = cpu_baseline(sa, args.cpu_n, d, seed) if args.cpu_n > 0 else None
-    print(json.dumps(result))
+    # ---- the headline: config 2
+    res = run_sumcheck(sa, "config2", steps, warmup, gold, n)
+    current = MEASURED["kernel_sources_sha256"] == kernel_sources_sha256()
+    kname = res["roofline"]["kernel"].split(" ")[0]
+    res["roofline"]["traffic"] = MEASURED["traffic"].get((kname, res["n"])) if current else None
+    out = line("sumcheck table entries/s at n=24 deg-3", res["entries_per_s"], "table entries/s", True,
+               "u32 (Montgomery KoalaBear, F_p^4 tower; exact integers in f64 for the first sweep's products)", SEEDED,
+               res, steps, warmup)
+    muls = MEASURED["int32_mul_per_prove"] if current and res["n"] == 24 else None
+    out["int32_mul"] = {"bound": "int32 multiply issue", "multiplies_per_step": muls, "peak": INT32_MUL_PEAK_PER_S,
+                        "unit": "32-bit multiplies/s (per lane)",
+                        "achieved": muls / (res["ms_per_step"] * 1e-3) if muls else None,
+                        "frac": muls / (res["ms_per_step"] * 1e-3) / INT32_MUL_PEAK_PER_S if muls else None,
+                        "note": "counts are from the kernels' instruction streams and go with one version of the "
+                                "sources (null when they have changed since)"}
+    out["cpu_baseline"] = cpu_baseline(sa, args.cpu_n, min(args.cpu_n + 2, 24)) if args.cpu_n > 0 else None
+    if args.others and n is None:
+        k = max(3, steps // 4)
+        others = {}
+        for name in ("config1", "config3"):
+            r = run_sumcheck(sa, name, k, 2, gold)
+            others[name] = {key: r[key] for key in ("workload", "ms_per_step", "entries_per_s", "proof_sha256",
+                                                    "proof_is_the_cpu_oracles", "loop_hbm_fraction")}
+            others[name]["roofline"] = r["roofline"]
+        r = run_gkr(sa, k, 2, gold)
+        others["config4"] = {key: r[key] for key in ("workload", "ms_per_step", "lookups_per_s", "proof_sha256",
+                                                     "proof_is_the_cpu_oracles", "timed_launches_per_step", "roofline")}
+        r = run_commit(sa, k, 2, gold)
+        others["config5"] = {key: r[key] for key in ("workload", "ms_per_step", "cap_sha256", "cap_is_the_cpu_oracles",
+                                                     "roofline")}
+        out["other_configs"] = others
+    print(json.dumps(out))
 
 
 if __name__ == "__main__":
