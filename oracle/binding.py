@@ -783,3 +783,80 @@ def basefold_verify(tr, nv, rr, v, grind_bits=4, queries=6):
     _check(lib().orc_basefold_verify(tr.h, nv, _p(rr), _p(v), grind_bits, queries, qs.ctypes.data_as(u64p)),
            "basefold")
     return [int(q) for q in qs]
+
+
+# ------------------------------------------------------------------ the opening over several classes (orc_open.c)
+class OpenKey(C.Structure):
+    _fields_ = [("c", C.c_int32), ("ncols", C.c_int32), ("codewords", u32p), ("levels", u8p), ("cap", u8p),
+                ("coef", u32p), ("h", u32p)]
+
+
+def merkle_levels_injected(leaves, injections):
+    """merkle-levels with injections (src/pcs.lisp:64-77): injections = {level: digests}; a list of levels."""
+    lv = np.ascontiguousarray(leaves, np.uint8).reshape(-1, 32)
+    n = len(lv)
+    levels = sorted(injections)
+    arrs = [np.ascontiguousarray(injections[l], np.uint8).reshape(-1, 32) for l in levels]
+    ptrs = (u8p * max(len(arrs), 1))(*[a.ctypes.data_as(u8p) for a in arrs])
+    lvl = np.array(levels if levels else [0], np.int32)
+    out = np.zeros((2 * n - 1, 32), np.uint8)
+    lib().orc_merkle_levels_injected(lv.ctypes.data_as(u8p), C.c_uint64(n), len(arrs), lvl.ctypes.data_as(i32p), ptrs,
+                                     out.ctypes.data_as(u8p))
+    res, pos = [], 0
+    while n >= 1:
+        res.append(out[pos:pos + n].copy())
+        pos += n
+        n //= 2
+    return res
+
+
+def check_path_injected(h, path, i, cap, injected_at):
+    """check-path with injected-at (src/pcs.lisp:86-95): injected_at = {level: digest}."""
+    h = np.frombuffer(bytes(h), np.uint8).copy()
+    p = np.ascontiguousarray(path, np.uint8).reshape(-1, 32)
+    capa = np.ascontiguousarray(cap, np.uint8).reshape(-1, 32)
+    levels = sorted(injected_at)
+    lvl = np.array(levels if levels else [0], np.int32)
+    dig = np.array([np.frombuffer(bytes(injected_at[l]), np.uint8) for l in levels], np.uint8).reshape(-1, 32) \
+        if levels else np.zeros((1, 32), np.uint8)
+    return bool(lib().orc_check_path_injected(h.ctypes.data_as(u8p), p.ctypes.data_as(u8p), len(p), C.c_uint64(i),
+                                              capa.ctypes.data_as(u8p), len(levels), lvl.ctypes.data_as(i32p),
+                                              dig.ctypes.data_as(u8p)))
+
+
+def _open_keys(keys, prover):
+    """keys: dicts with c, ncols, coef (ncols, 8) and, for the prover, codewords (ncols, 2^(c+1)), levels (list of
+    (n, 32) arrays), h (2^c, 8); for the verifier, cap (rows, 32)."""
+    arr = (OpenKey * len(keys))()
+    keep = []
+    for k, key in enumerate(keys):
+        coef = _u32(key["coef"]).reshape(-1, 8)
+        keep.append(coef)
+        arr[k].c, arr[k].ncols, arr[k].coef = key["c"], key["ncols"], _p(coef)
+        if prover:
+            cw = np.ascontiguousarray(key["codewords"], np.uint32)
+            lv = np.ascontiguousarray(np.concatenate(key["levels"]), np.uint8)
+            h = _u32(key["h"]).reshape(-1, 8)
+            keep += [cw, lv, h]
+            arr[k].codewords, arr[k].levels, arr[k].h = _p(cw), lv.ctypes.data_as(u8p), _p(h)
+        else:
+            cap = np.ascontiguousarray(key["cap"], np.uint8)
+            keep.append(cap)
+            arr[k].cap = cap.ctypes.data_as(u8p)
+    return arr, keep
+
+
+def pcs_open(tr, nv, keys, rr, v, grind_bits=4, queries=6):
+    arr, keep = _open_keys(keys, True)
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    qs = np.zeros(queries, np.uint64)
+    _check(lib().orc_pcs_open(tr.h, nv, len(keys), arr, _p(rr), _p(v), grind_bits, queries,
+                              qs.ctypes.data_as(u64p)), "pcs-open")
+    return [int(q) for q in qs]
+
+
+def pcs_verify_opening(tr, nv, keys, rr, v, grind_bits=4, queries=6):
+    arr, keep = _open_keys(keys, False)
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    _check(lib().orc_pcs_verify_opening(tr.h, nv, len(keys), arr, _p(rr), _p(v), grind_bits, queries), "pcs")
+    return True

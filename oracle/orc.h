@@ -31,6 +31,10 @@
  *                                             the round identity g(0) + g(1) of the folded tables = g(x)
  *   open-queries (leaves, paths)              numpy indexing of the codewords by the definition; every opened leaf,
  *                                             hashed and walked up its path, lands on the committed cap
+ *   opening over several classes, verify-      PARITY UNPINNED BY BYTES; prover -> verifier acceptance, rejection of every
+ *   queries, mixed-height Merkle trees        flipped opened symbol / path / cap / final-table word, the single-class case
+ *                                             being orc_basefold_prove byte for byte, injected levels against a
+ *                                             definition-level Python tree
  *   combine-columns                           the definition evaluated with big integers coordinate by
  *                                             coordinate (ext-scale is coordinate-wise, :ext vectors), unit
  *                                             coefficients, linearity; its output opening under BaseFold to
@@ -257,6 +261,30 @@ int orc_basefold_prove(orc_tr *tr, int nv, const uint32_t *rr, const uint32_t *v
                        uint32_t *out_chal /* fl*8 */, uint32_t *out_final /* 2^(nv-fl)*8 */);
 int orc_basefold_verify(orc_tr *tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits,
                         int queries, uint64_t *out_qs);
+
+/* ---- the final opening over several size classes (orc_open.c; src/pcs.lisp:64-95, 581-657, 721-843) */
+/* MERKLE-LEVELS with injections: inj[k] (nleaves >> inj_level[k] digests) is hashed into level inj_level[k] */
+void orc_merkle_levels_injected(const uint8_t *leaves, uint64_t nleaves, int ninj, const int32_t *inj_level,
+                                const uint8_t *const *inj, uint8_t *out);
+/* CHECK-PATH with INJECTED-AT: inj_digests[k] (32 bytes) is hashed in after level inj_level[k] */
+int orc_check_path_injected(const uint8_t h[32], const uint8_t *path, int depth, uint64_t i, const uint8_t *cap,
+                            int ninj, const int32_t *inj_level, const uint8_t *inj_digests);
+/* one key of the opening: a size class with its committed columns (a unit of its own with its own tree) */
+typedef struct {
+  int32_t c, ncols;
+  const uint32_t *codewords; /* prover: ncols * 2^(c+1) symbols */
+  const uint8_t *levels;     /* prover: the tree's levels, leaves first */
+  const uint8_t *cap;        /* verifier: the committed cap */
+  const uint32_t *coef;      /* ncols EXT8s: the columns' coefficients in the class's combined column */
+  const uint32_t *h;         /* prover: the combined column, 2^c EXT8s */
+} orc_open_key;
+/* BASEFOLD (classes ascending, the last one nv; class c joins at level nv - c) and OPEN-QUERIES: the claim is
+   sum_c H_c(the last c coordinates of rr) = v */
+int orc_pcs_open(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr, const uint32_t *v,
+                 int grind_bits, int queries, uint64_t *out_qs);
+/* BASEFOLD's verifier side and VERIFY-QUERIES; ORC_E_REJECT when a check fails */
+int orc_pcs_verify_opening(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr,
+                           const uint32_t *v, int grind_bits, int queries);
 
 #ifdef __cplusplus
 }
