@@ -86,6 +86,34 @@ int exh_basefold_prove(exh_transcript tr, int nv, const uint32_t *rr, const uint
 int exh_basefold_verify(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits,
                         int queries, uint64_t *out_qs);
 
+/* ---- the final opening over several size classes (src/pcs.lisp:434-441, 581-657, 721-843): one key per class,
+   each a unit of its own with its own tree; the classes ascend and the last one is nv.  Merge sets, segments and
+   the cross-unit sumcheck around it stay with the caller. */
+typedef struct {
+  int32_t c, ncols;
+  exh_table columns;   /* prover: the class's ncols base columns of 2^c values (as exh_pcs_commit took them) */
+  exh_table codewords; /* prover: their codewords (exh_pcs_commit / exh_rs_encode) */
+  exh_table levels;    /* prover: the tree's levels (exh_pcs_commit / exh_merkle_commit) */
+  const uint32_t *coefficients; /* ncols EXT8s: the columns' coefficients in the class's combined column (UC-COEF) */
+  const uint8_t *cap;  /* verifier: the committed cap, 32 * CAP-ROWS(2^(c-1)) bytes */
+} exh_open_key;
+/* COMBINE-COLUMNS per key, BASEFOLD with class c joining at level nv - c (:590-600, :635-639), OPEN-QUERIES per key
+   (:721-734).  The claim: sum_c H_c(the last c coordinates of rr) = v.  out_qs: the query positions */
+int exh_pcs_open(exh_transcript tr, int nv, int n_keys, const exh_open_key *keys, const uint32_t *rr, const uint32_t *v,
+                 int grind_bits, int queries, uint64_t *out_qs);
+/* BASEFOLD's verifier side and VERIFY-QUERIES (:752-843): every opened leaf against its tree's cap, the folding of
+   the combined codeword through the oracles down to the final table's codeword.  EXH_E_REJECT when a check fails */
+int exh_pcs_verify_opening(exh_transcript tr, int nv, int n_keys, const exh_open_key *keys, const uint32_t *rr,
+                           const uint32_t *v, int grind_bits, int queries);
+/* MERKLE-LEVELS with injections (:64-77): the levels (a new table, leaves first) of the tree over `leaves` (8-word
+   digests), the digests of injected[k] hashed into the nodes of level inject_level[k] (mixed-height trees) */
+int exh_merkle_levels_injected(exh_table leaves, int n_injected, const int32_t *inject_level, const exh_table *injected,
+                               exh_table *levels);
+/* CHECK-PATH with INJECTED-AT (:86-95): 1 when leaf digest h hashes up `path` (depth siblings) from leaf i to
+   cap[i >> depth], the digest injected_digests[k] hashed in after level inject_level[k] */
+int exh_check_path(const uint8_t h[32], const uint8_t *path, int depth, uint64_t i, const uint8_t *cap, int n_injected,
+                   const int32_t *inject_level, const uint8_t *injected_digests);
+
 #ifdef __cplusplus
 }
 #endif

@@ -474,3 +474,71 @@ def basefold_verify(tr, nv, rr, v, grind_bits=4, queries=6):
     qs = np.zeros(queries, np.uint64)
     check(load().exh_basefold_verify(tr.h, nv, _p(rr), _p(v), grind_bits, queries, qs.ctypes.data_as(u64p)))
     return [int(q) for q in qs]
+
+
+# ------------------------------------------------------------------ the opening over several size classes
+class _OpenKey(C.Structure):
+    _fields_ = [("c", C.c_int32), ("ncols", C.c_int32), ("columns", C.c_uint64), ("codewords", C.c_uint64),
+                ("levels", C.c_uint64), ("coefficients", u32p), ("cap", u8p)]
+
+
+def _open_keys(keys, prover):
+    """keys: dicts with c, ncols, coef (ncols, 8) and, for the prover, the Tables columns, codewords, levels; for the
+    verifier, cap (rows, 32) bytes."""
+    arr, keep = (_OpenKey * len(keys))(), []
+    for k, key in enumerate(keys):
+        coef = np.ascontiguousarray(_u32(key["coef"]).reshape(-1, 8))
+        keep.append(coef)
+        arr[k].c, arr[k].ncols = key["c"], key["ncols"]
+        arr[k].coefficients = coef.ctypes.data_as(u32p)
+        if prover:
+            arr[k].columns, arr[k].codewords, arr[k].levels = (key["columns"].handle, key["codewords"].handle,
+                                                              key["levels"].handle)
+        else:
+            cap = np.ascontiguousarray(key["cap"], np.uint8)
+            keep.append(cap)
+            arr[k].cap = cap.ctypes.data_as(u8p)
+    return arr, keep
+
+
+def pcs_open(tr, nv, keys, rr, v, grind_bits=4, queries=6):
+    """The final opening (combine-columns, basefold with class joins, open-queries): the query positions."""
+    arr, keep = _open_keys(keys, True)
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    qs = np.zeros(queries, np.uint64)
+    check(load().exh_pcs_open(tr.h, nv, len(keys), arr, _p(rr), _p(v), grind_bits, queries, qs.ctypes.data_as(u64p)))
+    return [int(q) for q in qs]
+
+
+def pcs_verify_opening(tr, nv, keys, rr, v, grind_bits=4, queries=6):
+    """basefold's verifier side and verify-queries; raises VerificationFailure when a check fails."""
+    arr, keep = _open_keys(keys, False)
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    check(load().exh_pcs_verify_opening(tr.h, nv, len(keys), arr, _p(rr), _p(v), grind_bits, queries))
+    return True
+
+
+def merkle_levels_injected(leaves, injections):
+    """merkle-levels with injections: leaves a Table of digests, injections {level: Table of digests} -> Table."""
+    levels = sorted(injections)
+    at = (C.c_int32 * max(len(levels), 1))(*levels)
+    tabs = (C.c_uint64 * max(len(levels), 1))(*[injections[l].handle for l in levels])
+    h = C.c_uint64()
+    check(load().exh_merkle_levels_injected(C.c_uint64(leaves.handle), len(levels), at, tabs, C.byref(h)))
+    return Table(h.value, 2 * leaves.n_u32 - 8, 8)
+
+
+def check_path(h, path, i, cap, injected_at=None):
+    """check-path (with injected-at {level: digest}) on the host."""
+    h = np.frombuffer(bytes(h), np.uint8).copy()
+    p = np.ascontiguousarray(path, np.uint8).reshape(-1, 32)
+    capa = np.ascontiguousarray(cap, np.uint8).reshape(-1, 32)
+    levels = sorted(injected_at or {})
+    at = (C.c_int32 * max(len(levels), 1))(*levels)
+    dig = np.array([np.frombuffer(bytes(injected_at[l]), np.uint8) for l in levels], np.uint8).reshape(-1, 32) \
+        if levels else np.zeros((1, 32), np.uint8)
+    out = load().exh_check_path(h.ctypes.data_as(u8p), p.ctypes.data_as(u8p), len(p), C.c_uint64(i),
+                                capa.ctypes.data_as(u8p), len(levels), at, dig.ctypes.data_as(u8p))
+    if out < 0:
+        check(out)
+    return out == 1

@@ -654,6 +654,84 @@ int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out) {
   return dot_pairs_device(te->ptr, tv->ptr, te->n_u32 / 8, out);
 }
 
+static int open_keys(const exh_open_key *keys, int n_keys, bool prover, std::vector<OpenClass> *out) {
+  if (!keys || n_keys < 1 || n_keys > 32) {
+    set_error("invalid-parameter: opening keys");
+    return E_PARAM;
+  }
+  for (int k = 0; k < n_keys; k++) {
+    OpenClass oc;
+    oc.c = keys[k].c, oc.ncols = keys[k].ncols, oc.coef = keys[k].coefficients, oc.cap = keys[k].cap;
+    if (oc.c < 1 || oc.c > 30 || oc.ncols < 1 || !oc.coef || (!prover && !oc.cap)) {
+      set_error("invalid-parameter: opening key");
+      return E_PARAM;
+    }
+    if (prover) {
+      DeviceTable *cols = table_of(keys[k].columns), *cw = table_of(keys[k].codewords), *lv = table_of(keys[k].levels);
+      const uint64_t nleaves = (uint64_t)1 << (oc.c - 1);
+      if (!cols || !cw || !lv) return E_PARAM;
+      if (cols->n_u32 != ((uint64_t)oc.ncols << oc.c) || cw->n_u32 != ((uint64_t)oc.ncols << (oc.c + 1)) ||
+          lv->n_u32 != (2 * nleaves - 1) * 8) {
+        set_error("invalid-parameter: opening key: columns, codewords or levels of another shape");
+        return E_PARAM;
+      }
+      oc.d_columns = cols->ptr, oc.d_codewords = cw->ptr, oc.d_levels = lv->ptr;
+    }
+    out->push_back(oc);
+  }
+  return OK;
+}
+
+int exh_pcs_open(exh_transcript h, int nv, int n_keys, const exh_open_key *keys, const uint32_t *rr, const uint32_t *v,
+                 int grind_bits, int queries, uint64_t *out_qs) {
+  Transcript *tr = tr_of(h);
+  if (!tr || !rr || !v) return E_PARAM;
+  std::vector<OpenClass> oc;
+  int status = open_keys(keys, n_keys, true, &oc);
+  if (status) return status;
+  return pcs_open(*tr, nv, n_keys, oc.data(), rr, v, grind_bits, queries, out_qs);
+}
+
+int exh_pcs_verify_opening(exh_transcript h, int nv, int n_keys, const exh_open_key *keys, const uint32_t *rr,
+                           const uint32_t *v, int grind_bits, int queries) {
+  Transcript *tr = tr_of(h);
+  if (!tr || !rr || !v) return E_PARAM;
+  std::vector<OpenClass> oc;
+  int status = open_keys(keys, n_keys, false, &oc);
+  if (status) return status;
+  return pcs_verify_opening(*tr, nv, n_keys, oc.data(), rr, v, grind_bits, queries);
+}
+
+int exh_merkle_levels_injected(exh_table leaves, int n_injected, const int32_t *inject_level, const exh_table *injected,
+                               exh_table *levels) {
+  DeviceTable *lv = table_of(leaves);
+  if (!lv || !levels || n_injected < 0 || n_injected > 16 || lv->n_u32 % 8) return E_PARAM;
+  const uint64_t nleaves = lv->n_u32 / 8;
+  std::vector<const uint32_t *> inj;
+  std::vector<int> at;
+  for (int k = 0; k < n_injected; k++) {
+    DeviceTable *t = table_of(injected[k]);
+    if (!t) return E_PARAM;
+    if (inject_level[k] < 1 || inject_level[k] > 40 || t->n_u32 != (nleaves >> inject_level[k]) * 8) {
+      set_error("invalid-parameter: an injected class has as many digests as its level has nodes");
+      return E_PARAM;
+    }
+    inj.push_back(t->ptr), at.push_back(inject_level[k]);
+  }
+  int status = exh_table_alloc((2 * nleaves - 1) * 8, 8, levels);
+  if (status) return status;
+  status = merkle_levels_injected_device(lv->ptr, nleaves, n_injected, at.data(), inj.data(), table_of(*levels)->ptr);
+  if (status) exh_table_free(*levels);
+  return status;
+}
+
+int exh_check_path(const uint8_t h[32], const uint8_t *path, int depth, uint64_t i, const uint8_t *cap, int n_injected,
+                   const int32_t *inject_level, const uint8_t *injected_digests) {
+  if (!h || !cap || depth < 0 || (depth && !path)) return E_PARAM;
+  std::vector<int> at(inject_level, inject_level + (n_injected > 0 ? n_injected : 0));
+  return check_path_host(h, path, depth, i, cap, n_injected, at.data(), injected_digests) ? 1 : 0;
+}
+
 int exh_dot_pairs_static(exh_table e, exh_table v, uint32_t *out) {
   DeviceTable *te = table_of(e), *tv = table_of(v);
   if (!te || !tv) return E_PARAM;

@@ -1,6 +1,8 @@
 // commit.hip -- see commit.hpp.
 #include "commit.hpp"
 
+#include <array>
+
 #include <string.h>
 
 #include <algorithm>
@@ -535,6 +537,65 @@ int merkle_commit_columns(const uint32_t *d_codewords, int ncols, int c, uint32_
   return merkle_tree_device(d_levels, nleaves, 1, d_codewords, ncols, cw_len, cap, cap_rows);
 }
 
+// ---- trees of mixed height (src/pcs.lisp:64-77): a shorter class's leaf digests are hashed into the level of the
+// taller class's tree that has as many nodes, node = H(H(left, right), injected).  One launch per level (these
+// trees sit beside the large single-class ones, whose levels go nine to a launch).
+__global__ __launch_bounds__(BLOCK) void node_level_kernel(const uint32_t *below, uint32_t *level, uint64_t count,
+                                                           const uint32_t *inj0, const uint32_t *inj1) {
+  const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (i >= count) return;
+  uint32_t left[8], right[8], h[8], t[8];
+  load_digest(below + 16 * i, left);
+  load_digest(below + 16 * i + 8, right);
+  b3_node(left, right, h);
+  if (inj0) {
+    load_digest(inj0 + 8 * i, right);
+    b3_node(h, right, t);
+#pragma unroll
+    for (int k = 0; k < 8; k++) h[k] = t[k];
+  }
+  if (inj1) {
+    load_digest(inj1 + 8 * i, right);
+    b3_node(h, right, t);
+#pragma unroll
+    for (int k = 0; k < 8; k++) h[k] = t[k];
+  }
+  store_digest(level + 8 * i, h);
+}
+
+int merkle_levels_injected_device(const uint32_t *d_leaves, uint64_t nleaves, int ninj, const int *inj_level,
+                                  const uint32_t *const *d_inj, uint32_t *d_levels) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  if (nleaves == 0 || (nleaves & (nleaves - 1))) {
+    set_error("invalid-parameter: a tree has a power of two of leaves");
+    return E_PARAM;
+  }
+  EXH_HIP(hipMemcpyAsync(d_levels, d_leaves, nleaves * 32, hipMemcpyDeviceToDevice, c.stream));
+  uint32_t *below = d_levels;
+  uint64_t n = nleaves;
+  for (int l = 1; n > 1; l++) {
+    uint32_t *level = below + 8 * n;
+    n /= 2;
+    const uint32_t *inj[2] = {nullptr, nullptr};
+    int found = 0;
+    for (int k = 0; k < ninj; k++)
+      if (inj_level[k] == l) {
+        if (found == 2) {
+          set_error("invalid-parameter: at most two classes are injected into one level");
+          return E_PARAM;
+        }
+        inj[found++] = d_inj[k];
+      }
+    hipLaunchKernelGGL(node_level_kernel, dim3((uint32_t)((n + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, c.stream, below,
+                       level, n, inj[0], inj[1]);
+    below = level;
+  }
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
 // ------------------------------------------------------------------ BaseFold
 // DOT-PAIRS (src/pcs.lisp:473-483) for the three parities at once: sums over pairs of
 // pick(tt) pick(et), pick = even entry, odd entry, 2 odd - even.  Partials per workgroup.
@@ -877,11 +938,24 @@ int open_queries_device(const uint32_t *d_codewords, int ncols, int c, const uin
   return OK;
 }
 
-int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
-                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final) {
+// BASEFOLD (src/pcs.lisp:581-657) over ncls size classes, ascending, the last one nv: class c's table d_h[k]
+// (2^c EXT8s) joins the message table and the codeword at level nv - c (:590-600, :635-639)
+int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, const uint32_t *const *d_hs,
+                           const uint32_t *rr, const uint32_t *v, int grind_bits, int queries, uint64_t *out_qs,
+                           uint32_t *out_chal, uint32_t *out_final) {
   Context &c = ctx();
   int status = c.require();
   if (status) return status;
+  if (ncls < 1 || cls[ncls - 1] != nv || queries < 1) {
+    set_error("invalid-parameter: basefold takes its classes in ascending order, the largest being nv");
+    return E_PARAM;
+  }
+  for (int k = 0; k < ncls; k++)
+    if (cls[k] < 1 || (k && cls[k] <= cls[k - 1])) {
+      set_error("invalid-parameter: basefold classes must ascend");
+      return E_PARAM;
+    }
+  const uint32_t *d_h = d_hs[ncls - 1];
   const int fl = nv - 5 > 0 ? nv - 5 : 0;
   const uint64_t len = (uint64_t)1 << nv;
   Owned mem;
@@ -914,6 +988,24 @@ int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v
   if ((status = get_domain(nv + 1, &dom))) return status;
 
   hf::E prf = hf::lift(1, 8), claim = hf::from(v, 8);
+  // y_c = H_c at the point's last c coordinates, for the classes still to join; ysum their sum (:593-595)
+  const uint32_t one8[8] = {1, 0, 0, 0, 0, 0, 0, 0};
+  std::vector<hf::E> yc(ncls, hf::zero(8));
+  hf::E ysum = hf::zero(8);
+  for (int k = 0; k + 1 < ncls; k++) {
+    const uint64_t clen = (uint64_t)1 << cls[k], n_pairs = clen / 2;
+    uint32_t *eqc = et2;  // the eq table of the point's tail (at most half of et2's room)
+    hipLaunchKernelGGL(eq8_kernel, dim3((uint32_t)((clen + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, c.stream,
+                       factors + (size_t)(nv - cls[k]) * 16, cls[k], eqc, clen);
+    uint32_t grid = (uint32_t)std::min<uint64_t>((n_pairs + BLOCK - 1) / BLOCK, max_grid);
+    hipLaunchKernelGGL(dot_pairs_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, d_hs[k], eqc, n_pairs, partials);
+    hipLaunchKernelGGL(sum_columns_kernel, dim3(24), dim3(BLOCK), 0, c.stream, partials, grid, 24u, sums);
+    uint32_t dots[24];
+    EXH_HIP(hipMemcpyAsync(dots, sums, 96, hipMemcpyDeviceToHost, c.stream));
+    EXH_HIP(hipStreamSynchronize(c.stream));
+    yc[k] = hf::add(hf::from(dots, 8), hf::from(dots + 8, 8));  // even entries' products + odd entries' products
+    ysum = hf::add(ysum, yc[k]);
+  }
   std::vector<OracleTree> oracles;
   for (int i = 0; i < fl; i++) {
     uint64_t cur = len >> i, n_pairs = cur / 2;
@@ -923,7 +1015,14 @@ int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v
     uint32_t ev[24];
     EXH_HIP(hipMemcpyAsync(ev, sums, 96, hipMemcpyDeviceToHost, c.stream));
     EXH_HIP(hipStreamSynchronize(c.stream));
-    // every class has joined at level 0, so the a = prf * ysum term of the reference is zero
+    if (ncls > 1) {  // the classes still to join: a = prf * ysum times (1 - r_i, r_i, 2 r_i - (1 - r_i)), :607-612
+      const hf::E ri = hf::from(rr + 8 * (size_t)i, 8), a = hf::mul(prf, ysum), one_r = hf::sub(hf::lift(1, 8), ri);
+      const hf::E eqx[3] = {one_r, ri, hf::sub(hf::scale(ri, 2), one_r)};
+      for (int parity = 0; parity < 3; parity++) {
+        hf::E t = hf::add(hf::from(ev + 8 * parity, 8), hf::mul(a, eqx[parity]));
+        memcpy(ev + 8 * parity, t.data(), 32);
+      }
+    }
     uint64_t dims[2] = {3, 8};
     if ((status = tr.send(ev, 2, dims, nullptr))) return status;
     if (hf::add(hf::from(ev, 8), hf::from(ev + 8, 8)) != claim) {
@@ -962,6 +1061,17 @@ int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v
       if ((status = tr.send_bytes(cap.data(), (int64_t)(32 * rows), nullptr))) return status;
       oracles.push_back(o);
     }
+    for (int k = 0; k + 1 < ncls; k++)  // the classes that join at this level, :635-639
+      if (nv - cls[k] == l) {
+        const uint64_t clen = (uint64_t)1 << cls[k];
+        const uint32_t gl = (uint32_t)((clen + BLOCK - 1) / BLOCK);
+        scale_add_launch<8>(tt, d_hs[k], tt, clen, one8);
+        hipLaunchKernelGGL(split_coords_kernel, dim3(gl), dim3(BLOCK), 0, c.stream, d_hs[k], cols, clen);
+        if ((status = rs_encode_columns(cols, 8, cls[k], cwcols))) return status;
+        hipLaunchKernelGGL(join_coords_kernel, dim3(2 * gl), dim3(BLOCK), 0, c.stream, cwcols, cw2, 2 * clen);
+        scale_add_launch<8>(cw, cw2, cw, 2 * clen, one8);
+        ysum = hf::sub(ysum, yc[k]);
+      }
   }
   // the final table in the clear, the final claim, grinding, the query positions
   uint64_t mlen = len >> fl;
@@ -1003,6 +1113,280 @@ int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v
     uint64_t d3[3] = {(uint64_t)queries, 8, 4};
     if ((status = tr.send(leaves.data(), 3, d3, nullptr, false))) return status;
     if ((status = tr.send_bytes((const uint8_t *)path.data(), (int64_t)path.size() * 4, nullptr, false))) return status;
+  }
+  return OK;
+}
+
+int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
+                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final) {
+  return basefold_prove_classes(tr, nv, 1, &nv, &d_h, rr, v, grind_bits, queries, out_qs, out_chal, out_final);
+}
+
+// The final opening over several size classes, one key per class, each a unit of its own with its own tree:
+// the class's combined column H_c = COMBINE-COLUMNS of its columns with the caller's coefficients
+// (src/pcs.lisp:434-441, 709-716), BASEFOLD over the classes, then OPEN-QUERIES (:721-734): per key the queried
+// leaves (Q, ncols, 4), recorded, and its tree's paths up to the cap level, recorded.
+int pcs_open(Transcript &tr, int nv, int nkeys, const OpenClass *keys, const uint32_t *rr, const uint32_t *v,
+             int grind_bits, int queries, uint64_t *out_qs) {
+  Context &c = ctx();
+  int status = c.require();
+  if (status) return status;
+  if (nkeys < 1 || nkeys > 32) {
+    set_error("invalid-parameter: opening keys");
+    return E_PARAM;
+  }
+  Owned mem;
+  std::vector<int> cls(nkeys);
+  std::vector<const uint32_t *> hs(nkeys);
+  for (int k = 0; k < nkeys; k++) {
+    cls[k] = keys[k].c;
+    if (keys[k].c < 1 || keys[k].c > 30 || keys[k].ncols < 1) {
+      set_error("invalid-parameter: opening key");
+      return E_PARAM;
+    }
+    uint32_t *h = mem.alloc(((uint64_t)8) << keys[k].c);
+    if (!h) return E_NOMEM;
+    if ((status = combine_columns_device(8, keys[k].d_columns, keys[k].ncols, (uint64_t)1 << keys[k].c, keys[k].coef, h)))
+      return status;
+    hs[k] = h;
+  }
+  std::vector<uint64_t> qs(queries > 0 ? queries : 1);
+  if ((status = basefold_prove_classes(tr, nv, nkeys, cls.data(), hs.data(), rr, v, grind_bits, queries, qs.data(),
+                                       nullptr, nullptr)))
+    return status;
+  if (out_qs) memcpy(out_qs, qs.data(), 8 * (size_t)queries);
+  for (int k = 0; k < nkeys; k++) {
+    const OpenClass &key = keys[k];
+    std::vector<uint64_t> leaves(queries);
+    for (int q = 0; q < queries; q++) leaves[q] = qs[q] >> (nv - key.c);
+    const int max_depth = cap_level_of((uint64_t)1 << (key.c - 1));
+    std::vector<uint32_t> rows((size_t)queries * key.ncols * 4);
+    std::vector<uint8_t> paths((size_t)queries * max_depth * 32 + 1);
+    int depth = 0;
+    if ((status = open_queries_device(key.d_codewords, key.ncols, key.c, key.d_levels, leaves.data(), queries,
+                                      rows.data(), paths.data(), &depth)))
+      return status;
+    uint64_t d3[3] = {(uint64_t)queries, (uint64_t)key.ncols, 4};
+    if ((status = tr.send(rows.data(), 3, d3, nullptr, false))) return status;
+    if ((status = tr.send_bytes(paths.data(), (int64_t)queries * depth * 32, nullptr, false))) return status;
+  }
+  return OK;
+}
+
+// ---- the verifier's side of that opening, on the host (src/pcs.lisp:39-95, 581-657, 752-843)
+namespace {
+using Digest = std::array<uint8_t, 32>;
+// LEAF-DIGEST (:44-52): rows of 4 values hashed 64 at a time, chained h = BLAKE3(h || d_i)
+Digest host_leaf_digest(const uint32_t *rows, uint64_t nrows) {
+  Digest h{}, d{};
+  bool have = false;
+  std::vector<uint8_t> buf;
+  for (uint64_t start = 0; start < nrows; start += 64) {
+    const uint64_t cnt = std::min<uint64_t>(64, nrows - start);
+    buf.resize(16 * cnt);
+    for (uint64_t k = 0; k < 4 * cnt; k++)
+      for (int b = 0; b < 4; b++) buf[4 * k + b] = (uint8_t)(rows[4 * start + k] >> (8 * b));
+    blake3_hash(buf.data(), buf.size(), d.data(), 32);
+    if (have) {
+      uint8_t hd[64];
+      memcpy(hd, h.data(), 32), memcpy(hd + 32, d.data(), 32);
+      blake3_hash(hd, 64, h.data(), 32);
+    } else {
+      h = d, have = true;
+    }
+  }
+  return h;
+}
+Digest host_node(const uint8_t *left, const uint8_t *right) {  // :54-55
+  uint8_t lr[64];
+  Digest out;
+  memcpy(lr, left, 32), memcpy(lr + 32, right, 32);
+  blake3_hash(lr, 64, out.data(), 32);
+  return out;
+}
+// the twiddle of fold level l at index s in a domain of 2^n points: level 0 holds the powers of the root in
+// bit-reversed order, level l + 1 [s] = level l [2 s]^2 (src/rs.lisp:39-55)
+uint32_t host_twiddle(int n, int l, uint64_t s) {
+  const uint32_t w = fpow(3, (uint64_t)(P - 1) >> n);
+  uint64_t i = s << l, rev = 0;
+  for (int b = 0; b < n - 1; b++) rev |= ((i >> b) & 1) << (n - 2 - b);
+  return fpow(fpow(w, rev), (uint64_t)1 << l);
+}
+// ENCODE (src/rs.lisp:60-85) of 2^(n-1) base values to 2^n symbols, for the final table's few entries
+std::vector<uint32_t> host_encode(const std::vector<uint32_t> &message, int n) {
+  const uint64_t len = (uint64_t)1 << n;
+  std::vector<uint32_t> x(len);
+  for (uint64_t i = 0; i < len; i++) x[i] = message[i % (len / 2)] % P;
+  for (int b = n - 2; b >= 0; b--) {
+    const uint64_t half = (uint64_t)1 << b;
+    for (uint64_t k = 0; k < len / (2 * half); k++) {
+      const uint32_t t = host_twiddle(n, b, k);
+      for (uint64_t j = 0; j < half; j++) {
+        uint32_t &a = x[2 * half * k + j], &cc = x[2 * half * k + half + j];
+        const uint32_t tc = fmul(t, cc), lo = fadd(a, tc), hi = fsub(a, tc);
+        a = lo, cc = hi;
+      }
+    }
+  }
+  return x;
+}
+}  // namespace
+
+// CHECK-PATH with INJECTED-AT (src/pcs.lisp:86-95)
+bool check_path_host(const uint8_t *h_in, const uint8_t *path, int depth, uint64_t i, const uint8_t *cap, int ninj,
+                     const int *inj_level, const uint8_t *inj_digests) {
+  Digest h;
+  memcpy(h.data(), h_in, 32);
+  for (int l = 1; l <= depth; l++) {
+    const uint8_t *sib = path + 32 * (size_t)(l - 1);
+    h = (i & 1) ? host_node(sib, h.data()) : host_node(h.data(), sib);
+    i >>= 1;
+    for (int k = 0; k < ninj; k++)
+      if (inj_level[k] == l) h = host_node(h.data(), inj_digests + 32 * (size_t)k);
+  }
+  return memcmp(h.data(), cap + 32 * i, 32) == 0;
+}
+
+static int reject(const std::string &what) {
+  set_error("verification-failure: pcs: " + what);
+  return E_REJECT;
+}
+
+int pcs_verify_opening(Transcript &tr, int nv, int nkeys, const OpenClass *keys, const uint32_t *rr, const uint32_t *v,
+                       int grind_bits, int queries) {
+  if (nkeys < 1 || nkeys > 32 || keys[nkeys - 1].c != nv || queries < 1) {
+    set_error("invalid-parameter: opening keys");
+    return E_PARAM;
+  }
+  const int fl = nv - 5 > 0 ? nv - 5 : 0, Q = queries;
+  int status;
+  hf::E prf = hf::lift(1, 8), claim = hf::from(v, 8);
+  std::vector<hf::E> chal;
+  std::vector<int> olv;
+  std::vector<std::vector<uint8_t>> caps;
+  for (int i = 0; i < fl; i++) {  // BASEFOLD, the verifier's side
+    uint32_t ev[24], x[8];
+    uint64_t dims[2] = {3, 8};
+    if ((status = tr.send(nullptr, 2, dims, ev))) return status;
+    if (hf::add(hf::from(ev, 8), hf::from(ev + 8, 8)) != claim) return reject("basefold sumcheck round " + std::to_string(i) + " failed");
+    tr.challenge(8, x);
+    chal.push_back(hf::from(x, 8));
+    claim = hf::lagrange({hf::from(ev, 8), hf::from(ev + 8, 8), hf::from(ev + 16, 8)}, hf::from(x, 8));
+    prf = hf::mul(prf, hf::eq1(hf::from(rr + 8 * (size_t)i, 8), hf::from(x, 8)));
+    const int l = i + 1;
+    if (l >= 2 && l < fl && l % 2 == 0) {
+      std::vector<uint8_t> cap;
+      if ((status = tr.send_bytes(nullptr, -1, &cap))) return status;
+      olv.push_back(l);
+      caps.push_back(cap);
+    }
+  }
+  const uint64_t mlen = (uint64_t)1 << (nv - fl);
+  std::vector<uint32_t> m(mlen * 8);
+  {
+    uint64_t dims[2] = {mlen, 8};
+    if ((status = tr.send(nullptr, 2, dims, m.data()))) return status;
+    hf::E mval = fl < nv ? hf::mle_eval(m.data(), nv - fl, rr + 8 * (size_t)fl, 8) : hf::from(m.data(), 8);
+    if (hf::mul(prf, mval) != claim) return reject("basefold final claim");
+  }
+  uint64_t nonce;
+  if ((status = tr.verify_grind(grind_bits, &nonce))) return status;
+  std::vector<uint64_t> qs(Q);
+  tr.challenge_bits(nv - 1, Q, qs.data());
+  // ---- VERIFY-QUERIES: the oracles' leaves and paths (:763-774)
+  std::vector<std::vector<uint32_t>> oleaves(olv.size());
+  for (size_t o = 0; o < olv.size(); o++) {
+    const int l = olv[o];
+    const uint64_t nleaves = (uint64_t)1 << (nv - 1 - l);
+    const int depth = cap_level_of(nleaves);
+    uint64_t d3[3] = {(uint64_t)Q, 8, 4};
+    oleaves[o].assign((size_t)Q * 32, 0);
+    std::vector<uint8_t> paths;
+    if ((status = tr.send(nullptr, 3, d3, oleaves[o].data(), false))) return status;
+    if ((status = tr.send_bytes(nullptr, -1, &paths, false))) return status;
+    if (paths.size() != (size_t)Q * depth * 32) return reject("merkle path length");
+    if (caps[o].size() != 32 * (nleaves >> depth)) return reject("oracle opening shape");
+    for (int q = 0; q < Q; q++) {
+      const Digest h = host_leaf_digest(oleaves[o].data() + 32 * (size_t)q, 8);
+      if (!check_path_host(h.data(), paths.data() + 32 * (size_t)q * depth, depth, qs[q] >> l, caps[o].data(), 0, nullptr,
+                           nullptr))
+        return reject("oracle merkle path");
+    }
+  }
+  // every key's leaves and its tree's paths; inj_c += sum_k coef_k leaf_k (:776-808)
+  std::vector<std::vector<hf::E>> inj(nkeys, std::vector<hf::E>((size_t)Q * 4, hf::zero(8)));
+  for (int k = 0; k < nkeys; k++) {
+    const OpenClass &key = keys[k];
+    if (key.c < 1 || key.c > nv || (k && key.c <= keys[k - 1].c)) {
+      set_error("invalid-parameter: opening keys must ascend in class");
+      return E_PARAM;
+    }
+    const uint64_t nleaves = (uint64_t)1 << (key.c - 1);
+    const int depth = cap_level_of(nleaves), nc = key.ncols;
+    uint64_t d3[3] = {(uint64_t)Q, (uint64_t)nc, 4};
+    std::vector<uint32_t> leaves((size_t)Q * nc * 4);
+    std::vector<uint8_t> paths;
+    if ((status = tr.send(nullptr, 3, d3, leaves.data(), false))) return status;
+    if ((status = tr.send_bytes(nullptr, -1, &paths, false))) return status;
+    if (paths.size() != (size_t)Q * depth * 32) return reject("merkle path length");
+    for (int q = 0; q < Q; q++) {
+      const Digest h = host_leaf_digest(leaves.data() + (size_t)q * nc * 4, nc);
+      if (!check_path_host(h.data(), paths.data() + 32 * (size_t)q * depth, depth, qs[q] >> (nv - key.c), key.cap, 0,
+                           nullptr, nullptr))
+        return reject("merkle path of class " + std::to_string(key.c));
+      for (int sy = 0; sy < 4; sy++) {
+        hf::E &held = inj[k][(size_t)q * 4 + sy];
+        for (int col = 0; col < nc; col++)
+          held = hf::add(held, hf::scale(hf::from(key.coef + 8 * (size_t)col, 8), leaves[((size_t)q * nc + col) * 4 + sy]));
+      }
+    }
+  }
+  // fold each query's symbols down to the final table's codeword (:810-843)
+  std::vector<std::vector<uint32_t>> menc(8);
+  for (int d = 0; d < 8; d++) {  // ENCODE-EXT of the final table, coordinate by coordinate
+    std::vector<uint32_t> col(mlen);
+    for (uint64_t i = 0; i < mlen; i++) col[i] = m[i * 8 + d];
+    menc[d] = host_encode(col, nv - fl + 1);
+  }
+  const uint32_t inv2 = finv(2);
+  for (int q = 0; q < Q; q++) {
+    uint64_t base = 4 * qs[q];
+    std::vector<hf::E> held(4, hf::zero(8));
+    for (int level = 0; level <= fl; level++) {
+      if (level > 0) {
+        const int l = level - 1;
+        std::vector<hf::E> next;
+        for (size_t t2 = 0; t2 + 1 < held.size(); t2 += 2) {  // RS:FOLD (src/rs.lisp:93-101)
+          const uint64_t sidx = base / 2 + t2 / 2;
+          const hf::E &a = held[t2], &b = held[t2 + 1];
+          const hf::E f0 = hf::scale(hf::add(a, b), inv2);
+          const hf::E f1 = hf::scale(hf::sub(a, b), finv(fmul(2, host_twiddle(nv + 1, l, sidx))));
+          next.push_back(hf::add(f0, hf::mul(chal[l], hf::sub(f1, f0))));
+        }
+        held = next;
+        base /= 2;
+        for (size_t o = 0; o < olv.size(); o++)
+          if (olv[o] == level) {
+            const uint32_t *leaf = oleaves[o].data() + 32 * (size_t)q;
+            const uint64_t ob = 4 * (qs[q] >> level);
+            std::vector<hf::E> sym(4, hf::zero(8));
+            for (int sy = 0; sy < 4; sy++)
+              for (int d = 0; d < 8; d++) sym[sy][d] = leaf[4 * d + sy];
+            if (sym[base - ob] != held[0]) return reject("fold consistency");
+            held = sym;
+            base = ob;
+          }
+      }
+      for (int k = 0; k < nkeys; k++)  // INJECT
+        if (nv - keys[k].c == level) {
+          const uint64_t cb = 4 * (qs[q] >> level);
+          for (size_t sy = 0; sy < held.size(); sy++)
+            held[sy] = hf::add(held[sy], inj[k][(size_t)q * 4 + (base - cb) + sy]);
+        }
+    }
+    for (size_t sy = 0; sy < held.size(); sy++)
+      for (int d = 0; d < 8; d++)
+        if (held[sy][d] != menc[d][base + sy]) return reject("final codeword consistency");
   }
   return OK;
 }

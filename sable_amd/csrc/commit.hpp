@@ -40,5 +40,31 @@ int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v
                    int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final);
 int basefold_verify(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,
                     uint64_t *out_qs);
+// BASEFOLD over several size classes (ascending, the last one nv): class c's table d_hs[k] joins at level nv - c
+int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, const uint32_t *const *d_hs,
+                           const uint32_t *rr, const uint32_t *v, int grind_bits, int queries, uint64_t *out_qs,
+                           uint32_t *out_chal, uint32_t *out_final);
+// one key of the final opening: a size class, a unit of its own with its own tree
+struct OpenClass {
+  int c = 0, ncols = 0;
+  const uint32_t *d_columns = nullptr;    // prover: ncols base columns of 2^c values (device)
+  const uint32_t *d_codewords = nullptr;  // prover: their codewords (device)
+  const uint32_t *d_levels = nullptr;     // prover: the tree's levels (device)
+  const uint32_t *coef = nullptr;         // ncols EXT8s (host): the columns' coefficients in the combined column
+  const uint8_t *cap = nullptr;           // verifier: the committed cap (host)
+};
+// COMBINE-COLUMNS per key, BASEFOLD over the classes, OPEN-QUERIES per key (src/pcs.lisp:434-441, 581-657, 721-734)
+int pcs_open(Transcript &tr, int nv, int nkeys, const OpenClass *keys, const uint32_t *rr, const uint32_t *v,
+             int grind_bits, int queries, uint64_t *out_qs);
+// BASEFOLD's verifier side and VERIFY-QUERIES (src/pcs.lisp:752-843), on the host
+int pcs_verify_opening(Transcript &tr, int nv, int nkeys, const OpenClass *keys, const uint32_t *rr, const uint32_t *v,
+                       int grind_bits, int queries);
+// CHECK-PATH with INJECTED-AT (src/pcs.lisp:86-95), on the host
+bool check_path_host(const uint8_t *h, const uint8_t *path, int depth, uint64_t i, const uint8_t *cap, int ninj,
+                     const int *inj_level, const uint8_t *inj_digests);
+// MERKLE-LEVELS with injections (src/pcs.lisp:64-77) from leaf digests on the device: d_levels receives every level,
+// leaves first; d_inj[k] (nleaves >> inj_level[k] digests) is hashed into the nodes of level inj_level[k]
+int merkle_levels_injected_device(const uint32_t *d_leaves, uint64_t nleaves, int ninj, const int *inj_level,
+                                  const uint32_t *const *d_inj, uint32_t *d_levels);
 
 }  // namespace exh

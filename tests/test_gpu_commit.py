@@ -140,8 +140,9 @@ def test_basefold_matches_the_oracle(nv):
 
 def test_basefold_round_trip_beyond_the_oracle_sizes():
     """nv = 19 (the oracle stops near 12): the claim comes from the device's hypercube sum with eq = the
-    point, the prover's own round checks pass, the verifier accepts the proof and its queries' fold
-    consistency, and rejects another claim."""
+    point, the prover's own round checks pass, the verifier's BaseFold side accepts the proof (rounds, final
+    claim, grinding; the query openings are checked by verify-queries, tests/test_gpu_open.py) and rejects
+    another claim."""
     nv = 19
     rng = np.random.default_rng(19)
     h = sa.Table.random(77, 1 << nv, 8)
