@@ -148,6 +148,24 @@ int exh_eq_table_device(int degree_d, int k, const uint32_t *r, exh_table *out);
    p, q: K * 2^(m+1) EXTs each; out_p, out_q: K * 2^m EXTs (children (b,x), (b,x+2^m)) */
 int exh_gkr_reduce_layer(exh_table p, exh_table q, int degree_d, int K, int m, exh_table *out_p, exh_table *out_q);
 
+/* ---- the domain layer's device side (src/domain.lisp:288-331).  A column as the domain holds it: base values,
+   K 2^n for :FULL (kind 0), K 2^(n-c) for :ROW c (kind 1), K 2^c for :COL c (kind 2), without the factor K when
+   shared (MAKE-DOMAIN, src/domain.lisp:36-51) */
+typedef struct {
+  const char *name;
+  int32_t kind, c, shared;
+  exh_table data;
+} exh_domain_column;
+/* TABLE-VALUES (src/domain.lisp:311-321): the sumcheck table of a column's half (0 or 1; -1 for a column with one
+   table, which does not depend on the top in-block variable): K blocks of 2^(n-1) base values -> a new table */
+int exh_domain_table(const exh_domain_column *column, int half, int n, int K, exh_table *out);
+/* DOMAIN-LEAVES (src/domain.lisp:298-309) of one lookup: the forms tag, values[0..n_values) and num (NULL: the
+   numerator 1) over the columns' names; z and betas (n_values * D) canonical.  out_p, out_q: new tables of
+   K * 2^n EXTs, p = num, q = Z - tag - sum_i beta_i v_i, as PROVE-UPPER takes them */
+int exh_domain_leaves(int degree_d, int n, int K, const exh_domain_column *columns, int n_columns, const char *tag,
+                      const char *const *values, int n_values, const char *num, const uint32_t *z,
+                      const uint32_t *betas, exh_table *out_p, exh_table *out_q);
+
 #ifdef __cplusplus
 }
 #endif

@@ -65,6 +65,11 @@ int exh_verify(exh_transcript tr, int n, exh_stmt stmt, const uint32_t *claim, c
 int exh_check_final(exh_stmt stmt, int degree_d, const uint32_t *reduced, const uint32_t *finals,
                     const uint32_t *constants);
 
+/* EVALUATE of the statement's form (src/forms.lisp:214-217) at table values (n_tables * D) and constants, as
+   VERIFY-DOMAIN applies it to the finals of each block (src/domain.lisp:247-248) */
+int exh_stmt_evaluate(exh_stmt stmt, int degree_d, const uint32_t *table_values, const uint32_t *constants,
+                      uint32_t *out);
+
 /* ---- LogUp-GKR (src/gkr.lisp) */
 /* PROVE-UPPER, :215-272.  leaves: 2 * lookups tables (p, q per lookup) of K * 2^n EXTs */
 int exh_gkr_prove_upper(exh_transcript tr, int n, int K, int lookups, const exh_table *leaves,

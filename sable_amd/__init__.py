@@ -105,6 +105,11 @@ class Statement:
     def has_generated_kernel(self, d):
         return load().exh_stmt_has_generated_kernel(C.c_uint64(self.handle), d) == 1
 
+    def free(self):
+        if self.handle:
+            load().exh_stmt_free(C.c_uint64(self.handle))
+            self.handle = 0
+
 
 # ------------------------------------------------------------------ transcript
 class Transcript:

@@ -7,6 +7,7 @@
 #include "../../include/exacta_host.h"
 #include "commit.hpp"
 #include "context.hpp"
+#include "domain.hpp"
 #include "gkr.hpp"
 #include "hostfield.hpp"
 #include "prover.hpp"
@@ -509,6 +510,78 @@ int exh_check_final(exh_stmt stmt, int D, const uint32_t *reduced, const uint32_
   Statement *st = stmt_of(stmt);
   if (!st) return E_PARAM;
   return check_final(*st, D, reduced, finals, constants);
+}
+
+int exh_stmt_evaluate(exh_stmt stmt, int D, const uint32_t *table_values, const uint32_t *constants, uint32_t *out) {
+  Statement *st = stmt_of(stmt);
+  if (!st) return E_PARAM;
+  if (D != 4 && D != 8) {
+    set_error("invalid-parameter: degree");
+    return E_PARAM;
+  }
+  evaluate_statement(*st, D, table_values, constants, out);
+  return OK;
+}
+
+// ------------------------------------------------------------------ domains
+namespace {
+int domain_column_of(const exh_domain_column *in, int n, int K, DomainColumn *out) {
+  DeviceTable *dt = table_of(in->data);
+  if (!dt) return E_PARAM;
+  if (!in->name || dt->stride != 1) {
+    set_error("invalid-parameter: a domain column is a named table of base values");
+    return E_PARAM;
+  }
+  out->name = in->name;
+  for (char &ch : out->name) ch = (char)toupper((unsigned char)ch);
+  out->kind = in->kind, out->c = in->kind == COL_FULL ? 0 : in->c, out->shared = in->shared != 0;
+  out->ptr = dt->ptr, out->entries = dt->n_u32;
+  (void)n, (void)K;
+  return OK;
+}
+}  // namespace
+
+int exh_domain_table(const exh_domain_column *column, int half, int n, int K, exh_table *out) {
+  DomainColumn col;
+  int status = domain_column_of(column, n, K, &col);
+  if (status) return status;
+  if (n < 2 || n > 40 || K < 1) {
+    set_error("invalid-parameter: domain table arguments");
+    return E_PARAM;
+  }
+  if ((status = exh_table_alloc((uint64_t)K << (n - 1), 1, out))) return status;
+  if ((status = domain_table(col, half, n, K, table_of(*out)->ptr))) {
+    exh_table_free(*out);
+    *out = 0;
+  }
+  return status;
+}
+
+int exh_domain_leaves(int D, int n, int K, const exh_domain_column *columns, int n_columns, const char *tag,
+                      const char *const *values, int n_values, const char *num, const uint32_t *z,
+                      const uint32_t *betas, exh_table *out_p, exh_table *out_q) {
+  if ((D != 4 && D != 8) || n < 2 || n > 40 || K < 1 || n_columns < 0 || n_values < 0 || !tag) {
+    set_error("invalid-parameter: domain leaves arguments");
+    return E_PARAM;
+  }
+  std::vector<DomainColumn> cols((size_t)n_columns);
+  int status;
+  for (int k = 0; k < n_columns; k++)
+    if ((status = domain_column_of(columns + k, n, K, &cols[(size_t)k]))) return status;
+  std::vector<std::string> vs;
+  for (int k = 0; k < n_values; k++) vs.push_back(values[k]);
+  uint64_t words = ((uint64_t)K << n) * D;
+  if ((status = exh_table_alloc(words, D, out_p))) return status;
+  if ((status = exh_table_alloc(words, D, out_q))) {
+    exh_table_free(*out_p);
+    return status;
+  }
+  if ((status = domain_leaves(D, n, K, cols, tag, vs, num, z, betas, table_of(*out_p)->ptr, table_of(*out_q)->ptr))) {
+    exh_table_free(*out_p);
+    exh_table_free(*out_q);
+    *out_p = *out_q = 0;
+  }
+  return status;
 }
 
 // ------------------------------------------------------------------ GKR
