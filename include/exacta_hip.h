@@ -46,6 +46,17 @@ const char *exh_last_error(void);
 int exh_synchronize(void);
 /* 1 when a kernel generated for the statement is used, 0 when the interpreter kernel is */
 int exh_stmt_has_generated_kernel(exh_stmt stmt, int degree_d);
+/* ROUND-KERNEL (src/sumcheck.lisp:270-280) compiles a kernel for any statement on first use.  Here the kernels of
+   the statements listed at build time are in the library; for any other statement whose tables have at least
+   2^20 entries (EXACTA_HIP_RTC_MIN_N changes the 20; EXACTA_HIP_NO_RTC switches this off), the first proof starts
+   a compilation of its kernels in the background (hiprtc, seconds to a minute) and runs on the interpreter kernel,
+   and proofs begun after the compilation has ended run on the generated kernels: the same bytes either way.  A
+   process that ends while a compilation runs ends at once with its exit status (C streams flushed, clean-ups
+   registered before the library's first compilation skipped).
+   exh_stmt_generate asks for that compilation ahead of a proof, for round polynomials of the given header degree
+   (-1: the statement's own).  Returns 1 when the kernels are in place, 0 while they compile (wait = 0), or
+   EXH_E_DEVICE with the compiler's log when the compilation failed; with wait != 0 it returns once it has ended. */
+int exh_stmt_generate(exh_stmt stmt, int degree_d, int degree, int wait);
 
 /* ---- measurement (no counterpart in the reference): with profiling on, every data-parallel kernel
    launch is bracketed by HIP events on the library's stream; entries report the kernel, the round it

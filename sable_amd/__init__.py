@@ -105,6 +105,13 @@ class Statement:
     def has_generated_kernel(self, d):
         return load().exh_stmt_has_generated_kernel(C.c_uint64(self.handle), d) == 1
 
+    def generate(self, d, degree=None, wait=True):
+        """exh_stmt_generate: compile kernels for the statement at run time; True once they are in place."""
+        out = load().exh_stmt_generate(C.c_uint64(self.handle), d, -1 if degree is None else degree, 1 if wait else 0)
+        if out < 0:
+            check(out)
+        return out == 1
+
     def free(self):
         if self.handle:
             load().exh_stmt_free(C.c_uint64(self.handle))

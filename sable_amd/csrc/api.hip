@@ -11,6 +11,7 @@
 #include "gkr.hpp"
 #include "hostfield.hpp"
 #include "prover.hpp"
+#include "rtc.hpp"
 #include "sumcheck.hpp"
 #include "transcript.hpp"
 
@@ -233,7 +234,29 @@ int exh_stmt_has_generated_kernel(exh_stmt stmt, int D) {
   if (!st) return E_PARAM;
   Statement copy = *st;
   copy.plan(copy.degree > 1 ? copy.degree : 1);
+  if (ctx().ready) (void)rtc_collect();
   return find_kernels(copy.key(), D) ? 1 : 0;
+}
+int exh_stmt_generate(exh_stmt stmt, int D, int degree, int wait) {
+  Statement *st = stmt_of(stmt);
+  if (!st) return E_PARAM;
+  int status = ctx().require();
+  if (status) return status;
+  if (D != 4 && D != 8) {
+    set_error("invalid-parameter: degree");
+    return E_PARAM;
+  }
+  Statement copy = *st;
+  if (degree < 0) degree = copy.degree;
+  copy.plan(degree > 1 ? degree : 1);
+  if (find_kernels(copy.key(), D)) return 1;
+  StmtDesc desc;
+  if (copy.T() > MAXT || !make_desc(copy, &desc)) {
+    set_error("invalid-parameter: statement beyond the kernels' limits");
+    return E_PARAM;
+  }
+  rtc_request(copy.key(), desc, D);
+  return rtc_status(copy.key(), D, wait != 0);
 }
 
 // ------------------------------------------------------------------ sumcheck sessions

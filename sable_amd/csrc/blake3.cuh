@@ -2,7 +2,9 @@
 // transcript and the device Merkle kernels.  Every hash on the commitment path is a single chunk
 // (at most 1024 bytes: src/pcs.lisp:35, 44-55), so no chunk tree is needed on the device.
 #pragma once
+#if !defined(__HIPCC_RTC__)
 #include <stdint.h>
+#endif
 
 #include "field.cuh"
 

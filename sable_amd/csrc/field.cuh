@@ -8,9 +8,29 @@
 // (four products below p^2 fit 64 bits, as in src/field.lisp:213-218; longer sums use a 96-bit
 // accumulator) and reduced once.
 #pragma once
+// (a run-time compilation of these kernels has the runtime's declarations built in and no host headers)
+#if !defined(__HIPCC_RTC__)
 #include <stdint.h>
+#else
+typedef unsigned char uint8_t;
+typedef unsigned short uint16_t;
+typedef unsigned int uint32_t;
+typedef int int32_t;
+typedef unsigned long long uint64_t;
+typedef long long int64_t;
+typedef __SIZE_TYPE__ size_t;
+#define offsetof(type, member) __builtin_offsetof(type, member)
+namespace std {
+template <class A, class B> struct is_same { static constexpr bool value = false; };
+template <class A> struct is_same<A, A> { static constexpr bool value = true; };
+template <bool C, class A, class B> struct conditional { typedef A type; };
+template <class A, class B> struct conditional<false, A, B> { typedef B type; };
+}  // namespace std
+#endif
 
-#if defined(__HIPCC__)
+#if defined(__HIPCC_RTC__)
+#define EXH_HD __host__ __device__ inline __attribute__((always_inline))
+#elif defined(__HIPCC__)
 #include <hip/hip_runtime.h>
 #define EXH_HD __host__ __device__ inline __attribute__((always_inline))
 #else

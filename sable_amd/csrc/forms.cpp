@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <map>
 #include <memory>
+#include <sstream>
 
 #include "hostfield.hpp"
 #include "transcript.hpp"
@@ -534,6 +535,48 @@ bool make_desc(const Statement &st, StmtDesc *out) {
   d.G = g, d.nacc = st.nacc, d.maxx = maxx;
   *out = d;
   return true;
+}
+
+std::string desc_source(const StmtDesc &d, const std::string &name) {
+  std::ostringstream o;
+  o << "struct " << name << " {\n  static constexpr StmtDesc d = {" << d.T << ", " << d.G << ", " << d.nacc << ", "
+        << d.maxx << ",\n    {";
+  for (int g = 0; g < MAXG; g++) o << d.deg[g] << (g + 1 < MAXG ? "," : "");
+  o << "},\n    {";
+  for (int g = 0; g < MAXG; g++) {
+    o << "{";
+    for (int j = 0; j < MAXDEG; j++) o << d.tab[g][j] << (j + 1 < MAXDEG ? "," : "");
+    o << "}" << (g + 1 < MAXG ? "," : "");
+  }
+  o << "},\n    {";
+  for (int g = 0; g < MAXG; g++) o << d.nev[g] << (g + 1 < MAXG ? "," : "");
+  o << "},\n    {";
+  for (int g = 0; g < MAXG; g++) {
+    o << "{";
+    for (int k = 0; k < MAXEV; k++) o << d.ev[g][k] << (k + 1 < MAXEV ? "," : "");
+    o << "}" << (g + 1 < MAXG ? "," : "");
+  }
+  o << "},\n    " << d.NV << ", {";
+  for (int v = 0; v < MAXV; v++) o << d.vn[v] << (v + 1 < MAXV ? "," : "");
+  o << "},\n    {";
+  for (int v = 0; v < MAXV; v++) {
+    o << "{";
+    for (int k = 0; k < MAXVT; k++) o << d.vtab[v][k] << (k + 1 < MAXVT ? "," : "");
+    o << "}" << (v + 1 < MAXV ? "," : "");
+  }
+  for (int which = 0; which < 2; which++) {
+    o << "},\n    {";
+    for (int v = 0; v < MAXV; v++) {
+      o << "{";
+      for (int k = 0; k < MAXVT; k++)
+        o << (which ? d.vcoefm[v][k] : d.vcoef[v][k]) << "u" << (k + 1 < MAXVT ? "," : "");
+      o << "}" << (v + 1 < MAXV ? "," : "");
+    }
+  }
+  o << "},\n    {";
+  for (int v = 0; v < MAXV; v++) o << d.vconst[v] << "u" << (v + 1 < MAXV ? "," : "");
+  o << "}};\n};\n";
+  return o.str();
 }
 
 void group_coefficients(const Statement &st, int D, const uint32_t *cv, uint32_t *out) {

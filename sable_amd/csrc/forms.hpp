@@ -78,6 +78,9 @@ void evaluate_statement(const Statement &st, int D, const uint32_t *table_vals, 
                         uint32_t *out);
 // the descriptor of the planned statement for the kernels; false when it exceeds their limits
 bool make_desc(const Statement &st, StmtDesc *out);
+// the descriptor as the text of `struct <name> { static constexpr StmtDesc d = {...}; };`, what a kernel is
+// instantiated with, at build time or at run time
+std::string desc_source(const StmtDesc &d, const std::string &name);
 // the groups' coefficients at the constants: out[g*D .. g*D+D)
 void group_coefficients(const Statement &st, int D, const uint32_t *const_vals, uint32_t *out);
 

@@ -1,5 +1,6 @@
 // sumcheck.hip -- sumcheck session: weight tables, round launches, partial-sum reduction, folds.
 #include "sumcheck.hpp"
+#include "rtc.hpp"
 #include <atomic>
 
 #include <string.h>
@@ -178,8 +179,15 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
     set_error("invalid-parameter: statement beyond the kernels' limits");
     return E_PARAM;
   }
+  (void)rtc_collect();
   kernels = find_kernels(st.key(), D);
   generated = kernels != nullptr;
+  if (!generated && !claim_mode && rtc_enabled()) {
+    // no kernel yet for this statement: the interpreter serves this proof; for tables large enough for the
+    // difference to matter, kernels are compiled in the background for the next one
+    static const int min_n = getenv("EXACTA_HIP_RTC_MIN_N") ? atoi(getenv("EXACTA_HIP_RTC_MIN_N")) : 20;
+    if (n >= min_n) rtc_request(st.key(), desc, D);
+  }
   has_eq = eq != nullptr;
   has_bw = bw != nullptr;
   size = (uint64_t)K << n;

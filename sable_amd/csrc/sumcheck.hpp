@@ -13,13 +13,13 @@
 
 namespace exh {
 
-struct KernelSet {  // the launchers generated for one statement and one degree D
-  void (*launch)(const void *args, bool in_base, bool fold, uint32_t grid, hipStream_t stream);
-  void (*launch_tail)(const void *args, uint32_t grid, hipStream_t stream);
+struct KernelSet {  // the launchers generated for one statement and one degree D, at build time or at run time
+  std::function<void(const void *args, bool in_base, bool fold, uint32_t grid, hipStream_t stream)> launch;
+  std::function<void(const void *args, uint32_t grid, hipStream_t stream)> launch_tail;
   // base tables folded twice at once (round 2 after the base-field sweep), and that sweep's slot sums
-  void (*launch_fold2)(const void *args, uint32_t grid, hipStream_t stream);
-  void (*launch_nodes)(const void *args, int pass, uint32_t grid, hipStream_t stream);
-  int nodes_passes;  // launches of launch_nodes per round (0: not available)
+  std::function<void(const void *args, uint32_t grid, hipStream_t stream)> launch_fold2;
+  std::function<void(const void *args, int pass, uint32_t grid, hipStream_t stream)> launch_nodes;
+  int nodes_passes = 0;  // launches of launch_nodes per round (0: not available)
 };
 // EQ-TABLE of k coordinates (canonical, host) into 2^k elements of device memory
 int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out);

@@ -14,10 +14,13 @@
 // Tables, weights and outputs are canonical residues; the sums come out scaled by a power of 1/R
 // (R = 2^32) that the host removes: a group of degree d carries R^-d.
 #pragma once
+// (a run-time compilation of these kernels has the runtime's declarations built in and no host headers)
+#if !defined(__HIPCC_RTC__)
 #include <hip/hip_runtime.h>
 
 #include <stddef.h>
 #include <type_traits>
+#endif
 
 #include "dev_transcript.cuh"
 #include "field.cuh"
