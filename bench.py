@@ -43,7 +43,7 @@ MEASURED = {
     "traffic": {("round_nodes_base", 24): 203495288, ("round_fold2_base", 24): 403802364},
     "int32_mul_per_prove": None,
 }
-KERNEL_SOURCES = ["sumcheck_kernels.cuh", "field.cuh", "dev_transcript.cuh", "blake3.cuh", "stmtdesc.hpp"]
+KERNEL_SOURCES = ["sumcheck_kernels.hpp", "field.hpp", "dev_transcript.hpp", "blake3.hpp", "stmtdesc.hpp"]
 
 
 def kernel_sources_sha256():

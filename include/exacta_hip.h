@@ -13,8 +13,9 @@
  *   - host buffers are borrowed for the duration of a call only; device tables live behind handles;
  *   - every function returns EXH_OK or a negative status; exh_last_error() describes the last failure
  *     of the calling thread in the words of the reference's condition classes (src/conditions.lisp);
- *   - one context, calls serialised by the caller; every call returns after its small result is on
- *     the host; nothing calls back into the host language.
+ *   - one context per process: every entry point takes one process-wide lock, so calls from several threads
+ *     are safe and take turns (they never overlap on the device); handles are shared by all threads; every
+ *     call returns after its small result is on the host; nothing calls back into the host language.
  */
 #ifndef EXACTA_HIP_H
 #define EXACTA_HIP_H

@@ -3,6 +3,7 @@
 
 #include <map>
 #include <memory>
+#include <mutex>
 
 #include "../../include/exacta_host.h"
 #include "commit.hpp"
@@ -18,6 +19,13 @@
 using namespace exh;
 
 namespace {
+// Every entry point runs under one lock: the context, its handle maps, pool, arenas and pinned staging area are
+// one per process, and a host with several threads (ctypes releases Python's lock during a call) would otherwise
+// interleave inside them.  Calls from several threads are therefore safe and take turns; they do not overlap.
+std::recursive_mutex g_api_mutex;
+struct ApiLock {
+  std::lock_guard<std::recursive_mutex> guard{g_api_mutex};
+};
 std::map<uint64_t, std::unique_ptr<Statement>> g_stmts;
 std::map<uint64_t, std::unique_ptr<SumcheckSession>> g_sessions;
 std::map<uint64_t, std::unique_ptr<Transcript>> g_transcripts;
@@ -79,13 +87,18 @@ int gather_tables(const exh_table *tables, int n, int D, uint64_t entries, std::
 extern "C" {
 
 // ------------------------------------------------------------------ context
-int exh_init(int device) { return ctx_init(device); }
+int exh_init(int device) {
+  ApiLock api_lock;
+  return ctx_init(device);
+}
 void exh_shutdown(void) {
+  ApiLock api_lock;
   g_sessions.clear();
   ctx_shutdown();
 }
 const char *exh_last_error(void) { return last_error(); }
 int exh_synchronize(void) {
+  ApiLock api_lock;
   int status = ctx().require();
   if (status) return status;
   EXH_HIP(hipDeviceSynchronize());
@@ -93,6 +106,7 @@ int exh_synchronize(void) {
 }
 
 int exh_profile_enable(int on) {
+  ApiLock api_lock;
   Context &c = ctx();
   int status = c.require();
   if (status) return status;
@@ -101,8 +115,12 @@ int exh_profile_enable(int on) {
   c.profiling = on != 0;
   return OK;
 }
-int exh_profile_count(void) { return (int)ctx().profile.size(); }
+int exh_profile_count(void) {
+  ApiLock api_lock;
+  return (int)ctx().profile.size();
+}
 int exh_profile_entry(int index, char *name, int name_cap, int *round, float *ms, uint64_t *alg_bytes) {
+  ApiLock api_lock;
   Context &c = ctx();
   if (index < 0 || index >= (int)c.profile.size()) {
     set_error("invalid-parameter: profile index");
@@ -125,6 +143,7 @@ int exh_profile_entry(int index, char *name, int name_cap, int *round, float *ms
 
 // ------------------------------------------------------------------ tables
 int exh_table_alloc(uint64_t n_u32, int stride, exh_table *out) {
+  ApiLock api_lock;
   int status = ctx().require();
   if (status) return status;
   if (stride < 1 || stride > 8 || n_u32 % stride) {
@@ -141,6 +160,7 @@ int exh_table_alloc(uint64_t n_u32, int stride, exh_table *out) {
 }
 
 int exh_table_upload(const uint32_t *host, uint64_t n_u32, int stride, exh_table *out) {
+  ApiLock api_lock;
   for (uint64_t i = 0; i < n_u32; i++)
     if (host[i] >= P) {
       set_error("invalid-parameter: table values must be canonical (below p)");
@@ -154,6 +174,7 @@ int exh_table_upload(const uint32_t *host, uint64_t n_u32, int stride, exh_table
 }
 
 int exh_table_wrap(void *device_ptr, uint64_t n_u32, int stride, exh_table *out) {
+  ApiLock api_lock;
   int status = ctx().require();
   if (status) return status;
   if (!device_ptr || stride < 1 || stride > 8 || ((uintptr_t)device_ptr & 15)) {
@@ -165,6 +186,7 @@ int exh_table_wrap(void *device_ptr, uint64_t n_u32, int stride, exh_table *out)
 }
 
 int exh_table_download(exh_table table, uint64_t offset_u32, uint32_t *host, uint64_t n_u32) {
+  ApiLock api_lock;
   DeviceTable *dt = table_of(table);
   if (!dt) return E_PARAM;
   if (offset_u32 + n_u32 > dt->n_u32) {
@@ -177,6 +199,7 @@ int exh_table_download(exh_table table, uint64_t offset_u32, uint32_t *host, uin
 }
 
 int exh_table_free(exh_table table) {
+  ApiLock api_lock;
   DeviceTable *dt = table_of(table);
   if (!dt) return E_PARAM;
   if (dt->owned && dt->ptr) ctx().pool.release(dt->ptr);  // stream-ordered reuse: no wait
@@ -185,11 +208,13 @@ int exh_table_free(exh_table table) {
 }
 
 void *exh_table_device_ptr(exh_table table) {
+  ApiLock api_lock;
   DeviceTable *dt = table_of(table);
   return dt ? dt->ptr : nullptr;
 }
 
 int exh_table_random(uint64_t seed, uint64_t n_u32, int stride, exh_table *out) {
+  ApiLock api_lock;
   std::vector<uint32_t> host(n_u32);
   uint64_t x = seed;
   for (uint64_t i = 0; i < n_u32;) {
@@ -210,6 +235,7 @@ int exh_table_random(uint64_t seed, uint64_t n_u32, int stride, exh_table *out) 
 // ------------------------------------------------------------------ statements
 int exh_stmt_compile(const char *form, const char *const *tables, int n_tables, const char *const *constants,
                      int n_constants, exh_stmt *out) {
+  ApiLock api_lock;
   auto st = std::make_unique<Statement>();
   std::vector<std::string> tn, cn;
   for (int i = 0; i < n_tables; i++) tn.push_back(tables[i]);
@@ -221,15 +247,18 @@ int exh_stmt_compile(const char *form, const char *const *tables, int n_tables, 
   return OK;
 }
 int exh_stmt_degree(exh_stmt stmt) {
+  ApiLock api_lock;
   Statement *st = stmt_of(stmt);
   return st ? st->degree : E_PARAM;
 }
 int exh_stmt_free(exh_stmt stmt) {
+  ApiLock api_lock;
   if (!stmt_of(stmt)) return E_PARAM;
   g_stmts.erase(stmt);
   return OK;
 }
 int exh_stmt_has_generated_kernel(exh_stmt stmt, int D) {
+  ApiLock api_lock;
   Statement *st = stmt_of(stmt);
   if (!st) return E_PARAM;
   Statement copy = *st;
@@ -238,6 +267,7 @@ int exh_stmt_has_generated_kernel(exh_stmt stmt, int D) {
   return find_kernels(copy.key(), D) ? 1 : 0;
 }
 int exh_stmt_generate(exh_stmt stmt, int D, int degree, int wait) {
+  ApiLock api_lock;
   Statement *st = stmt_of(stmt);
   if (!st) return E_PARAM;
   int status = ctx().require();
@@ -262,6 +292,7 @@ int exh_stmt_generate(exh_stmt stmt, int D, int degree, int wait) {
 // ------------------------------------------------------------------ sumcheck sessions
 int exh_sumcheck_begin(exh_stmt stmt, int D, int n, const exh_table *tables, int n_tables, const uint32_t *eq,
                        const uint32_t *bw, int K, const uint32_t *constants, int degree, exh_session *out) {
+  ApiLock api_lock;
   Statement *st = stmt_of(stmt);
   if (!st) return E_PARAM;
   if (n_tables != st->T() || (!bw && K != 1) || K < 1 || n < 0 || n > 40) {
@@ -287,15 +318,18 @@ static SumcheckSession *session_of(exh_session h) {
   return it->second.get();
 }
 int exh_sumcheck_round(exh_session session, uint32_t *out_sums) {
+  ApiLock api_lock;
   SumcheckSession *s = session_of(session);
   return s ? s->round_sums(out_sums) : E_PARAM;
 }
 int exh_sumcheck_fold(exh_session session, const uint32_t *r) {
+  ApiLock api_lock;
   SumcheckSession *s = session_of(session);
   return s ? s->fold(r) : E_PARAM;
 }
 int exh_sumcheck_run(exh_session session, const uint32_t *cv, const uint8_t *block, uint32_t used, uint64_t counter,
                      uint32_t *out_messages, uint32_t *out_challenges) {
+  ApiLock api_lock;
   SumcheckSession *s = session_of(session);
   if (!s || !cv || !block || used > 64 || !out_messages || !out_challenges) {
     set_error("invalid-parameter: exh_sumcheck_run arguments");
@@ -311,6 +345,7 @@ int exh_sumcheck_run(exh_session session, const uint32_t *cv, const uint8_t *blo
   return s->run_device(state, out_messages, out_challenges);
 }
 int exh_sumcheck_finish(exh_session session, uint32_t *finals, uint32_t *const *folded) {
+  ApiLock api_lock;
   SumcheckSession *s = session_of(session);
   if (!s) return E_PARAM;
   int status = s->finish(finals, folded);
@@ -320,11 +355,13 @@ int exh_sumcheck_finish(exh_session session, uint32_t *finals, uint32_t *const *
 
 // ------------------------------------------------------------------ host field helpers
 int exh_ext_mul(int D, const uint32_t *a, const uint32_t *b, uint32_t *out) {
+  ApiLock api_lock;
   if (D != 4 && D != 8) return E_PARAM;
   hf::mul_raw(D, a, b, out);
   return OK;
 }
 int exh_ext_inv(int D, const uint32_t *a, uint32_t *out) {
+  ApiLock api_lock;
   if (D != 4 && D != 8) return E_PARAM;
   hf::E x = hf::from(a, D);
   if (hf::is_zero(x)) {
@@ -337,6 +374,7 @@ int exh_ext_inv(int D, const uint32_t *a, uint32_t *out) {
   return OK;
 }
 int exh_eq_table(int D, int k, const uint32_t *r, uint32_t *out) {
+  ApiLock api_lock;
   if ((D != 4 && D != 8) || k < 0 || k > 24) return E_PARAM;
   std::vector<uint32_t> t = hf::eq_table(r, k, D);
   memcpy(out, t.data(), t.size() * 4);
@@ -344,6 +382,7 @@ int exh_eq_table(int D, int k, const uint32_t *r, uint32_t *out) {
 }
 
 int exh_eq_table_device(int D, int k, const uint32_t *r, exh_table *out) {
+  ApiLock api_lock;
   if ((D != 4 && D != 8) || k < 0 || k > 26 || (k > 0 && !r) || !out) {
     set_error("invalid-parameter: eq table of k <= 26 coordinates of degree 4 or 8");
     return E_PARAM;
@@ -357,11 +396,13 @@ int exh_eq_table_device(int D, int k, const uint32_t *r, exh_table *out) {
 
 // ------------------------------------------------------------------ transcript
 int exh_blake3(const uint8_t *in, uint64_t len, uint8_t *out, uint64_t out_len) {
+  ApiLock api_lock;
   blake3_hash(in, len, out, out_len);
   return OK;
 }
 int exh_transcript_new(const uint8_t *label, uint64_t label_len, int D, const uint8_t *proof, uint64_t proof_len,
                        exh_transcript *out) {
+  ApiLock api_lock;
   if (D != 4 && D != 8) {
     set_error("invalid-parameter: degree: expected 4 or 8");
     return E_PARAM;
@@ -381,11 +422,13 @@ int exh_transcript_new(const uint8_t *label, uint64_t label_len, int D, const ui
   return OK;
 }
 int exh_transcript_free(exh_transcript h) {
+  ApiLock api_lock;
   if (!tr_of(h)) return E_PARAM;
   g_transcripts.erase(h);
   return OK;
 }
 int exh_transcript_absorb(exh_transcript h, const uint8_t *data, uint64_t len) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   tr->absorb(data, len);
@@ -393,6 +436,7 @@ int exh_transcript_absorb(exh_transcript h, const uint8_t *data, uint64_t len) {
 }
 int exh_transcript_send(exh_transcript h, const uint32_t *vals, int rank, const uint64_t *dims, uint32_t *out,
                         int absorb) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   int status = tr->send(vals, rank, dims, out, absorb != 0);
@@ -402,6 +446,7 @@ int exh_transcript_send(exh_transcript h, const uint32_t *vals, int rank, const 
 }
 int exh_transcript_send_bytes(exh_transcript h, const uint8_t *bytes, int64_t len, uint8_t *out, uint64_t cap,
                               uint64_t *out_len, int absorb) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   std::vector<uint8_t> got;
@@ -414,24 +459,28 @@ int exh_transcript_send_bytes(exh_transcript h, const uint8_t *bytes, int64_t le
   return OK;
 }
 int exh_transcript_challenge_base(exh_transcript h, int k, uint32_t *out) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   tr->challenge_base(k, out);
   return OK;
 }
 int exh_transcript_challenge_bits(exh_transcript h, int nbits, int k, uint64_t *out) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   tr->challenge_bits(nbits, k, out);
   return OK;
 }
 int exh_transcript_grind(exh_transcript h, int bits, uint64_t *nonce) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   *nonce = tr->grind(bits);
   return OK;
 }
 int exh_transcript_verify_grind(exh_transcript h, int bits, uint64_t *nonce) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   int status = tr->verify_grind(bits, nonce);
@@ -439,12 +488,14 @@ int exh_transcript_verify_grind(exh_transcript h, int bits, uint64_t *nonce) {
   return status;
 }
 int exh_transcript_digest(exh_transcript h, uint8_t out[32]) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   tr->state.digest(out, 32);
   return OK;
 }
 int exh_transcript_state(exh_transcript h, uint32_t cv[8], uint8_t block[64], uint32_t *used, uint64_t *counter) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr || !cv || !block || !used || !counter) return E_PARAM;
   memcpy(cv, tr->state.cv, 32);
@@ -455,16 +506,19 @@ int exh_transcript_state(exh_transcript h, uint32_t cv[8], uint8_t block[64], ui
   return OK;
 }
 int exh_transcript_finished(exh_transcript h) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   return tr ? (tr->finished() ? 1 : 0) : E_PARAM;
 }
 int exh_transcript_message_count(exh_transcript h, uint64_t *count) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   *count = tr->messages.size();
   return OK;
 }
 int exh_transcript_proof(exh_transcript h, uint8_t *out, uint64_t cap, uint64_t *out_len) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   std::vector<uint8_t> bytes = tr->encode_proof();
@@ -476,6 +530,7 @@ int exh_transcript_proof(exh_transcript h, uint8_t *out, uint64_t cap, uint64_t 
 // ------------------------------------------------------------------ sumcheck protocol
 int exh_hypercube_sum(exh_stmt stmt, int D, int n, const exh_table *tables, int n_tables, const uint32_t *eq,
                       const uint32_t *constants, uint32_t *out) {
+  ApiLock api_lock;
   Statement *st = stmt_of(stmt);
   if (!st) return E_PARAM;
   if (n_tables != st->T()) {
@@ -504,6 +559,7 @@ int exh_hypercube_sum(exh_stmt stmt, int D, int n, const exh_table *tables, int 
 int exh_prove(exh_transcript h, int n, exh_stmt stmt, const exh_table *tables, int n_tables, const uint32_t *eq,
               const uint32_t *constants, const uint8_t *label, uint64_t label_len, const uint32_t *bw, int K,
               int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   Statement *st = stmt_of(stmt);
   if (!tr || !st) return E_PARAM;
@@ -522,6 +578,7 @@ int exh_prove(exh_transcript h, int n, exh_stmt stmt, const exh_table *tables, i
 int exh_verify(exh_transcript h, int n, exh_stmt stmt, const uint32_t *claim, const uint32_t *eq,
                const uint32_t *constants, int blocks, const uint8_t *label, uint64_t label_len, int degree,
                uint32_t *out_chal, uint32_t *out_reduced) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   Statement *st = stmt_of(stmt);
   if (!tr || !st) return E_PARAM;
@@ -530,12 +587,14 @@ int exh_verify(exh_transcript h, int n, exh_stmt stmt, const uint32_t *claim, co
 }
 
 int exh_check_final(exh_stmt stmt, int D, const uint32_t *reduced, const uint32_t *finals, const uint32_t *constants) {
+  ApiLock api_lock;
   Statement *st = stmt_of(stmt);
   if (!st) return E_PARAM;
   return check_final(*st, D, reduced, finals, constants);
 }
 
 int exh_stmt_evaluate(exh_stmt stmt, int D, const uint32_t *table_values, const uint32_t *constants, uint32_t *out) {
+  ApiLock api_lock;
   Statement *st = stmt_of(stmt);
   if (!st) return E_PARAM;
   if (D != 4 && D != 8) {
@@ -565,6 +624,7 @@ int domain_column_of(const exh_domain_column *in, int n, int K, DomainColumn *ou
 }  // namespace
 
 int exh_domain_table(const exh_domain_column *column, int half, int n, int K, exh_table *out) {
+  ApiLock api_lock;
   DomainColumn col;
   int status = domain_column_of(column, n, K, &col);
   if (status) return status;
@@ -583,6 +643,7 @@ int exh_domain_table(const exh_domain_column *column, int half, int n, int K, ex
 int exh_domain_leaves(int D, int n, int K, const exh_domain_column *columns, int n_columns, const char *tag,
                       const char *const *values, int n_values, const char *num, const uint32_t *z,
                       const uint32_t *betas, exh_table *out_p, exh_table *out_q) {
+  ApiLock api_lock;
   if ((D != 4 && D != 8) || n < 2 || n > 40 || K < 1 || n_columns < 0 || n_values < 0 || !tag) {
     set_error("invalid-parameter: domain leaves arguments");
     return E_PARAM;
@@ -609,6 +670,7 @@ int exh_domain_leaves(int D, int n, int K, const exh_domain_column *columns, int
 
 // ------------------------------------------------------------------ GKR
 int exh_gkr_reduce_layer(exh_table p, exh_table q, int D, int K, int m, exh_table *out_p, exh_table *out_q) {
+  ApiLock api_lock;
   DeviceTable *dp = table_of(p), *dq = table_of(q);
   if (!dp || !dq) return E_PARAM;
   uint64_t in_entries = (uint64_t)K << (m + 1);
@@ -625,6 +687,7 @@ int exh_gkr_reduce_layer(exh_table p, exh_table q, int D, int K, int m, exh_tabl
 
 int exh_gkr_prove_upper(exh_transcript h, int n, int K, int lookups, const exh_table *leaves, const uint8_t *label,
                         uint64_t label_len, uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp, uint32_t *out_cq) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   std::vector<const uint32_t *> ptrs;
@@ -643,6 +706,7 @@ int exh_gkr_prove_upper(exh_transcript h, int n, int K, int lookups, const exh_t
 int exh_gkr_verify_upper(exh_transcript h, int n, int K, int lookups, const uint8_t *label, uint64_t label_len,
                          uint32_t *out_roots, uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp,
                          uint32_t *out_cq) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   return gkr_verify_upper(*tr, n, K, lookups, std::string((const char *)label, label_len), out_roots, out_ri, out_rb,
@@ -651,6 +715,7 @@ int exh_gkr_verify_upper(exh_transcript h, int n, int K, int lookups, const uint
 
 // ------------------------------------------------------------------ Reed-Solomon, Merkle, BaseFold
 int exh_rs_encode(exh_table messages, int ncols, int c, exh_table *codewords) {
+  ApiLock api_lock;
   DeviceTable *m = table_of(messages);
   if (!m) return E_PARAM;
   if (ncols < 1 || c < 0 || c > 23 || m->stride != 1 || m->n_u32 != ((uint64_t)ncols << c)) {
@@ -663,6 +728,7 @@ int exh_rs_encode(exh_table messages, int ncols, int c, exh_table *codewords) {
 }
 
 int exh_merkle_commit(exh_table codewords, int ncols, int c, exh_table *levels, uint8_t *cap, uint64_t *cap_rows) {
+  ApiLock api_lock;
   DeviceTable *cw = table_of(codewords);
   if (!cw) return E_PARAM;
   if (ncols < 1 || c < 1 || c > 23 || cw->n_u32 != ((uint64_t)ncols << (c + 1))) {
@@ -683,6 +749,7 @@ int exh_merkle_commit(exh_table codewords, int ncols, int c, exh_table *levels, 
 
 int exh_open_queries(exh_table codewords, int ncols, int c, exh_table levels, const uint64_t *leaves, int count,
                      uint32_t *out_leaves, uint8_t *out_paths, int *out_depth) {
+  ApiLock api_lock;
   DeviceTable *cw = table_of(codewords);
   if (!cw) return E_PARAM;
   if (ncols < 1 || c < 1 || c > 23 || cw->n_u32 != ((uint64_t)ncols << (c + 1))) {
@@ -713,6 +780,7 @@ int exh_open_queries(exh_table codewords, int ncols, int c, exh_table levels, co
 }
 
 int exh_rs_fold(exh_table codeword, int D, uint64_t m, int n_domain, int level, const uint32_t *r, exh_table *out) {
+  ApiLock api_lock;
   DeviceTable *cw = table_of(codeword);
   if (!cw) return E_PARAM;
   if ((D != 4 && D != 8) || cw->n_u32 != 2 * m * D || n_domain < 1 || n_domain > 24 || level < 0 ||
@@ -722,10 +790,15 @@ int exh_rs_fold(exh_table codeword, int D, uint64_t m, int n_domain, int level, 
   }
   int status = exh_table_alloc(m * D, D, out);
   if (status) return status;
-  return rs_fold_device(D, m, n_domain, level, cw->ptr, r, table_of(*out)->ptr);
+  if ((status = rs_fold_device(D, m, n_domain, level, cw->ptr, r, table_of(*out)->ptr))) {
+    exh_table_free(*out);
+    *out = 0;
+  }
+  return status;
 }
 
 int exh_table_scale_add(exh_table h, const uint32_t *scale, exh_table column, exh_table *out) {
+  ApiLock api_lock;
   DeviceTable *tc = table_of(column), *th = h ? table_of(h) : nullptr;
   if (!tc || (h && !th)) return E_PARAM;
   const int D = tc->stride;
@@ -741,6 +814,7 @@ int exh_table_scale_add(exh_table h, const uint32_t *scale, exh_table column, ex
 }
 
 int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out) {
+  ApiLock api_lock;
   DeviceTable *te = table_of(e), *tv = table_of(v);
   if (!te || !tv) return E_PARAM;
   if (!out || te->stride != 8 || tv->stride != 8 || te->n_u32 != tv->n_u32 || te->n_u32 < 16 || (te->n_u32 / 8) % 2) {
@@ -780,6 +854,7 @@ static int open_keys(const exh_open_key *keys, int n_keys, bool prover, std::vec
 
 int exh_pcs_open(exh_transcript h, int nv, int n_keys, const exh_open_key *keys, const uint32_t *rr, const uint32_t *v,
                  int grind_bits, int queries, uint64_t *out_qs) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr || !rr || !v) return E_PARAM;
   std::vector<OpenClass> oc;
@@ -790,6 +865,7 @@ int exh_pcs_open(exh_transcript h, int nv, int n_keys, const exh_open_key *keys,
 
 int exh_pcs_verify_opening(exh_transcript h, int nv, int n_keys, const exh_open_key *keys, const uint32_t *rr,
                            const uint32_t *v, int grind_bits, int queries) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr || !rr || !v) return E_PARAM;
   std::vector<OpenClass> oc;
@@ -800,6 +876,7 @@ int exh_pcs_verify_opening(exh_transcript h, int nv, int n_keys, const exh_open_
 
 int exh_merkle_levels_injected(exh_table leaves, int n_injected, const int32_t *inject_level, const exh_table *injected,
                                exh_table *levels) {
+  ApiLock api_lock;
   DeviceTable *lv = table_of(leaves);
   if (!lv || !levels || n_injected < 0 || n_injected > 16 || lv->n_u32 % 8) return E_PARAM;
   const uint64_t nleaves = lv->n_u32 / 8;
@@ -823,12 +900,14 @@ int exh_merkle_levels_injected(exh_table leaves, int n_injected, const int32_t *
 
 int exh_check_path(const uint8_t h[32], const uint8_t *path, int depth, uint64_t i, const uint8_t *cap, int n_injected,
                    const int32_t *inject_level, const uint8_t *injected_digests) {
+  ApiLock api_lock;
   if (!h || !cap || depth < 0 || (depth && !path)) return E_PARAM;
   std::vector<int> at(inject_level, inject_level + (n_injected > 0 ? n_injected : 0));
   return check_path_host(h, path, depth, i, cap, n_injected, at.data(), injected_digests) ? 1 : 0;
 }
 
 int exh_dot_pairs_static(exh_table e, exh_table v, uint32_t *out) {
+  ApiLock api_lock;
   DeviceTable *te = table_of(e), *tv = table_of(v);
   if (!te || !tv) return E_PARAM;
   if (!out || te->stride != 8 || tv->stride != 8 || te->n_u32 != tv->n_u32 || te->n_u32 < 16 || (te->n_u32 / 8) % 2) {
@@ -839,6 +918,7 @@ int exh_dot_pairs_static(exh_table e, exh_table v, uint32_t *out) {
 }
 
 int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out) {
+  ApiLock api_lock;
   DeviceTable *t = table_of(table);
   if (!t) return E_PARAM;
   const int D = t->stride;
@@ -855,6 +935,7 @@ int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out) {
 }
 
 int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int D, const uint32_t *coefficients, exh_table *out) {
+  ApiLock api_lock;
   DeviceTable *cols = table_of(columns);
   if (!cols) return E_PARAM;
   if ((D != 4 && D != 8) || ncols < 1 || len < 1 || !coefficients || !out || cols->stride != 1 ||
@@ -870,6 +951,7 @@ int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int D, const
 }
 
 int exh_pcs_commit(exh_transcript h, exh_table columns, int ncols, int c, exh_table *codewords, exh_table *levels) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   exh_table cw;
@@ -882,15 +964,24 @@ int exh_pcs_commit(exh_transcript h, exh_table columns, int ncols, int c, exh_ta
     return status;
   }
   status = tr->send_bytes(cap.data(), (int64_t)(32 * rows), nullptr);
+  if (status) {  // nothing is handed back on failure
+    exh_table_free(cw);
+    if (levels) {
+      exh_table_free(*levels);
+      *levels = 0;
+    }
+    return status;
+  }
   if (codewords)
     *codewords = cw;
   else
     exh_table_free(cw);
-  return status;
+  return OK;
 }
 
 int exh_basefold_prove(exh_transcript h, int nv, const uint32_t *rr, const uint32_t *v, exh_table table, int grind_bits,
                        int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   DeviceTable *dt = table_of(table);
   if (!tr || !dt) return E_PARAM;
@@ -903,6 +994,7 @@ int exh_basefold_prove(exh_transcript h, int nv, const uint32_t *rr, const uint3
 
 int exh_basefold_verify(exh_transcript h, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,
                         uint64_t *out_qs) {
+  ApiLock api_lock;
   Transcript *tr = tr_of(h);
   if (!tr) return E_PARAM;
   return basefold_verify(*tr, nv, rr, v, grind_bits, queries, out_qs);

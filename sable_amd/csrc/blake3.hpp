@@ -1,4 +1,4 @@
-// blake3.cuh -- the BLAKE3 compression function and single-chunk hashing, shared by the host
+// blake3.hpp -- the BLAKE3 compression function and single-chunk hashing, shared by the host
 // transcript and the device Merkle kernels.  Every hash on the commitment path is a single chunk
 // (at most 1024 bytes: src/pcs.lisp:35, 44-55), so no chunk tree is needed on the device.
 #pragma once
@@ -6,7 +6,7 @@
 #include <stdint.h>
 #endif
 
-#include "field.cuh"
+#include "field.hpp"
 
 namespace exh {
 

@@ -9,10 +9,10 @@
 #include <map>
 #include <vector>
 
-#include "blake3.cuh"
+#include "blake3.hpp"
 #include "context.hpp"
 #include "hostfield.hpp"
-#include "sumcheck_kernels.cuh"
+#include "sumcheck_kernels.hpp"
 
 namespace exh {
 

@@ -1,4 +1,4 @@
-// dev_transcript.cuh -- the Fiat-Shamir transcript on the device, so the rounds of a sumcheck run back
+// dev_transcript.hpp -- the Fiat-Shamir transcript on the device, so the rounds of a sumcheck run back
 // to back without a host round trip: the sequential BLAKE3 mode (src/blake3.lisp:125-155) and the
 // transcript operations a prover round needs (src/transcript.lisp:95-100, 116-128, 152-176).  It absorbs
 // and squeezes exactly the bytes the host transcript would; the host replays the logged messages into
@@ -11,7 +11,7 @@
 // is a DevB3S in device memory; while running, the pending block is a 128-byte ring in LDS (two 64-byte
 // halves used alternately), so words are appended with one (possibly unaligned) store.
 #pragma once
-#include "blake3.cuh"
+#include "blake3.hpp"
 
 namespace exh {
 

@@ -4,7 +4,7 @@
 #include <string.h>
 
 #include "context.hpp"
-#include "field.cuh"
+#include "field.hpp"
 #include "forms.hpp"
 
 namespace exh {

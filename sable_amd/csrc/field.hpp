@@ -1,4 +1,4 @@
-// field.cuh -- KoalaBear F_p (p = 2^31 - 2^24 + 1) and its towers F_p^4 / F_p^8 for gfx950.
+// field.hpp -- KoalaBear F_p (p = 2^31 - 2^24 + 1) and its towers F_p^4 / F_p^8 for gfx950.
 //
 // Values in memory are canonical residues in [0, p), extension elements are D words in the
 // reference's tower order (src/field.lisp:8-11): coordinate i is the coefficient of w^bitrev(i) in

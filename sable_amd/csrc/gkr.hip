@@ -9,7 +9,7 @@
 #include "forms.hpp"
 #include "hostfield.hpp"
 #include "prover.hpp"
-#include "sumcheck_kernels.cuh"
+#include "sumcheck_kernels.hpp"
 
 namespace exh {
 

@@ -5,7 +5,7 @@
 
 #include <vector>
 
-#include "field.cuh"
+#include "field.hpp"
 
 namespace exh {
 namespace hf {

@@ -69,7 +69,7 @@ void compile_part(Job *job, Part *part) {
   }
   // the descriptor sits in an unnamed namespace, as in the sources generated at build time: with external linkage
   // its fields do not fold to constants before the loops over them are unrolled, and the compilation does not end
-  std::string source = "#include \"sumcheck_kernels.cuh\"\nnamespace exh {\nnamespace {\n" +
+  std::string source = "#include \"sumcheck_kernels.hpp\"\nnamespace exh {\nnamespace {\n" +
                        desc_source(job->desc, "RtStmt") + "}\n}\n";
   const char *names[kNSources], *texts[kNSources];
   for (int i = 0; i < kNSources; i++) names[i] = kSources[i].name, texts[i] = kSources[i].text;
@@ -186,6 +186,11 @@ int load_job(Job *job) {
   };
   set.launch_tail = [=](const void *args, uint32_t grid, hipStream_t s) {
     launch_module(tail, args, grid, D == 4 ? tail_lds<4>(args) : tail_lds<8>(args), s);
+  };
+  set.tail_blocks_per_cu = [=](uint32_t lds_bytes) {
+    int blocks = 0;
+    if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, tail, BLOCK, lds_bytes) != hipSuccess) return -1;
+    return blocks;
   };
   set.nodes_passes = passes;
   register_kernels(job->key, job->D, set);

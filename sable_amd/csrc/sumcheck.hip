@@ -128,6 +128,18 @@ static void launch_tail_interp(const TailArgs<D> &a, const StmtDesc &d, uint32_t
   hipLaunchKernelGGL((tail_kernel_interp<D>), dim3(grid), dim3(BLOCK), a.lds_bytes, s, a, d);
 }
 
+template <int D>
+static int tail_interp_blocks_per_cu(uint32_t lds_bytes) {
+  if (lds_bytes > TAIL_LDS_BYTES)
+    (void)hipFuncSetAttribute((const void *)tail_kernel_interp<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              SLICE_LDS_BYTES);
+  int blocks = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, (const void *)tail_kernel_interp<D>, BLOCK, lds_bytes) !=
+      hipSuccess)
+    return -1;
+  return blocks;
+}
+
 // ------------------------------------------------------------------ registry of generated kernels
 static std::map<std::pair<std::string, int>, KernelSet> &registry() {
   static std::map<std::pair<std::string, int>, KernelSet> r;
@@ -376,6 +388,11 @@ int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out) {
     set_error("device-out-of-memory: eq factors");
     return E_NOMEM;
   }
+  struct Release {  // the pooled buffer goes back on every way out
+    Pool &pool;
+    void *ptr;
+    ~Release() { pool.release(ptr); }
+  } release{c.pool, d_factors};
   EXH_HIP(hipMemcpyAsync(d_factors, factors.data(), factors.size() * 4, hipMemcpyHostToDevice, c.stream));
   EqTables eqt;
   memset(&eqt, 0, sizeof(eqt));
@@ -390,7 +407,6 @@ int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out) {
                        (uint32_t)factors.size(), d_out, total, nullptr, (uint64_t)0);
   EXH_HIP(hipGetLastError());
   EXH_HIP(hipStreamSynchronize(c.stream));  // `factors` (pageable) and the pooled buffer are free to go after this
-  c.pool.release(d_factors);
   return OK;
 }
 
@@ -752,11 +768,21 @@ static uint64_t tail_pairs(int T, int D) {
   return p;
 }
 
+bool SumcheckSession::device_capable() const {
+  if (points > MAXPTS || n > MAXROUNDS) return false;
+  // the session's staged eq point and block weights, then the loop's message map, constant terms and the head
+  // of the control block share one pinned staging area (many block weights overflow it: the host-driven rounds
+  // take such a session)
+  const size_t up_words = (size_t)points * std::max(st.nacc, 1) * D + (size_t)n * points * D + offsetof(Ctrl, msg) / 4;
+  return setup_words + up_words <= PIN_BEGIN_WORDS + PIN_LOOP_WORDS;
+}
+
 int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges, DevB3S *final_state) {
   Context &c = ctx();
   if (int owned = owns_arenas()) return owned;
   if (round != 0 || pending_fold || claim_mode || !device_capable()) {
-    set_error("invalid-parameter: the device loop starts a fresh session of at most 7 wire points");
+    set_error("invalid-parameter: the device loop starts a fresh session of at most 7 wire points whose constants "
+              "fit its staging buffer");
     return E_PARAM;
   }
   if (n == 0) return OK;
@@ -765,10 +791,6 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   // (staged in pinned memory: message map | constant terms | head of the control block)
   const size_t mt_words = (size_t)points * std::max(nacc, 1) * D, c0_words = (size_t)n * points * D;
   const size_t head_words = offsetof(Ctrl, msg) / 4, up_words = mt_words + c0_words + head_words;
-  if (setup_words + up_words > PIN_BEGIN_WORDS + PIN_LOOP_WORDS) {
-    set_error("invalid-parameter: statement beyond the device loop's staging buffer");
-    return E_PARAM;
-  }
   // (right behind the session's staged eq point and block weights: the device keeps the same order)
   uint32_t *up = c.host_pinned + PIN_BEGIN + setup_words;
   memset(up, 0, up_words * 4);
@@ -862,7 +884,23 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       uint64_t grid = 1;
       while (grid * 2 <= grid_max && grid * 2 <= left && (n_pairs / (grid * 2)) >= BLOCK) grid *= 2;
       while (n_pairs / grid > slice_max && grid * 2 <= grid_max && grid * 2 <= left) grid *= 2;
+      // the grid's workgroups wait for one another: all of them must be resident at once.  The runtime says how
+      // many of this kernel a compute unit holds with the slices' LDS; a grid beyond that stays on the streaming
+      // kernels (asked once per kernel and size)
+      bool resident = true;
       if (count > 0 && grid > 1 && n_pairs / grid <= slice_max) {
+        const uint32_t lds_bytes = (uint32_t)((uint64_t)T * (2 * n_pairs / grid) * D * 4);
+        static std::map<std::pair<const void *, uint32_t>, int> asked;
+        auto key = std::make_pair(generated ? (const void *)kernels : (const void *)(uintptr_t)D, lds_bytes);
+        auto it = asked.find(key);
+        if (it == asked.end()) {
+          int blocks = generated ? (kernels->tail_blocks_per_cu ? kernels->tail_blocks_per_cu(lds_bytes) : -1)
+                                 : (D == 4 ? tail_interp_blocks_per_cu<4>(lds_bytes) : tail_interp_blocks_per_cu<8>(lds_bytes));
+          it = asked.emplace(key, blocks).first;
+        }
+        resident = it->second < 0 || (uint64_t)it->second * (uint64_t)std::max(c.compute_units, 1) >= grid;
+      }
+      if (count > 0 && grid > 1 && n_pairs / grid <= slice_max && resident) {
         status = launch_tail(j, count, (uint32_t)grid, fold_due);
         folds_due = 0;
         tail_done = status == OK;  // the tables are contiguous in one arena, nothing pending
@@ -951,6 +989,10 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   const Ctrl *rc = reinterpret_cast<const Ctrl *>(down);
   if (with_finals) final_cache.assign(down + ctrl_words, down + ctrl_words + final_words);
   if (in_ctrl) final_cache.assign(rc->finals, rc->finals + final_words);
+  if (rc->gave_up) {
+    set_error("device-error: a workgroup of the grid launch gave up waiting for the others");
+    return E_DEVICE;
+  }
   if ((int)rc->round != n) {
     set_error("device-error: the device loop completed " + std::to_string(rc->round) + " of " + std::to_string(n) +
               " rounds");

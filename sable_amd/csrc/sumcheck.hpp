@@ -9,7 +9,7 @@
 #include <vector>
 
 #include "forms.hpp"
-#include "sumcheck_kernels.cuh"
+#include "sumcheck_kernels.hpp"
 
 namespace exh {
 
@@ -20,6 +20,8 @@ struct KernelSet {  // the launchers generated for one statement and one degree 
   std::function<void(const void *args, uint32_t grid, hipStream_t stream)> launch_fold2;
   std::function<void(const void *args, int pass, uint32_t grid, hipStream_t stream)> launch_nodes;
   int nodes_passes = 0;  // launches of launch_nodes per round (0: not available)
+  // workgroups of the tail kernel a compute unit holds at once with that much dynamic LDS (-1: unknown)
+  std::function<int(uint32_t lds_bytes)> tail_blocks_per_cu;
 };
 // EQ-TABLE of k coordinates (canonical, host) into 2^k elements of device memory
 int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out);
@@ -89,7 +91,8 @@ struct SumcheckSession {
   int run_device(const DevB3S &state, uint32_t *messages, uint32_t *challenges, DevB3S *final_state = nullptr);
   // rounds first_round .. first_round + rounds - 1 with the tables in LDS, over `grid` workgroups
   int launch_tail(int first_round, int rounds, uint32_t grid, bool first_fold);
-  bool device_capable() const { return points <= MAXPTS && n <= MAXROUNDS; }
+  // the device-driven loop fits this session: rounds, wire points, and its constants in the pinned staging area
+  bool device_capable() const;
   int fold(const uint32_t *r /* D */);
   // finals: T * D; folded[t] (optional): K * D each
   int finish(uint32_t *finals, uint32_t *const *folded);

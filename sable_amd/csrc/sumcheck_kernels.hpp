@@ -1,4 +1,4 @@
-// sumcheck_kernels.cuh -- the sumcheck prover's round kernel for gfx950, generated per statement.
+// sumcheck_kernels.hpp -- the sumcheck prover's round kernel for gfx950, generated per statement.
 //
 // One launch does, for every pair i of the tables being summed,
 //   [FOLD]  bind the previous round's variable: read four entries per table, write the two folded
@@ -22,8 +22,8 @@
 #include <type_traits>
 #endif
 
-#include "dev_transcript.cuh"
-#include "field.cuh"
+#include "dev_transcript.hpp"
+#include "field.hpp"
 #include "stmtdesc.hpp"
 
 namespace exh {
@@ -38,8 +38,9 @@ constexpr int MAXTAIL = 16;    // rounds the tail kernel can take
 struct Ctrl {
   DevB3S tr;
   uint32_t r_mont[8];
-  uint32_t round;  // rounds completed
-  uint32_t pad[3];
+  uint32_t round;    // rounds completed
+  uint32_t gave_up;  // set by a workgroup of a grid launch whose wait for the others ran out: the proof is void
+  uint32_t pad[2];
   uint32_t msg[MAXROUNDS][MAXPTS * 8];
   uint32_t chal[MAXROUNDS][8];
   uint32_t finals[MAXT * 8];  // entry 0 of every table once a single entry is left
@@ -950,7 +951,12 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
           }
           epi.prod[u] = f_canonical((double)(v & (((unsigned long long)1 << 48) - 1)));  // exact below 2^53
         }
-        if (!__syncthreads_and(complete)) return;
+        if (!__syncthreads_and(complete)) {
+          // leave a mark: the others may have seen this workgroup's sums and go on to publish the rounds, but
+          // its slice is never written
+          if (tid == 0) __hip_atomic_store(&args.ctrl->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          return;
+        }
         for (uint32_t o = tid; o < width; o += BLOCK) {
           uint32_t v = 0;
           for (uint32_t g = 0; g < NG; g++) v = fadd(v, epi.prod[g * width + o]);
@@ -1049,7 +1055,7 @@ struct NodesArgs {
   uint32_t low_bits, pairs_per_thread, deferred, pstride;
 };
 
-// the slot sums: lines and products in double precision (field.cuh), weighted sums in integers
+// the slot sums: lines and products in double precision (field.hpp), weighted sums in integers
 template <int D, int PASS, int SPP, class Desc>
 __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &args) {
   // magnitudes, in units of p: a table line's ends < 1, a linear form < 5 (MAXVT terms and the constant),

@@ -3,7 +3,7 @@
 
 #include <string.h>
 
-#include "blake3.cuh"
+#include "blake3.hpp"
 
 namespace exh {
 
