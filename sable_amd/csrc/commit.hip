@@ -297,7 +297,7 @@ int rs_fold_device(int D, uint64_t m, int n_domain, int level, const uint32_t *d
 // the table BaseFold opens.  One pass: 4 ncols bytes read and 4 D written per x, one x per thread (four per
 // thread measured a third slower: the 128-byte strides between lanes' stores).  The coefficients arrive as
 // kernel arguments in Montgomery form, so a reduction of four products gives their exact sum.
-constexpr int COMBINE_COLS = 32;  // columns per launch; more accumulate over launches
+constexpr int COMBINE_COLS = 32;  // columns whose coefficients travel as kernel arguments; more take the other kernel
 template <int D>
 struct CombineArgs {
   uint32_t coef_mont[COMBINE_COLS][D];
@@ -323,9 +323,68 @@ __global__ __launch_bounds__(BLOCK) void combine_columns_kernel(const uint32_t *
   store_ext<D>(out + x * D, g);  // (non-temporal stores measured a third slower)
 }
 
+// The same sum for many columns in one pass: the output stays in registers across all of them instead of being
+// read and written again every 32 columns.  The coefficients (Montgomery form, padded with zeros to a multiple of
+// eight columns) come from device memory at addresses every lane shares, eight columns' loads are in flight at
+// once, and a lane walks the columns at its own x.
+template <int D>
+__global__ __launch_bounds__(BLOCK) void combine_columns_many_kernel(const uint32_t *__restrict__ cols, uint64_t len,
+                                                                     int ncols, const uint32_t *__restrict__ coef_mont,
+                                                                     uint32_t *__restrict__ out) {
+  const uint64_t x = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (x >= len) return;
+  Ext<D> g = ext_zero<D>();
+  for (int k0 = 0; k0 < ncols; k0 += 8) {
+    uint32_t val[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {  // a column past the last is read again with a zero coefficient
+      const int k = k0 + q < ncols ? k0 + q : ncols - 1;
+      val[q] = cols[(uint64_t)k * len + x];
+    }
+#pragma unroll
+    for (int half = 0; half < 2; half++) {  // four columns per reduction: 4 p^2 < 2^64
+      const uint32_t *cf = coef_mont + (size_t)(k0 + 4 * half) * D;
+#pragma unroll
+      for (int c = 0; c < D; c++) {
+        uint64_t t = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) t += (uint64_t)cf[q * D + c] * val[4 * half + q];
+        g.c[c] = fadd(g.c[c], mont_reduce4(t));
+      }
+    }
+  }
+  store_ext<D>(out + x * D, g);
+}
+
+template <int D>
+static int combine_many_launch(const uint32_t *d_cols, int ncols, uint64_t len, const uint32_t *coef, uint32_t *d_out) {
+  Context &c = ctx();
+  const int padded = (ncols + 7) / 8 * 8;
+  std::vector<uint32_t> cm((size_t)padded * D, 0u);
+  for (size_t i = 0; i < (size_t)ncols * D; i++) cm[i] = to_mont(coef[i] % P);
+  uint32_t *d_coef = (uint32_t *)c.pool.alloc(cm.size() * 4);
+  if (!d_coef) {
+    set_error("device-out-of-memory: combine-columns coefficients");
+    return E_NOMEM;
+  }
+  struct Release {
+    Pool &pool;
+    void *ptr;
+    ~Release() { pool.release(ptr); }
+  } release{c.pool, d_coef};
+  // (from pageable memory: the call returns once the words are staged, so `cm` may go)
+  EXH_HIP(hipMemcpyAsync(d_coef, cm.data(), cm.size() * 4, hipMemcpyHostToDevice, c.stream));
+  uint32_t grid = (uint32_t)((len + BLOCK - 1) / BLOCK);
+  hipLaunchKernelGGL((combine_columns_many_kernel<D>), dim3(grid), dim3(BLOCK), 0, c.stream, d_cols, len, ncols, d_coef,
+                     d_out);
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
 template <int D>
 static int combine_launch(const uint32_t *d_cols, int ncols, uint64_t len, const uint32_t *coef, uint32_t *d_out) {
   Context &c = ctx();
+  if (ncols > COMBINE_COLS) return combine_many_launch<D>(d_cols, ncols, len, coef, d_out);
   for (int first = 0; first < ncols; first += COMBINE_COLS) {
     const int count = ncols - first < COMBINE_COLS ? ncols - first : COMBINE_COLS;
     CombineArgs<D> a;

@@ -158,10 +158,10 @@ def test_basefold_round_trip_beyond_the_oracle_sizes():
 
 
 @pytest.mark.parametrize("d,ncols,length", [(8, 1, 16), (8, 2, 1 << 12), (8, 5, 1001), (4, 3, 4096), (8, 40, 512),
-                                            (4, 33, 7)])
+                                            (4, 33, 7), (8, 128, 300), (4, 70, 1 << 10), (8, 41, 3)])
 def test_combine_columns_matches_the_oracle(d, ncols, length):
-    """combine-columns (src/pcs.lisp:434-441): lengths that are not multiples of four and more columns than one
-    launch takes included."""
+    """combine-columns (src/pcs.lisp:434-441): lengths that are not multiples of four included, and more than 32
+    columns (the one-pass kernel that takes its coefficients from device memory, eight columns at a time)."""
     rng = np.random.default_rng(ncols * 1000 + length)
     cols = rng.integers(0, P, (ncols, length), dtype=np.uint32)
     cf = rng.integers(0, P, (ncols, d), dtype=np.uint32)
