@@ -4,6 +4,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
+#include <memory>
 #include <vector>
 
 #include "hostfield.hpp"
@@ -19,6 +21,77 @@ void absorb_header(Transcript &tr, const std::string &label, int n, int degree, 
   tr.absorb((const uint8_t *)h.data(), h.size());
 }
 
+// A statement with more table monomials or accumulators than one kernel holds (the leaf-layer and zerocheck
+// statement of a domain with many lookups and constraints, src/domain.lisp:95-114) is a sum of statements that
+// fit: the monomials are dealt into parts, every part is a session of its own over the same tables, the parts'
+// rounds run in step and a round's message is the sum of theirs.  Host-driven rounds: the reference's
+// GENERIC-ROUND-SUMS role (src/sumcheck.lisp:282-317), the way that always works, not the fast one.
+static bool fits_one_kernel(const Statement &st, int points) {
+  Statement planned = st;
+  planned.plan(points);
+  StmtDesc d;
+  return planned.T() <= MAXT && make_desc(planned, &d);
+}
+
+static int sumcheck_prove_wide(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables,
+                               const int *strides, const uint32_t *eq, const uint32_t *consts, const std::string &label,
+                               const uint32_t *bw, int K, int degree, int points, uint32_t *out_chal,
+                               uint32_t *out_finals, uint32_t *const *out_folded) {
+  const int D = tr.D;
+  if (st.T() > MAXT || points > 16) {
+    set_error("invalid-parameter: statement beyond the kernels' limits");
+    return E_PARAM;
+  }
+  // the parts: as many of the expanded form's groups each as still fit
+  std::vector<Statement> parts;
+  Statement part = st;
+  part.factored_groups.clear(), part.factored_linear.clear(), part.expanded_groups.clear();
+  auto with = [&](Statement base, const Group &g) {
+    base.expanded_groups.push_back(g);
+    base.groups = base.expanded_groups, base.planned_points = -1;
+    return base;
+  };
+  for (const Group &g : st.expanded_groups) {
+    Statement grown = with(part, g);
+    if (fits_one_kernel(grown, points)) {
+      part = grown;
+      continue;
+    }
+    if (!part.expanded_groups.empty()) parts.push_back(part);
+    part.expanded_groups.clear();
+    part = with(part, g);
+    if (!fits_one_kernel(part, points)) {
+      set_error("invalid-parameter: a monomial of the statement is beyond the kernels' limits");
+      return E_PARAM;
+    }
+  }
+  if (!part.expanded_groups.empty()) parts.push_back(part);
+  std::vector<std::unique_ptr<SumcheckSession>> sessions;
+  int status;
+  for (Statement &p : parts) {
+    sessions.emplace_back(new SumcheckSession());
+    sessions.back()->private_buffers = true;
+    if ((status = sessions.back()->begin(p, D, n, d_tables, strides, eq, bw, K, consts, degree, false, false)))
+      return status;
+  }
+  absorb_header(tr, label, n, degree, bw ? K : 1);
+  std::vector<uint32_t> sums((size_t)points * D), total((size_t)points * D);
+  for (int j = 0; j < n; j++) {
+    std::fill(total.begin(), total.end(), 0u);
+    for (auto &s : sessions) {
+      if ((status = s->round_sums(sums.data()))) return status;
+      for (size_t o = 0; o < total.size(); o++) total[o] = fadd(total[o], sums[o]);
+    }
+    uint64_t dims[2] = {(uint64_t)points, (uint64_t)D};
+    if ((status = tr.send(total.data(), 2, dims, nullptr))) return status;
+    uint32_t *r = out_chal + (size_t)j * D;
+    tr.challenge(D, r);
+    for (auto &s : sessions)
+      if ((status = s->fold(r))) return status;
+  }
+  return sessions[0]->finish(out_finals, out_folded);  // every part folded the same tables
+}
+
 int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables, const int *strides,
                    const uint32_t *eq, const uint32_t *consts, const std::string &label, const uint32_t *bw, int K,
                    int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded) {
@@ -30,6 +103,9 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
   // the device drives the rounds when it can: the session then sends all its constants in one copy
   const bool device_rounds = n > 0 && n <= MAXROUNDS && points <= MAXPTS && !(host_rounds && host_rounds[0] == '1');
   int status = s.begin(st, D, n, d_tables, strides, eq, bw, K, consts, degree, false, device_rounds);
+  if (status == E_PARAM && s.beyond_limits)
+    return sumcheck_prove_wide(tr, n, st, d_tables, strides, eq, consts, label, bw, K, degree, points, out_chal,
+                               out_finals, out_folded);
   if (status) return status;
   absorb_header(tr, label, n, degree, bw ? K : 1);
   if (device_rounds && s.device_capable()) {

@@ -189,6 +189,7 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   int T = st.T();
   if (T > MAXT || points > 16 || !make_desc(st, &desc)) {
     set_error("invalid-parameter: statement beyond the kernels' limits");
+    beyond_limits = true;
     return E_PARAM;
   }
   (void)rtc_collect();
@@ -299,8 +300,8 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   if (any_base && !all_base)
     for (int t = 0; t < T; t++)
       if (strides[t] == 1) words += size * D;
-  if ((status = c.misc.reserve(words * 4))) return status;
-  uint32_t *base = (uint32_t *)c.misc.ptr;
+  if ((status = arena_misc().reserve(words * 4))) return status;
+  uint32_t *base = (uint32_t *)arena_misc().ptr;
   d_weights = base;
   d_partials = base + partial_off;
   d_sums = d_partials + partial_rows * (uint64_t)pstride;
@@ -330,7 +331,8 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   // staged in pinned memory when it fits (no wait: the region is not written again before this
   // session's next wait), else in a vector that must outlive the copy
   const size_t host_words = (size_t)(2 * n + (has_bw ? K : 0)) * D;
-  const bool staged = host_words <= PIN_BEGIN_WORDS;
+  // (a session with buffers of its own may be one of several begun back to back: each waits for its copy)
+  const bool staged = host_words <= PIN_BEGIN_WORDS && !private_buffers;
   std::vector<uint32_t> spill(staged ? 0 : host_words, 0);
   uint32_t *host = staged ? c.host_pinned + PIN_BEGIN : spill.data();
   if (staged) memset(host, 0, host_words * 4);
@@ -356,8 +358,8 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   }
   // the folded generations: the first holds half the input, the second a quarter
   if (n > 0) {
-    if ((status = c.fold_a.reserve((size_t)T * (size / 2) * D * 4))) return status;
-    if (n > 1 && (status = c.fold_b.reserve((size_t)T * (size / 4) * D * 4))) return status;
+    if ((status = arena_a().reserve((size_t)T * (size / 2) * D * 4))) return status;
+    if (n > 1 && (status = arena_b().reserve((size_t)T * (size / 4) * D * 4))) return status;
   }
   EXH_HIP(hipGetLastError());
   return OK;
@@ -589,8 +591,18 @@ static hf::E weight_sum(const SumcheckSession &s, int j) {
   return wsum;
 }
 
+Arena &SumcheckSession::arena_a() { return private_buffers ? own_a : ctx().fold_a; }
+Arena &SumcheckSession::arena_b() { return private_buffers ? own_b : ctx().fold_b; }
+Arena &SumcheckSession::arena_misc() { return private_buffers ? own_misc : ctx().misc; }
+SumcheckSession::~SumcheckSession() {
+  if (private_buffers) {  // everything queued on them has to have run before they go back to the driver
+    if (own_a.ptr || own_b.ptr || own_misc.ptr) (void)hipStreamSynchronize(ctx().stream);
+    own_a.release(), own_b.release(), own_misc.release();
+  }
+}
+
 int SumcheckSession::owns_arenas() const {
-  if (epoch == ctx().session_epoch) return OK;
+  if (private_buffers || epoch == ctx().session_epoch) return OK;
   set_error("invalid-parameter: another sumcheck session was begun since; one session is open at a time");
   return E_PARAM;
 }
@@ -614,7 +626,7 @@ int SumcheckSession::round_sums(uint32_t *out) {
   uint64_t n_pairs;
   if (pending_fold) {  // fused: fold round j-1's variable, then sum round j
     uint64_t out_size = size / 2;
-    Arena &dst = (generation % 2 == 0) ? c.fold_a : c.fold_b;
+    Arena &dst = (generation % 2 == 0) ? arena_a() : arena_b();
     out_buf.assign(T, nullptr);
     for (int t = 0; t < T; t++) out_buf[t] = (uint32_t *)dst.ptr + (uint64_t)t * out_size * D;
     n_pairs = out_size / 2;
@@ -702,7 +714,7 @@ int SumcheckSession::flush() {
   if (!pending_fold) return OK;
   int T = st.T();
   uint64_t out_size = size / 2;
-  Arena &dst = (generation % 2 == 0) ? c.fold_a : c.fold_b;
+  Arena &dst = (generation % 2 == 0) ? arena_a() : arena_b();
   RoundArgs<4> a4;
   RoundArgs<8> a8;
   memset(&a4, 0, sizeof(a4));
@@ -855,7 +867,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     if (folds_due == 2) {  // round 2 after the base-field sweep: both folds at once, then the sums
       round = j;
       uint64_t out_size = size / 4;
-      Arena &dst = ((generation + 1) % 2 == 0) ? c.fold_a : c.fold_b;
+      Arena &dst = ((generation + 1) % 2 == 0) ? arena_a() : arena_b();
       out_buf.assign(T, nullptr);
       for (int t = 0; t < T; t++) out_buf[t] = (uint32_t *)dst.ptr + (uint64_t)t * out_size * D;
       status = D == 4 ? launch_round<4>(*this, true, true, out_buf, n_pairs, j, true)
@@ -925,7 +937,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
                       : launch_round<8>(*this, false, true, out_buf, n_pairs, j);
     } else {
       uint64_t out_size = size / 2;
-      Arena &dst = (generation % 2 == 0) ? c.fold_a : c.fold_b;
+      Arena &dst = (generation % 2 == 0) ? arena_a() : arena_b();
       out_buf.assign(T, nullptr);
       for (int t = 0; t < T; t++) out_buf[t] = (uint32_t *)dst.ptr + (uint64_t)t * out_size * D;
       status = D == 4 ? launch_round<4>(*this, true, true, out_buf, n_pairs, j)
@@ -1016,7 +1028,7 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
   int folds = (first_fold ? 1 : 0) + rounds;
   uint64_t final_size = size >> folds;
   int last_gen = generation + folds - 1;
-  Arena &dst = (last_gen % 2 == 0) ? c.fold_a : c.fold_b;
+  Arena &dst = (last_gen % 2 == 0) ? arena_a() : arena_b();
   int status = dst.reserve((size_t)T * final_size * D * 4);
   if (status) return status;
   const uint64_t slice_entries = (first_fold ? size / 2 : size) / grid;

@@ -8,6 +8,7 @@
 #include <functional>
 #include <vector>
 
+#include "context.hpp"
 #include "forms.hpp"
 #include "sumcheck_kernels.hpp"
 
@@ -70,6 +71,16 @@ struct SumcheckSession {
             bool claim_mode = false, bool defer_setup = false);
   // With defer_setup the eq point and block weights stay staged on the host and the weight-table
   // kernels are not launched: run_device sends them with its own constants in one copy and launches then.
+  // Set before begin: the session keeps its folded generations and weights in buffers of its own instead of the
+  // context's, so that several sessions can be open side by side (the parts of a statement too wide for one
+  // kernel, proved in step).  Such a session runs host-driven rounds.
+  bool private_buffers = false;
+  bool beyond_limits = false;  // begin refused the statement for its size alone: its parts may still fit
+  Arena own_a, own_b, own_misc;
+  Arena &arena_a();
+  Arena &arena_b();
+  Arena &arena_misc();
+  ~SumcheckSession();
   uint64_t epoch = 0;  // Context::session_epoch at begin
   // OK while this is the latest session begun (its arenas have not been handed to another one)
   int owns_arenas() const;

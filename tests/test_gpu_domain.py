@@ -9,7 +9,7 @@ import sable_amd as sa
 from oracle import binding as orc
 from oracle import domain as od
 from sable_amd import domain as sd
-from test_oracle_domain import lookup_challenges, toy_domain
+from test_oracle_domain import CASES as ORACLE_CASES, lookup_challenges, toy_domain
 
 pytestmark = pytest.mark.gpu
 P = orc.P
@@ -151,11 +151,33 @@ def test_rejects(merge):
             sd.verify_domain(sa.Transcript("dom-test", d, proof=orc.encode_messages(forged)), mine, z, betas)
 
 
-def test_a_statement_beyond_the_kernels_limits_is_refused():
-    """The reference's toy domain expands to 41 table monomials; the round kernels hold 16 (and 36 accumulators,
-    which the products domain with merged blocks exceeds too): the prover refuses it (invalid-parameter) instead of
-    proving something else."""
-    theirs = toy_domain(n=3, k=3)
-    z, betas = lookup_challenges(4, 1)
-    with pytest.raises(sa.InvalidParameter):
-        sd.prove_domain(sa.Transcript("dom-test", 4), device_toy(theirs), z, betas)
+@pytest.mark.parametrize("d", [4, 8])
+@pytest.mark.parametrize("case", ORACLE_CASES, ids=lambda c: "-".join("%s%s" % kv for kv in c.items()))
+def test_the_toy_domain_in_parts(case, d):
+    """The reference's toy domain (tests/tests.lisp:487-512: every kind of column, three lookups, three
+    constraints) in every shape its round-trip test takes.  Its statement expands to 41 table monomials, more than
+    one kernel holds: the prover deals them into parts proved in step, and the bytes are the oracle's."""
+    theirs = toy_domain(seed=d + case["n"] + case["k"], **case)
+    mine = device_toy(theirs)
+    z, betas = lookup_challenges(d, case["n"])
+    otr = orc.Transcript("dom-test", d)
+    want_claims = od.prove_domain(otr, theirs, z, betas)
+    tr = sa.Transcript("dom-test", d)
+    claims = sd.prove_domain(tr, mine, z, betas)
+    assert tr.proof() == otr.proof() and same_claims(claims, want_claims)
+    vtr = sa.Transcript("dom-test", d, proof=tr.proof())
+    got, _ = sd.verify_domain(vtr, mine, z, betas)
+    assert vtr.finished() and same_claims(got, claims)
+
+
+def test_a_wide_statement_at_size():
+    """The toy domain at n = 14 with three blocks (tables of 3 * 2^13 entries, 41 monomials in three parts)."""
+    d = 4
+    theirs = toy_domain(n=14, k=3, seed=77)
+    mine = device_toy(theirs)
+    z, betas = lookup_challenges(d, 77)
+    otr = orc.Transcript("dom-test", d)
+    od.prove_domain(otr, theirs, z, betas)
+    tr = sa.Transcript("dom-test", d)
+    sd.prove_domain(tr, mine, z, betas)
+    assert tr.proof() == otr.proof()
