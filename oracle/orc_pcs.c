@@ -1,8 +1,9 @@
 /* orc_pcs.c -- the commitment's data-parallel part: leaf digests, Merkle trees with caps, column
  * commitment, combine-columns and the BaseFold loop, restated from src/pcs.lisp:37-101, 271-304, 434-441, 473-483,
  * 569-657
- * (test oracle; see orc.h).  The multi-unit bookkeeping around them (units, merge sets, segments,
- * point reductions, query verification) is not restated: BaseFold runs here on one class. */
+ * (test oracle; see orc.h).  BaseFold runs here on one class; the opening over several size classes, query
+ * verification and trees with injections are in orc_open.c.  The multi-unit bookkeeping around them (units,
+ * merge sets, segments, point reductions) is not restated. */
 #include "orc.h"
 #include <stdlib.h>
 #include <string.h>

@@ -57,6 +57,141 @@ __global__ __launch_bounds__(BLOCK) void halves_kernel(const uint32_t *v, uint32
   store_ext<D>(upper + o * D, load_ext<D>(v + (b * 2 * size + size + x) * D));
 }
 
+
+// ------------------------------------------------------------------ the layers chained on the device
+// With one block, the layers' sumchecks run back to back without the host: between two of them one small launch
+// (one wavefront) does what PROVE-UPPER does on the host there (src/gkr.lisp:248-271) -- it sends the finished
+// layer's finals and draws the fresh point (SEND-FINALS), forms the next layer's point, draws the layer's
+// challenges (LAYER-CHALLENGES), absorbs the next sumcheck's header and writes that sumcheck's constants where its
+// launches expect them: the eq point's factors, the message map, the head of the control block with the
+// transcript's state.  Everything the host needs afterwards goes to a log it reads once at the end.
+struct GkrChainState {
+  DevB3S tr;                       // the transcript between launches
+  uint32_t point[MAXROUNDS + 1][8];  // the next layer's eq point (canonical)
+};
+
+constexpr int GLUE_MAXCONST = 8;  // constants of a layer statement the launch can form: a_l and a_l lambda, l < 4
+
+template <int D>
+struct GlueArgs {
+  GkrChainState *chain;
+  int close_kind;  // 0: nothing to close, 1: send the roots, 2: a layer's finals from its control block, 3: from tables
+  const Ctrl *prev_ctrl;
+  int prev_rounds, prev_points;
+  const uint32_t *tabs[MAXT];  // kind 1: the root of p and of q per lookup; kind 3: the layer's tables (one entry each)
+  int NT, L;
+  uint32_t *log;  // kind 1: the roots (2 L D words); kinds 2, 3: the layer's messages, challenges, finals, fresh point
+  int open;       // open the next layer's sumcheck
+  int n;          // its rounds
+  uint32_t header[16];  // its header's bytes (src/sumcheck.lisp:24-27), as little-endian words
+  int header_len;
+  uint32_t *factors, *mtilde, *c0;
+  Ctrl *ctrl;
+  int points, nacc, c0_words;
+  uint32_t lagfix[MAXPTS * MAXACC];
+  uint8_t acc_const[MAXACC];  // the constant (a_l: 2 l, a_l lambda: 2 l + 1) that is the accumulator's group coefficient
+};
+
+// absorb(bytes) for LEN bytes held as little-endian words in LDS: the length as u64 LE, then the bytes
+__device__ inline void dev_absorb_bytes(RunB3S &s, const uint32_t *words, uint32_t len) {
+  const uint32_t lane = threadIdx.x & 63, total = 8 + len;
+  for (uint32_t base = 0; base < total; base += 64) {
+    const uint32_t g = base + lane;
+    uint32_t word = g < 4 ? len : (g < 8 || g >= total) ? 0 : words[(g - 8) >> 2];
+    rb3s_append_bytes(s, (word >> (8 * (g & 3))) & 0xff, total - base < 64 ? total - base : 64);
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(64) void gkr_glue_kernel(GlueArgs<D> a) {
+  __shared__ uint32_t ring[RING_WORDS];
+  __shared__ uint32_t buf[64];
+  __shared__ uint32_t chal[16];
+  __shared__ uint32_t consts[GLUE_MAXCONST][8];
+  __shared__ uint32_t point[MAXROUNDS + 1][8];
+  const uint32_t lane = threadIdx.x;
+  RunB3S tr;
+  rb3s_load(tr, ring, a.close_kind == 2 ? &a.prev_ctrl->tr : &a.chain->tr);
+  __builtin_amdgcn_wave_barrier();
+  if (a.close_kind == 1) {  // the roots: one message (2, D) per lookup
+    for (int l = 0; l < a.L; l++) {
+      if (lane < 2 * D) buf[lane] = a.tabs[2 * l + lane / D][lane % D];
+      __builtin_amdgcn_wave_barrier();
+      dev_absorb_words(tr, buf, 2 * D);
+      if (lane < 2 * D) a.log[l * 2 * D + lane] = buf[lane];
+      __builtin_amdgcn_wave_barrier();
+    }
+  } else if (a.close_kind != 0) {
+    const int R = a.prev_rounds, mw = a.prev_points * D;
+    uint32_t *log_msg = a.log, *log_chal = log_msg + R * mw, *log_fin = log_chal + R * D, *log_tt = log_fin + a.NT * D;
+    if (a.close_kind == 2) {
+      for (int u = lane; u < R * mw; u += 64) log_msg[u] = a.prev_ctrl->msg[u / mw][u % mw];
+      for (int u = lane; u < R * D; u += 64) {
+        const uint32_t v = a.prev_ctrl->chal[u / D][u % D];
+        log_chal[u] = v;
+        point[u / D][u % D] = v;  // the layer's challenges open the next layer's point
+      }
+    }
+    for (int t = 0; t < a.NT; t++) {  // SEND-FINALS: one message (1, D) per table, then the fresh point
+      if (lane < D) buf[lane] = a.close_kind == 2 ? a.prev_ctrl->finals[t * D + lane] : a.tabs[t][lane];
+      __builtin_amdgcn_wave_barrier();
+      dev_absorb_words(tr, buf, D);
+      if (lane < D) log_fin[t * D + lane] = buf[lane];
+      __builtin_amdgcn_wave_barrier();
+    }
+    dev_challenge(tr, D, chal);
+    __builtin_amdgcn_wave_barrier();
+    if (lane < D) {
+      log_tt[lane] = chal[lane];
+      point[R][lane] = chal[lane];
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int u = lane; u < (R + 1) * D; u += 64) a.chain->point[u / D][u % D] = point[u / D][u % D];
+  }
+  if (a.open) {
+    if (a.close_kind == 0 || a.close_kind == 1)
+      for (int u = lane; u < a.n * D; u += 64) point[u / D][u % D] = a.chain->point[u / D][u % D];
+    // LAYER-CHALLENGES: a_l from one stream of L D base challenges, then lambda
+    dev_challenge(tr, a.L * D, chal);
+    __builtin_amdgcn_wave_barrier();
+    if (lane < (uint32_t)(a.L * D)) consts[2 * (lane / D)][lane % D] = chal[lane];
+    __builtin_amdgcn_wave_barrier();
+    dev_challenge(tr, D, chal);
+    __builtin_amdgcn_wave_barrier();
+    if (lane < (uint32_t)a.L) {  // a_l lambda, exact: one factor carries R
+      Ext<D> x, y;
+#pragma unroll
+      for (int c = 0; c < D; c++) x.c[c] = consts[2 * lane][c], y.c[c] = to_mont(chal[c]);
+      const Ext<D> z = ext_mul_mont<D>(x, y);
+#pragma unroll
+      for (int c = 0; c < D; c++) consts[2 * lane + 1][c] = z.c[c];
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (lane < 16) buf[lane] = a.header[lane];
+    __builtin_amdgcn_wave_barrier();
+    dev_absorb_bytes(tr, buf, (uint32_t)a.header_len);
+    if (a.n > 0) {
+      // the eq point's factors r_v R and (1 - r_v) R, variable by variable
+      for (int u = lane; u < a.n * D; u += 64) {
+        const uint32_t v = u / D, k = u % D, r = point[v][k];
+        a.factors[(2 * v) * D + k] = to_mont(r);
+        a.factors[(2 * v + 1) * D + k] = to_mont(fsub(k == 0 ? 1u : 0u, r));
+      }
+      // the message map: the accumulator's group coefficient times its scalar, in Montgomery form
+      for (int u = lane; u < a.points * a.nacc * D; u += 64) {
+        const int e = u / D, c = u % D;
+        a.mtilde[u] = to_mont(fmul(consts[a.acc_const[e % a.nacc]][c], a.lagfix[e]));
+      }
+      for (int u = lane; u < a.c0_words; u += 64) a.c0[u] = 0;
+      uint32_t *head = reinterpret_cast<uint32_t *>(a.ctrl);
+      for (uint32_t u = sizeof(DevB3S) / 4 + lane; u < offsetof(Ctrl, msg) / 4; u += 64) head[u] = 0;
+      __builtin_amdgcn_wave_barrier();
+      rb3s_store(tr, &a.ctrl->tr);
+    }
+  }
+  rb3s_store(tr, &a.chain->tr);
+}
+
 namespace {
 
 int block_bits(int k) {  // src/gkr.lisp:23-25
@@ -163,6 +298,163 @@ struct DeviceBuffers {  // frees what it allocated when the proof ends
   }
 };
 
+
+// PROVE-UPPER's in-block layers with one block, chained on the device (see gkr_glue_kernel): every launch of every
+// layer's sumcheck is enqueued at once, the host waits once and reads the log.
+template <int D>
+static int launch_glue(const GlueArgs<D> &a) {
+  Context &c = ctx();
+  c.prof_begin("gkr_glue", a.n, 0);
+  hipLaunchKernelGGL(gkr_glue_kernel<D>, dim3(1), dim3(64), 0, c.stream, a);
+  c.prof_end();
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
+template <int D>
+static int prove_upper_chained(Transcript &tr, int n, int L, const std::vector<std::vector<const uint32_t *>> &layers,
+                               const std::string &label, uint32_t *out_ri, uint32_t *out_cp, uint32_t *out_cq) {
+  Context &c = ctx();
+  const int NT = 4 * L;
+  Statement st = layer_statement(L, false);
+  // the log: the roots, then per layer its round messages, challenges, finals and fresh point
+  std::vector<size_t> log_off(n - 1);
+  size_t words = (size_t)2 * L * D;
+  for (int layer = 0; layer < n - 1; layer++) {
+    const int points = layer > 0 ? 2 : 1;
+    log_off[layer] = words;
+    words += (size_t)layer * points * D + (size_t)layer * D + (size_t)NT * D + D;
+  }
+  DeviceBuffers bufs;
+  GkrChainState *chain = reinterpret_cast<GkrChainState *>(bufs.alloc((sizeof(GkrChainState) + 3) / 4));
+  uint32_t *d_log = bufs.alloc(words);
+  if (!chain || !d_log) {
+    set_error("device-out-of-memory: the GKR chain's log");
+    return E_NOMEM;
+  }
+  const DevB3S first = device_state(tr);
+  EXH_HIP(hipMemcpyAsync(&chain->tr, &first, sizeof(first), hipMemcpyHostToDevice, c.stream));
+  const std::vector<int> strides(NT, D);
+  const std::vector<uint32_t> no_point((size_t)n * D, 0), no_consts((size_t)2 * L * D, 0);
+  auto layer_tables = [&](int layer) {  // with one block the halves are views (LAYER-TABLES, src/gkr.lisp:199-206)
+    std::vector<const uint32_t *> tabs(NT);
+    const uint64_t size = (uint64_t)1 << layer;
+    for (int l = 0; l < L; l++)
+      for (int w = 0; w < 2; w++) {
+        const uint32_t *v = layers[layer + 1][2 * l + w];
+        tabs[4 * l + 2 * w] = v;
+        tabs[4 * l + 2 * w + 1] = v + size * D;
+      }
+    return tabs;
+  };
+  int status;
+  {  // the largest layer first, for its buffers alone: the arenas then never grow (and never wait) mid-chain
+    SumcheckSession widest;
+    std::vector<const uint32_t *> tabs = layer_tables(n - 2);
+    if ((status = widest.begin(st, D, n - 2, tabs.data(), strides.data(), no_point.data(), nullptr, 1, no_consts.data(),
+                               n - 2 > 0 ? 2 : 0, false, true)))
+      return status;
+  }
+  const Ctrl *prev_ctrl = nullptr;
+  std::vector<const uint32_t *> prev_tabs;
+  const DevB3S unused_state = first;
+  for (int layer = 0; layer <= n - 1; layer++) {  // launch `layer` closes layer - 1 and opens `layer`; the last only closes
+    GlueArgs<D> a;
+    memset(&a, 0, sizeof(a));
+    a.chain = chain, a.L = L, a.NT = NT;
+    if (layer == 0) {
+      a.close_kind = 1, a.log = d_log;
+      for (int i = 0; i < 2 * L; i++) a.tabs[i] = layers[0][i];
+    } else if (layer == 1) {  // layer 0 has no rounds: its finals are its tables' single entries
+      a.close_kind = 3, a.prev_rounds = 0, a.prev_points = 1, a.log = d_log + log_off[0];
+      for (int t = 0; t < NT; t++) a.tabs[t] = prev_tabs[t];
+    } else {
+      a.close_kind = 2, a.prev_ctrl = prev_ctrl, a.prev_rounds = layer - 1, a.prev_points = 2;
+      a.log = d_log + log_off[layer - 1];
+    }
+    if (layer == n - 1) {
+      if ((status = launch_glue<D>(a))) return status;
+      break;
+    }
+    const int degree = layer > 0 ? 2 : 0;
+    const std::string header = header_bytes(label, layer, degree, 1);
+    if (header.size() > 64) {
+      set_error("invalid-parameter: label too long for the chained layers");
+      return E_PARAM;
+    }
+    a.open = 1, a.n = layer, a.header_len = (int)header.size();
+    for (size_t i = 0; i < header.size(); i++) a.header[i / 4] |= (uint32_t)(uint8_t)header[i] << (8 * (i % 4));
+    std::vector<const uint32_t *> tabs = layer_tables(layer);
+    if (layer == 0) {
+      if ((status = launch_glue<D>(a))) return status;
+    } else {
+      SumcheckSession s;
+      if ((status = s.begin(st, D, layer, tabs.data(), strides.data(), no_point.data(), nullptr, 1, no_consts.data(),
+                            degree, false, true)))
+        return status;
+      std::vector<uint32_t> lagfix;
+      std::vector<int> acc_group;
+      s.message_map_scalars(&lagfix, &acc_group);
+      a.points = s.points, a.nacc = std::max(s.st.nacc, 1), a.c0_words = layer * s.points * D;
+      if ((int)lagfix.size() > MAXPTS * MAXACC || !s.setup_deferred) {
+        set_error("invalid-parameter: layer statement beyond the chained layers' limits");
+        return E_PARAM;
+      }
+      memcpy(a.lagfix, lagfix.data(), lagfix.size() * 4);
+      for (int e = 0; e < a.nacc; e++) {
+        const Group *g = acc_group[e] >= 0 ? &s.st.groups[acc_group[e]] : nullptr;
+        if (!g || g->parts.size() != 1 || g->parts[0].coeff != 1 || g->parts[0].consts.size() != 1 ||
+            g->parts[0].consts[0] >= GLUE_MAXCONST) {
+          set_error("invalid-parameter: layer statement beyond the chained layers' limits");
+          return E_PARAM;
+        }
+        a.acc_const[e] = (uint8_t)g->parts[0].consts[0];
+      }
+      a.factors = s.d_weights, a.mtilde = s.d_mtilde, a.c0 = s.d_c0, a.ctrl = s.d_ctrl;
+      s.chain_hook = [&a]() { return launch_glue<D>(a); };
+      if ((status = s.run_device(unused_state, nullptr, nullptr, nullptr))) return status;
+      prev_ctrl = s.d_ctrl;
+    }
+    prev_tabs = tabs;
+  }
+  // ---- one wait, then the log
+  std::vector<uint32_t> log(words);
+  DevB3S last;
+  EXH_HIP(hipMemcpyAsync(log.data(), d_log, words * 4, hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipMemcpyAsync(&last, &chain->tr, sizeof(last), hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipStreamSynchronize(c.stream));
+  // the messages as they were sent, recorded without hashing them again; the transcript takes the device's state
+  uint64_t dims[2] = {2, (uint64_t)D};
+  for (int l = 0; l < L; l++)
+    if ((status = tr.send(&log[(size_t)l * 2 * D], 2, dims, nullptr, false))) return status;
+  const uint32_t *fin = nullptr, *tt = nullptr, *rho = nullptr;
+  for (int layer = 0; layer < n - 1; layer++) {
+    const int points = layer > 0 ? 2 : 1;
+    const uint32_t *msg = &log[log_off[layer]];
+    rho = msg + (size_t)layer * points * D;
+    fin = rho + (size_t)layer * D;
+    tt = fin + (size_t)NT * D;
+    dims[0] = (uint64_t)points;
+    for (int j = 0; j < layer; j++)
+      if ((status = tr.send(msg + (size_t)j * points * D, 2, dims, nullptr, false))) return status;
+    dims[0] = 1;
+    for (int t = 0; t < NT; t++)
+      if ((status = tr.send(fin + (size_t)t * D, 2, dims, nullptr, false))) return status;
+  }
+  if ((status = adopt_device_state(tr, last))) return status;
+  if (out_ri) {
+    memcpy(out_ri, rho, (size_t)(n - 2) * D * 4);
+    memcpy(out_ri + (size_t)(n - 2) * D, tt, (size_t)D * 4);
+  }
+  std::vector<hf::E> cp(L), cq(L);
+  next_claims(D, L, fin, hf::from(tt, D), cp, cq);
+  for (int l = 0; l < L; l++) {
+    if (out_cp) memcpy(out_cp + (size_t)l * D, cp[l].data(), 4 * D);
+    if (out_cq) memcpy(out_cq + (size_t)l * D, cq[l].data(), 4 * D);
+  }
+  return OK;
+}
+
 }  // namespace
 
 int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *leaves, const std::string &label,
@@ -192,6 +484,17 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
       layers[m][2 * l] = pp;
       layers[m][2 * l + 1] = qq;
     }
+  {  // one block: the layers chained on the device, one wait for the whole proof
+    const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS"), *no_chain = getenv("EXACTA_HIP_NO_GKR_CHAIN");
+    const bool off = (host_rounds && host_rounds[0] == '1') || (no_chain && no_chain[0] == '1');
+    if (K == 1 && n >= 2 && n - 2 <= MAXROUNDS && L * D <= 8 && 2 * L <= GLUE_MAXCONST && !off) {
+      status = D == 4 ? prove_upper_chained<4>(tr, n, L, layers, label, out_ri, out_cp, out_cq)
+                      : prove_upper_chained<8>(tr, n, L, layers, label, out_ri, out_cp, out_cq);
+      if (status) return status;
+      EXH_HIP(hipStreamSynchronize(c.stream));
+      return OK;
+    }
+  }
   // the per-block roots, and the top tree over the block index on the host (2^lk entries)
   std::vector<std::vector<std::vector<uint32_t>>> top(lk + 1, std::vector<std::vector<uint32_t>>(2 * L));
   EXH_HIP(hipStreamSynchronize(c.stream));

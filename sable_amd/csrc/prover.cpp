@@ -13,12 +13,38 @@
 namespace exh {
 
 // label | n u16 | degree u16 | blocks u32, little-endian (src/sumcheck.lisp:24-27)
-void absorb_header(Transcript &tr, const std::string &label, int n, int degree, int blocks) {
+std::string header_bytes(const std::string &label, int n, int degree, int blocks) {
   std::string h = label + "|";
   h.push_back((char)(n & 0xff)), h.push_back((char)((n >> 8) & 0xff));
   h.push_back((char)(degree & 0xff)), h.push_back((char)((degree >> 8) & 0xff));
   for (int i = 0; i < 4; i++) h.push_back((char)(((uint32_t)blocks >> (8 * i)) & 0xff));
+  return h;
+}
+void absorb_header(Transcript &tr, const std::string &label, int n, int degree, int blocks) {
+  std::string h = header_bytes(label, n, degree, blocks);
   tr.absorb((const uint8_t *)h.data(), h.size());
+}
+
+DevB3S device_state(const Transcript &tr) {
+  DevB3S state;
+  memcpy(state.cv, tr.state.cv, 32);
+  for (int i = 0; i < 16; i++)
+    state.block[i] = (uint32_t)tr.state.block[4 * i] | (uint32_t)tr.state.block[4 * i + 1] << 8 |
+                     (uint32_t)tr.state.block[4 * i + 2] << 16 | (uint32_t)tr.state.block[4 * i + 3] << 24;
+  state.used = tr.state.used;
+  state.counter_lo = (uint32_t)tr.state.counter, state.counter_hi = (uint32_t)(tr.state.counter >> 32);
+  return state;
+}
+int adopt_device_state(Transcript &tr, const DevB3S &state) {
+  if (state.used > 64) {
+    set_error("device-error: the device transcript's final state is malformed");
+    return E_DEVICE;
+  }
+  memcpy(tr.state.cv, state.cv, 32);
+  for (int i = 0; i < 64; i++) tr.state.block[i] = (uint8_t)(state.block[i / 4] >> (8 * (i % 4)));
+  tr.state.used = state.used;
+  tr.state.counter = ((uint64_t)state.counter_hi << 32) | state.counter_lo;
+  return OK;
 }
 
 // A statement with more table monomials or accumulators than one kernel holds (the leaf-layer and zerocheck
@@ -113,13 +139,7 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
     // as they were sent and the hash state the device's transcript ended in; with EXACTA_HIP_REPLAY=1 it absorbs
     // the messages itself instead and checks that it draws the same challenges (a diagnostic: the two
     // transcripts are the same function, and the tests hold the device's to the oracle's bytes)
-    DevB3S state, final_state;
-    memcpy(state.cv, tr.state.cv, 32);
-    for (int i = 0; i < 16; i++)
-      state.block[i] = (uint32_t)tr.state.block[4 * i] | (uint32_t)tr.state.block[4 * i + 1] << 8 |
-                       (uint32_t)tr.state.block[4 * i + 2] << 16 | (uint32_t)tr.state.block[4 * i + 3] << 24;
-    state.used = tr.state.used;
-    state.counter_lo = (uint32_t)tr.state.counter, state.counter_hi = (uint32_t)(tr.state.counter >> 32);
+    DevB3S state = device_state(tr), final_state;
     std::vector<uint32_t> messages((size_t)n * points * D), challenges((size_t)n * D);
     if ((status = s.run_device(state, messages.data(), challenges.data(), &final_state))) return status;
     const char *replay = getenv("EXACTA_HIP_REPLAY");
@@ -139,16 +159,7 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
         memcpy(r, &challenges[(size_t)j * D], 4 * D);
       }
     }
-    if (!replaying) {
-      if (final_state.used > 64) {
-        set_error("device-error: the device transcript's final state is malformed");
-        return E_DEVICE;
-      }
-      memcpy(tr.state.cv, final_state.cv, 32);
-      for (int i = 0; i < 64; i++) tr.state.block[i] = (uint8_t)(final_state.block[i / 4] >> (8 * (i % 4)));
-      tr.state.used = final_state.used;
-      tr.state.counter = ((uint64_t)final_state.counter_hi << 32) | final_state.counter_lo;
-    }
+    if (!replaying && (status = adopt_device_state(tr, final_state))) return status;
     return s.finish(out_finals, out_folded);
   }
   uint32_t sums[16 * 8];

@@ -20,5 +20,10 @@ int sumcheck_verify(Transcript &tr, int n, const Statement &st, const uint32_t *
                     uint32_t *out_reduced);
 int check_final(const Statement &st, int D, const uint32_t *reduced, const uint32_t *finals, const uint32_t *consts);
 void absorb_header(Transcript &tr, const std::string &label, int n, int degree, int blocks);
+// the header's bytes: label | n u16 | degree u16 | blocks u32, little-endian (src/sumcheck.lisp:24-27)
+std::string header_bytes(const std::string &label, int n, int degree, int blocks);
+// the host transcript's hash state as the device transcript keeps it, and back
+DevB3S device_state(const Transcript &tr);
+int adopt_device_state(Transcript &tr, const DevB3S &state);
 
 }  // namespace exh

@@ -780,6 +780,36 @@ static uint64_t tail_pairs(int T, int D) {
   return p;
 }
 
+// the Lagrange basis of the group's node e over its nodes at wire point k (0, 2, 3, ...), times the power of R the
+// group's sums carry (R^-degree)
+static uint32_t map_scalar(const Group &grp, size_t e, int k, int points) {
+  const uint32_t fix = fpow(R1, grp.tabs.size());
+  if ((int)grp.tabs.size() >= points) return (int)e == k ? fix : 0u;  // evaluated at the wire points themselves
+  const int wire = k == 0 ? 0 : k + 1;
+  uint32_t num = 1, den = 1;
+  for (size_t o = 0; o < grp.evalx.size(); o++) {
+    if (o == e) continue;
+    int64_t a = wire - grp.evalx[o], b = grp.evalx[e] - grp.evalx[o];
+    num = fmul(num, (uint32_t)(((a % (int64_t)P) + P) % P));
+    den = fmul(den, (uint32_t)(((b % (int64_t)P) + P) % P));
+  }
+  return fmul(fmul(num, finv(den)), fix);
+}
+
+void SumcheckSession::message_map_scalars(std::vector<uint32_t> *lagfix, std::vector<int> *acc_group) const {
+  const int nacc = std::max(st.nacc, 1);
+  lagfix->assign((size_t)points * nacc, 0u);
+  acc_group->assign((size_t)nacc, -1);
+  for (size_t g = 0; g < st.groups.size(); g++) {
+    const Group &grp = st.groups[g];
+    if (grp.tabs.empty()) continue;
+    for (size_t e = 0; e < grp.evalx.size(); e++) {
+      (*acc_group)[grp.acc_base + e] = (int)g;
+      for (int k = 0; k < points; k++) (*lagfix)[(size_t)k * nacc + grp.acc_base + e] = map_scalar(grp, e, k, points);
+    }
+  }
+}
+
 bool SumcheckSession::device_capable() const {
   if (points > MAXPTS || n > MAXROUNDS) return false;
   // the session's staged eq point and block weights, then the loop's message map, constant terms and the head
@@ -809,8 +839,6 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   uint32_t *mt = up, *c0 = mt + mt_words;
   Ctrl *hc = reinterpret_cast<Ctrl *>(c0 + c0_words);  // only its head is staged
   hc->tr = state;
-  std::vector<int> wire(points);
-  for (int k = 0; k < points; k++) wire[k] = k == 0 ? 0 : k + 1;
   for (size_t g = 0; g < st.groups.size(); g++) {
     const Group &grp = st.groups[g];
     hf::E coef(group_coef.begin() + g * D, group_coef.begin() + (g + 1) * D);
@@ -823,30 +851,24 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       }
       continue;
     }
-    uint32_t fix = fpow(R1, grp.tabs.size());  // the sums carry R^-degree
-    bool direct = (int)grp.tabs.size() >= points;
     for (size_t e = 0; e < grp.evalx.size(); e++) {
       for (int k = 0; k < points; k++) {
-        uint32_t lag;  // the Lagrange basis of node e over the group's nodes, at wire point k
-        if (direct)
-          lag = (int)e == k ? 1u : 0u;
-        else {
-          uint32_t num = 1, den = 1;
-          for (size_t o = 0; o < grp.evalx.size(); o++) {
-            if (o == e) continue;
-            int64_t a = wire[k] - grp.evalx[o], b = grp.evalx[e] - grp.evalx[o];
-            num = fmul(num, (uint32_t)(((a % (int64_t)P) + P) % P));
-            den = fmul(den, (uint32_t)(((b % (int64_t)P) + P) % P));
-          }
-          lag = fmul(num, finv(den));
-        }
-        hf::E m = hf::scale(coef, fmul(lag, fix));
+        hf::E m = hf::scale(coef, map_scalar(grp, e, k, points));
         uint32_t *dst = mt + ((size_t)k * nacc + grp.acc_base + e) * D;
         for (int cc = 0; cc < D; cc++) dst[cc] = to_mont(m[cc]);
       }
     }
   }
-  if (setup_deferred) {  // one copy for the session's constants and the loop's, then the weight tables
+  if (chain_hook) {  // the chain's launch writes what the copy below would bring
+    if (!setup_deferred) {
+      set_error("invalid-parameter: a chained session defers its set-up");
+      return E_PARAM;
+    }
+    int st_hook = chain_hook();
+    if (st_hook) return st_hook;
+    setup_deferred = false;
+    if ((st_hook = launch_setup())) return st_hook;
+  } else if (setup_deferred) {  // one copy for the session's constants and the loop's, then the weight tables
     EXH_HIP(hipMemcpyAsync(d_weights, c.host_pinned + PIN_BEGIN, (setup_words + up_words) * 4, hipMemcpyHostToDevice,
                            c.stream));
     setup_deferred = false;
@@ -956,7 +978,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
     // when a single entry per table is left at the end (the finals travel in the control block), the launch
     // itself delivers the control block to pinned host memory
-    const bool deliver = !c.profiling && (size >> ((folds_due > 0 ? 1 : 0) + (n - j))) == 1;
+    const bool deliver = !c.profiling && !chain_hook && (size >> ((folds_due > 0 ? 1 : 0) + (n - j))) == 1;
     if (deliver) {
       if (++c.log_seq == 0) ++c.log_seq;  // 0 is what the flag is reset to
       host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = c.log_seq;
@@ -971,6 +993,14 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   }
   device_loop = false;
   if (status) return status;
+  if (chain_hook) {  // nothing comes back here: the chain reads the control block on the device
+    if (!tail_done || size != 1) {
+      set_error("device-error: a chained sumcheck did not end in the one-workgroup launch");
+      return E_DEVICE;
+    }
+    round = n;
+    return OK;
+  }
   // ---- read the logs back, and with them what the tail left of the tables: one wait for both
   const size_t final_words = (size_t)T * size * D;
   final_cache.clear();

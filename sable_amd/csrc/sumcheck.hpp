@@ -75,6 +75,15 @@ struct SumcheckSession {
   // context's, so that several sessions can be open side by side (the parts of a statement too wide for one
   // kernel, proved in step).  Such a session runs host-driven rounds.
   bool private_buffers = false;
+  // Set before run_device by a caller that chains several sumchecks on the device (the layers of LogUp-GKR): the
+  // loop's constants (eq factors, message map, constant terms, the head of the control block with the transcript's
+  // state) are then written in device memory by the launch this hook enqueues, instead of being staged and copied
+  // from the host; run_device enqueues its launches and returns without waiting or reading anything back, and the
+  // control block (logs, finals) stays in device memory for the chain's next launch.
+  std::function<int()> chain_hook;
+  // the scalar (Lagrange basis times the power of R the sums carry) that maps accumulator `acc` to wire point k in
+  // the message map: lagfix[k * nacc + acc], and the group each accumulator belongs to
+  void message_map_scalars(std::vector<uint32_t> *lagfix, std::vector<int> *acc_group) const;
   bool beyond_limits = false;  // begin refused the statement for its size alone: its parts may still fit
   Arena own_a, own_b, own_misc;
   Arena &arena_a();
