@@ -107,6 +107,7 @@ __global__ __launch_bounds__(64) void gkr_glue_kernel(GlueArgs<D> a) {
   __shared__ uint32_t ring[RING_WORDS];
   __shared__ uint32_t buf[64];
   __shared__ uint32_t chal[16];
+  __shared__ uint32_t fin[MAXT * 8];
   __shared__ uint32_t consts[GLUE_MAXCONST][8];
   __shared__ uint32_t point[MAXROUNDS + 1][8];
   const uint32_t lane = threadIdx.x;
@@ -132,13 +133,14 @@ __global__ __launch_bounds__(64) void gkr_glue_kernel(GlueArgs<D> a) {
         point[u / D][u % D] = v;  // the layer's challenges open the next layer's point
       }
     }
-    for (int t = 0; t < a.NT; t++) {  // SEND-FINALS: one message (1, D) per table, then the fresh point
-      if (lane < D) buf[lane] = a.close_kind == 2 ? a.prev_ctrl->finals[t * D + lane] : a.tabs[t][lane];
-      __builtin_amdgcn_wave_barrier();
-      dev_absorb_words(tr, buf, D);
-      if (lane < D) log_fin[t * D + lane] = buf[lane];
-      __builtin_amdgcn_wave_barrier();
+    // SEND-FINALS: one message (1, D) per table, then the fresh point (the finals fetched in one trip)
+    for (int u = lane; u < a.NT * D; u += 64) {
+      const uint32_t v = a.close_kind == 2 ? a.prev_ctrl->finals[u] : a.tabs[u / D][u % D];
+      fin[u] = v;
+      log_fin[u] = v;
     }
+    __builtin_amdgcn_wave_barrier();
+    for (int t = 0; t < a.NT; t++) dev_absorb_words(tr, fin + t * D, D);
     dev_challenge(tr, D, chal);
     __builtin_amdgcn_wave_barrier();
     if (lane < D) {
