@@ -38,7 +38,10 @@ def test_reduce_layer(d, k, m):
 
 
 CASES = [(3, 1, 1, 4), (3, 3, 2, 4), (2, 4, 1, 8), (4, 5, 2, 4), (1, 2, 1, 4), (1, 1, 2, 8), (2, 2, 3, 4),
-         (10, 1, 1, 4), (6, 1, 2, 8)]
+         (10, 1, 1, 4), (6, 1, 2, 8),
+         # one block: the layers chained on the device (up to eight base challenges per layer), from the smallest
+         # tree that chains to one whose upper layers take the grid of slices
+         (2, 1, 1, 4), (5, 1, 2, 4), (7, 1, 1, 8), (13, 1, 1, 4), (12, 1, 2, 4)]
 
 
 @pytest.mark.parametrize("n,k,lookups,d", CASES)
@@ -65,6 +68,23 @@ def test_prove_upper_matches_the_oracle(n, k, lookups, d):
             total = orc.ext_add(total, orc.ext_mul(a, orc.ext_inv(b)))
         if n <= 8:
             assert same(orc.ext_mul(root[0], orc.ext_inv(root[1])), total)
+    for p, q in dev:
+        p.free(), q.free()
+
+
+@pytest.mark.parametrize("n,lookups,d", [(9, 1, 4), (6, 2, 4), (8, 1, 8)])
+def test_the_chained_layers_and_the_host_driven_layers_send_the_same_bytes(n, lookups, d, monkeypatch):
+    rng = np.random.default_rng(100 + n)
+    leaves = random_leaves(rng, lookups, n, 1, d)
+    dev = [(sa.Table.upload(p), sa.Table.upload(q)) for p, q in leaves]
+    chained = sa.Transcript("gkr-test", d)
+    got = sa.prove_upper(chained, n, 1, dev)
+    monkeypatch.setenv("EXACTA_HIP_NO_GKR_CHAIN", "1")
+    driven = sa.Transcript("gkr-test", d)
+    want = sa.prove_upper(driven, n, 1, dev)
+    assert chained.proof() == driven.proof() and chained.state_digest() == driven.state_digest()
+    for a, b in zip(got, want):
+        assert same(a, b)
     for p, q in dev:
         p.free(), q.free()
 
