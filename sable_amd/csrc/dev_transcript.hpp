@@ -38,15 +38,16 @@ __host__ __device__ constexpr uint32_t b3_lane_words(int r, int first) {
 #define EXH_QUAD(v, ctrl) ((uint32_t)__builtin_amdgcn_update_dpp(0, (int)(v), (ctrl), 0xf, 0xf, false))
 
 // compress(cv, m, counter, block_len, flags) with the state's columns spread over the lanes of a quad.
-// cv: uniform registers; m: the 16 message words in LDS.  Lane i of each quad returns
+// cv: the chaining value's 8 words in LDS (lane i takes words i and 4 + i: from registers the choice by lane
+// becomes an indexed access, and the compiler moves the value to scratch memory for it, two trips to memory per
+// compression); m: the 16 message words in LDS.  Lane i of each quad returns
 // w0 = out[i], w1 = out[4+i], w2 = out[8+i], w3 = out[12+i].
-__device__ __forceinline__ void b3_compress_quad(const uint32_t cv[8], const uint32_t *m, uint64_t counter,
+__device__ __forceinline__ void b3_compress_quad(const uint32_t *cv, const uint32_t *m, uint64_t counter,
                                                  uint32_t block_len, uint32_t flags, uint32_t &w0, uint32_t &w1,
                                                  uint32_t &w2, uint32_t &w3) {
   const uint32_t i = threadIdx.x & 3;
   const uint32_t iv = i == 0 ? EXH_B3_IV0 : i == 1 ? EXH_B3_IV1 : i == 2 ? EXH_B3_IV2 : EXH_B3_IV3;
-  const uint32_t cva = i == 0 ? cv[0] : i == 1 ? cv[1] : i == 2 ? cv[2] : cv[3];
-  const uint32_t cvb = i == 0 ? cv[4] : i == 1 ? cv[5] : i == 2 ? cv[6] : cv[7];
+  const uint32_t cva = cv[i], cvb = cv[4 + i];
   uint32_t a = cva, b = cvb, c = iv;
   uint32_t d = i == 0 ? (uint32_t)counter : i == 1 ? (uint32_t)(counter >> 32) : i == 2 ? block_len : flags;
   uint32_t mx[7][2], my[7][2];
@@ -66,40 +67,39 @@ __device__ __forceinline__ void b3_compress_quad(const uint32_t cv[8], const uin
   w0 = a ^ c, w1 = b ^ d, w2 = c ^ cva, w3 = d ^ cvb;
 }
 
-// the first 8 output words, uniform
-__device__ __forceinline__ void b3_quad_cv(uint32_t w0, uint32_t w1, uint32_t out[8]) {
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    out[i] = (uint32_t)__builtin_amdgcn_readlane((int)w0, i);
-    out[4 + i] = (uint32_t)__builtin_amdgcn_readlane((int)w1, i);
-  }
+// the first 8 output words into the chaining value in LDS (lanes 0-3 hold them; a wavefront's LDS operations
+// complete in order, so the next compression reads the new value)
+__device__ __forceinline__ void b3_quad_cv(uint32_t w0, uint32_t w1, uint32_t *cv) {
+  const uint32_t lane = threadIdx.x & 63;
+  if (lane < 4) cv[lane] = w0, cv[4 + lane] = w1;
+  __builtin_amdgcn_wave_barrier();
 }
 
-// The running state: chaining value and counters in registers, the pending block as a 128-byte ring in
-// LDS (`ring`, the first 32 of RING_WORDS words) whose two halves are used alternately; the other 16
-// words stage a squeeze's output.  Input is appended by all lanes at once, lane k storing byte k.
-constexpr int RING_WORDS = 48;
+// The running state: counters in registers; in LDS (`ring`, RING_WORDS words) the pending block as a 128-byte
+// ring (the first 32 words) whose two halves are used alternately, 16 words that stage a squeeze's output, and the
+// chaining value (the last 8).  Input is appended by all lanes at once, lane k storing byte k.
+constexpr int RING_WORDS = 56;
 struct RunB3S {
-  uint32_t cv[8];
+  uint32_t *cv;  // ring + 48
   uint32_t *ring;
   uint32_t used, half;
   uint64_t counter;
 };
 
 __device__ inline void rb3s_load(RunB3S &s, uint32_t *ring, const DevB3S *g) {
-#pragma unroll
-  for (int i = 0; i < 8; i++) s.cv[i] = g->cv[i];
-#pragma unroll
-  for (int i = 0; i < 16; i++) ring[i] = g->block[i], ring[16 + i] = 0;
+  const uint32_t lane = threadIdx.x & 63;
+  if (lane < 8) ring[48 + lane] = g->cv[lane];
+  if (lane < 16) ring[lane] = g->block[lane], ring[16 + lane] = 0;
+  __builtin_amdgcn_wave_barrier();
+  s.cv = ring + 48;
   s.ring = ring;
   s.used = g->used, s.half = 0;
   s.counter = ((uint64_t)g->counter_hi << 32) | g->counter_lo;
 }
 __device__ inline void rb3s_store(const RunB3S &s, DevB3S *g) {
-#pragma unroll
-  for (int i = 0; i < 8; i++) g->cv[i] = s.cv[i];
-#pragma unroll
-  for (int i = 0; i < 16; i++) g->block[i] = s.ring[16 * s.half + i];
+  const uint32_t lane = threadIdx.x & 63;
+  if (lane < 8) g->cv[lane] = s.cv[lane];
+  if (lane < 16) g->block[lane] = s.ring[16 * s.half + lane];
   g->used = s.used;
   g->counter_lo = (uint32_t)s.counter, g->counter_hi = (uint32_t)(s.counter >> 32);
 }

@@ -185,12 +185,13 @@ __device__ __forceinline__ void v_mul_acc(Acc96 *acc, uint32_t a, uint32_t b) { 
 template <int D>
 __device__ __forceinline__ void v_mul_acc(Acc96 *acc, const Ext<D> &a, const Ext<D> &b) { ext_mul_acc<D>(acc, a, b); }
 
-// With PARTS > 1 only the accumulators a with a % PARTS == part are computed (part is uniform over the
-// wavefront): the last rounds, with a pair per lane and lanes to spare, give each of a workgroup's wavefronts a
+// With PARTS > 1 only the accumulators a with a % PARTS == PART are computed (a compile-time constant: with the
+// part as a run-time value, uniform as it is, the compiler folds the parts' branches into one path that indexes
+// the accumulators by it, and they move from registers to scratch memory): the last rounds, with a pair per lane and lanes to spare, give each of a workgroup's wavefronts a
 // share of a pair's accumulators, so that a round waits for a quarter of the products.
-template <int D, class V, class Desc, int PARTS = 1>
+template <int D, class V, class Desc, int PARTS = 1, int PART = 0>
 __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, const V *hi, const Ext<D> &w,
-                                                Acc96 (*acc)[D], uint32_t part = 0) {
+                                                Acc96 (*acc)[D]) {
   V cur[MAXT], slope[MAXT];
 #pragma unroll
   for (int t = 0; t < MAXT; t++)
@@ -247,7 +248,7 @@ __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, cons
 #pragma unroll
           for (int k = 0; k < MAXEV; k++) {
             if (k < d.nev[g]) {
-              if (d.ev[g][k] == x && (PARTS == 1 || (uint32_t)(a % PARTS) == part)) {
+              if (d.ev[g][k] == x && (PARTS == 1 || a % PARTS == PART)) {
                 // the product of the factors but the last; the last goes with the accumulation
                 const bool pre = EXT && d.nev[g] >= 3 && d.deg[g] >= 2;
                 V prod = pre ? wcur[g] : cur[d.tab[g][0]];
@@ -798,6 +799,20 @@ __global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) 
   round_epilogue<D>(args.ctrl, sums, args.nacc, args.points, epi.mtilde, epi.c0, &epi, true);
 }
 
+// A small round's sums on one wavefront: the accumulators PART, PART + 4, ... of the lane's pair, summed over the
+// wavefront into sums (LDS).  The accumulators are this function's own, so that they live in registers.
+template <int D, int PART, class Desc>
+__device__ __forceinline__ void small_round_sums(const Desc &d, const Ext<D> *lo, const Ext<D> *hi, const Ext<D> &w,
+                                                 uint32_t *sums) {
+  Acc96 acc[MAXACC][D];
+#pragma unroll
+  for (int a = 0; a < MAXACC; a++)
+#pragma unroll
+    for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
+  accumulate_pair<D, Ext<D>, Desc, 4, PART>(d, lo, hi, w, acc);
+  part_wave_sums<D, PART, 4>(d, acc, sums);
+}
+
 // Load (folding or lifting on the way in) into LDS, then per round sums -> message -> challenge -> fold
 // on the slice this workgroup holds: entries [w * E, (w + 1) * E) of every table, E = entries / grid.
 // A grid launch ends when its rounds are done and leaves the slices in `out` for the one-workgroup
@@ -880,50 +895,51 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
     const uint32_t pairs = entries / 2;
     const bool small = pairs <= 64 && BLOCK == 256;
     {  // the round's sums
-      Acc96 acc[MAXACC][D];
-#pragma unroll
-      for (int a = 0; a < MAXACC; a++)
-#pragma unroll
-        for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
-      if (small && lane < pairs) {
+      if (small) {  // each wavefront its own share of the pair's accumulators, in code of its own
         Ext<D> lo[MAXT], hi[MAXT];
+        const uint32_t at = lane < pairs ? lane : 0;
 #pragma unroll
         for (int t = 0; t < MAXT; t++)
           if (t < d.T) {
-            const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * lane) * D;
+            const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * at) * D;
             lo[t] = load_ext<D>(p);
             hi[t] = load_ext<D>(p + D);
           }
-        accumulate_pair<D, Ext<D>, Desc, 4>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc, wave);
-      }
-      for (uint32_t i = tid; i < pairs && !small; i += BLOCK) {
-        Ext<D> lo[MAXT], hi[MAXT];
-#pragma unroll
-        for (int t = 0; t < MAXT; t++)
-          if (t < d.T) {
-            const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * i) * D;
-            lo[t] = load_ext<D>(p);
-            hi[t] = load_ext<D>(p + D);
-          }
-        if (i >= BLOCK) {  // beyond the prefetched pair
-          const uint64_t gi = (uint64_t)wg * pairs + i;
-          wl = load_ext<D>(args.weights + (args.low_off[jj] + (gi & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
-          wh = load_ext<D>(args.weights + (args.high_off[jj] + (gi >> args.low_bits[jj])) * D);
-        }
-        accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
-      }
-      if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
-      if (small) {
+        Ext<D> ww = ext_mul_mont<D>(wl, wh);
+        if (lane >= pairs) ww = ext_zero<D>();  // lanes without a pair add nothing
+        if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
         if (wave == 0)
-          part_wave_sums<D, 0, 4>(d, acc, sums);
+          small_round_sums<D, 0>(d, lo, hi, ww, sums);
         else if (wave == 1)
-          part_wave_sums<D, 1, 4>(d, acc, sums);
+          small_round_sums<D, 1>(d, lo, hi, ww, sums);
         else if (wave == 2)
-          part_wave_sums<D, 2, 4>(d, acc, sums);
+          small_round_sums<D, 2>(d, lo, hi, ww, sums);
         else
-          part_wave_sums<D, 3, 4>(d, acc, sums);
+          small_round_sums<D, 3>(d, lo, hi, ww, sums);
         lds_barrier();
       } else {
+        Acc96 acc[MAXACC][D];
+#pragma unroll
+        for (int a = 0; a < MAXACC; a++)
+#pragma unroll
+          for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
+        for (uint32_t i = tid; i < pairs; i += BLOCK) {
+          Ext<D> lo[MAXT], hi[MAXT];
+#pragma unroll
+          for (int t = 0; t < MAXT; t++)
+            if (t < d.T) {
+              const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * i) * D;
+              lo[t] = load_ext<D>(p);
+              hi[t] = load_ext<D>(p + D);
+            }
+          if (i >= BLOCK) {  // beyond the prefetched pair
+            const uint64_t gi = (uint64_t)wg * pairs + i;
+            wl = load_ext<D>(args.weights + (args.low_off[jj] + (gi & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
+            wh = load_ext<D>(args.weights + (args.high_off[jj] + (gi >> args.low_bits[jj])) * D);
+          }
+          accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
+        }
+        if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
         block_sums<D, true>(d, acc, lds, sums);
       }
       if (G > 1) {
@@ -1344,7 +1360,7 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(2, 2))) v
   round_body<D, IN_BASE, FOLD, decltype(S::d), false, true>(S::d, args);
 }
 template <int D, class S>
-__global__ __launch_bounds__(BLOCK) void tail_kernel(TailArgs<D> args) {
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(1, 1))) void tail_kernel(TailArgs<D> args) {
   tail_body<D>(S::d, args);
 }
 template <int D, class S>
