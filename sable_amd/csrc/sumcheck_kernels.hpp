@@ -744,24 +744,27 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
 // XCD's whole L2 and costs more than a launch.)
 // sums[o] = sum over the workgroups' partial rows of word o (o < width <= blockDim.x): thread t takes column
 // t % width of the rows t / width, t / width + groups, ... with groups = blockDim.x / width, so that all
-// threads share the rows whatever the row stride; eight loads in flight per thread.
+// threads share the rows whatever the row stride; sixteen loads in flight per thread.
 // All threads of the workgroup call; scratch holds blockDim.x words.
 __device__ __forceinline__ void sum_partials(const uint32_t *partials, uint32_t nblocks, uint32_t ps, uint32_t width,
                                              uint32_t *scratch, uint32_t *sums) {
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   const uint32_t groups = width ? nthreads / width : 0, col = width ? tid % width : 0, row0 = width ? tid / width : 0;
+  // sixteen loads in flight per thread and trip to memory, the last batch's rows beyond the end masked off (a loop
+  // over single rows behind full batches would be a trip to memory per row)
   uint32_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if (row0 < groups) {
     const uint32_t *p = partials + col;
-    uint32_t b = row0;
-    for (; b + 7 * groups < nblocks; b += 8 * groups) {
-      uint32_t x[8];
+    for (uint32_t b = row0; b < nblocks; b += 16 * groups) {
+      uint32_t x[16];
 #pragma unroll
-      for (int q = 0; q < 8; q++) x[q] = p[(uint64_t)(b + q * groups) * ps];
+      for (int q = 0; q < 16; q++) {
+        const uint32_t row = b + q * groups;
+        x[q] = row < nblocks ? p[(uint64_t)row * ps] : 0u;
+      }
 #pragma unroll
-      for (int q = 0; q < 8; q++) v[q] = fadd(v[q], x[q]);
+      for (int q = 0; q < 16; q++) v[q & 7] = fadd(v[q & 7], x[q]);
     }
-    for (; b < nblocks; b += groups) v[0] = fadd(v[0], p[(uint64_t)b * ps]);
   }
   __syncthreads();
   scratch[tid] = fadd(fadd(fadd(v[0], v[1]), fadd(v[2], v[3])), fadd(fadd(v[4], v[5]), fadd(v[6], v[7])));
@@ -1258,6 +1261,13 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
   __shared__ uint32_t basis[(MAXDEG + 1) * (MAXDEG + 1) * D];  // [deg][node]: Lagrange basis at r0, Montgomery form
   __shared__ EpilogueLds epi;
   const uint32_t tid = threadIdx.x, ps = args.e.pstride, points = args.e.points, nacc = args.e.nacc;
+  // the statement's shape into LDS first: indexed by lane-dependent values out of the kernel's arguments, every
+  // access would be a load from memory with the next one waiting behind it
+  __shared__ uint32_t s_deg[MAXG], s_nev[MAXG], s_inv_den[(MAXDEG + 1) * (MAXDEG + 1)];
+  __shared__ uint8_t s_ev[MAXG][MAXEV];
+  if (tid < MAXG) s_deg[tid] = args.deg[tid], s_nev[tid] = args.nev[tid];
+  if (tid < MAXG * MAXEV) s_ev[tid / MAXEV][tid % MAXEV] = args.ev[tid / MAXEV][tid % MAXEV];
+  if (tid < (MAXDEG + 1) * (MAXDEG + 1)) s_inv_den[tid] = args.inv_den[tid];
   if (tid < sizeof(DevB3S) / 4) epi.state[tid] = reinterpret_cast<const uint32_t *>(&args.e.ctrl->tr)[tid];
   for (uint32_t u = tid; u < points * nacc * D; u += EPI_BLOCK) epi.mtilde[u] = args.e.mtilde[u];
   for (uint32_t u = tid; u < points * D; u += EPI_BLOCK) epi.c0[u] = args.e.c0[u];
@@ -1269,9 +1279,9 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
     return v;
   };
   auto row_of = [&](uint32_t g, uint32_t x) {  // the index of X among group g's points, or nev
-    uint32_t at = args.nev[g];
-    for (uint32_t e = 0; e < args.nev[g]; e++)
-      if (args.ev[g][e] == x) at = e;
+    uint32_t at = s_nev[g];
+    for (uint32_t e = 0; e < s_nev[g]; e++)
+      if (s_ev[g][e] == x) at = e;
     return at;
   };
   // accumulator tid is point e of group g, whose slots start at `base` (every thread finds its own, so that the
@@ -1281,19 +1291,19 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
   {
     uint32_t a = 0;
     for (uint32_t k = 0; k < args.groups && !mine; k++) {
-      const uint32_t nev = args.nev[k];
+      const uint32_t nev = s_nev[k];
       if (tid < a + nev) {
         g = k, e = tid - a, mine = true;
       } else {
         a += nev;
-        base += nev * (args.deg[k] + 1) + (row_of(k, 1) < nev ? 0 : nev);
+        base += nev * (s_deg[k] + 1) + (row_of(k, 1) < nev ? 0 : nev);
       }
     }
   }
   // ---- round 0: accumulator (g, e) = eq(w1, 0) * slot(X1 = 0, node ev_e) + eq(w1, 1) * slot(X1 = 1, node ev_e)
   if (mine) {
-    const uint32_t deg = args.deg[g], nev = args.nev[g], row0 = row_of(g, 0), row1 = row_of(g, 1);
-    const uint32_t node = args.ev[g][e];
+    const uint32_t deg = s_deg[g], nev = s_nev[g], row0 = row_of(g, 0), row1 = row_of(g, 1);
+    const uint32_t node = s_ev[g][e];
     Ext<D> at0 = slot(base + row0 * (deg + 1) + node);
     Ext<D> at1 = row1 < nev ? slot(base + row1 * (deg + 1) + node) : slot(base + nev * (deg + 1) + e);
     if (args.eq1) {
@@ -1326,7 +1336,7 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
         f.c[0] = fsub(f.c[0], to_mont(q));  // (r0 - q) R
         acc = ext_mul_mont<D>(acc, f);
       }
-      acc = ext_scale_mont<D>(acc, args.inv_den[tid]);
+      acc = ext_scale_mont<D>(acc, s_inv_den[tid]);
 #pragma unroll
       for (int c = 0; c < D; c++) basis[tid * D + c] = acc.c[c];
     }
@@ -1334,7 +1344,7 @@ __global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogue
   __syncthreads();
   // accumulator (g, e) = sum over nodes of basis * slot
   if (mine) {
-    const uint32_t deg = args.deg[g];
+    const uint32_t deg = s_deg[g];
     Ext<D> total = ext_zero<D>();
     for (uint32_t m = 0; m <= deg; m++) {
       Ext<D> lb;
