@@ -39,7 +39,7 @@ INT32_MUL_PEAK_PER_S = 256 * 4 * 64 / 4.7 * 2.4e9
 # the same counter reads for the plain copy kernel of `--workload copy`), and 32-bit integer multiply instructions
 # per lane and prove from the kernels' instruction streams times their trip counts (profiles/ holds both summaries).
 MEASURED = {
-    "kernel_sources_sha256": "e7a998c12cbd1c73f47dfc4fb29bbfb8c7070d731fc306b70abddcdf28c232b2",
+    "kernel_sources_sha256": "25798b90bc808a00208308fa49982b309a94d1ff3b97bc27610242b52e854c0d",
     "traffic": {("round_nodes_base", 24): 203430854, ("round_fold2_base", 24): 403997705},
     "int32_mul_per_prove": 2063597568,
 }

@@ -187,8 +187,9 @@ __device__ __forceinline__ void v_mul_acc(Acc96 *acc, const Ext<D> &a, const Ext
 
 // With PARTS > 1 only the accumulators a with a % PARTS == PART are computed (a compile-time constant: with the
 // part as a run-time value, uniform as it is, the compiler folds the parts' branches into one path that indexes
-// the accumulators by it, and they move from registers to scratch memory): the last rounds, with a pair per lane and lanes to spare, give each of a workgroup's wavefronts a
-// share of a pair's accumulators, so that a round waits for a quarter of the products.
+// the accumulators by it, and they move from registers to scratch memory): the last rounds, with a pair per lane
+// and lanes to spare, give each of a workgroup's wavefronts a share of a pair's accumulators, so that a round
+// waits for a quarter of the products.
 template <int D, class V, class Desc, int PARTS = 1, int PART = 0>
 __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, const V *hi, const Ext<D> &w,
                                                 Acc96 (*acc)[D]) {
