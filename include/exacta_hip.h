@@ -58,6 +58,9 @@ int exh_stmt_has_generated_kernel(exh_stmt stmt, int degree_d);
    (-1: the statement's own).  Returns 1 when the kernels are in place, 0 while they compile (wait = 0), or
    EXH_E_DEVICE with the compiler's log when the compilation failed; with wait != 0 it returns once it has ended. */
 int exh_stmt_generate(exh_stmt stmt, int degree_d, int degree, int wait);
+/* 1 when no compilation is running, 0 while one is; with wait != 0 it returns 1 once none is (a host that wants an
+   orderly exit calls it before it ends: see above) */
+int exh_stmt_generate_idle(int wait);
 
 /* ---- measurement (no counterpart in the reference): with profiling on, every data-parallel kernel
    launch is bracketed by HIP events on the library's stream; entries report the kernel, the round it

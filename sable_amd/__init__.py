@@ -214,6 +214,11 @@ class Transcript:
         return bytes(out[:n.value])
 
 
+def generation_idle(wait=True):
+    """exh_stmt_generate_idle: True when no run-time compilation of kernels is running (waits for that when asked)."""
+    return load().exh_stmt_generate_idle(1 if wait else 0) == 1
+
+
 def blake3(data, n=32):
     out = (C.c_uint8 * n)()
     check(load().exh_blake3(bytes(data), C.c_uint64(len(data)), out, C.c_uint64(n)))

@@ -266,6 +266,10 @@ int exh_stmt_has_generated_kernel(exh_stmt stmt, int D) {
   if (ctx().ready) (void)rtc_collect();
   return find_kernels(copy.key(), D) ? 1 : 0;
 }
+int exh_stmt_generate_idle(int wait) {
+  ApiLock api_lock;
+  return rtc_idle(wait != 0);
+}
 int exh_stmt_generate(exh_stmt stmt, int D, int degree, int wait) {
   ApiLock api_lock;
   Statement *st = stmt_of(stmt);

@@ -288,6 +288,20 @@ int rtc_collect() {
   return status;
 }
 
+int rtc_idle(bool wait) {
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    for (auto &kv : g_jobs) {
+      if (kv.second->running.load() == 0) continue;
+      if (!wait) return 0;
+      for (std::thread &t : kv.second->threads)
+        if (t.joinable()) t.join();
+    }
+  }
+  int status = rtc_collect();
+  return status ? status : 1;
+}
+
 int rtc_status(const std::string &key, int D, bool wait) {
   {
     std::lock_guard<std::mutex> lock(g_mutex);

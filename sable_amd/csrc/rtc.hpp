@@ -21,5 +21,7 @@ int rtc_collect();
 // 1: kernels for (key, D) are registered; 0: their compilation is still running (or was never asked for);
 // E_DEVICE with the compiler's log as the error text when it failed.  With wait, blocks until it has ended.
 int rtc_status(const std::string &key, int D, bool wait);
+// 1 when no compilation is running (with wait: once none is, their kernels loaded), 0 while one runs
+int rtc_idle(bool wait);
 
 }  // namespace exh

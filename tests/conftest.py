@@ -13,6 +13,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionfinish(session, exitstatus):
+    """A proof of an unseen statement over large tables starts a compilation of its kernels in the background; the
+    session waits for the last of them, so that the process ends in the ordinary way."""
+    lib = sys.modules.get("sable_amd.lib")
+    if lib is not None and getattr(lib, "_lib", None) is not None:
+        lib._lib.exh_stmt_generate_idle(1)
+
+
 @pytest.fixture(scope="session")
 def vectors():
     """The reference's golden vectors (tests/vectors.sexp converted by tests/golden/make_vectors.py)."""
