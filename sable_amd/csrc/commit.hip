@@ -19,7 +19,7 @@ namespace exh {
 // ------------------------------------------------------------------ twiddle tables of a domain
 // Level l of the 2^n tables (src/rs.lisp:44-55) holds x_s = w_n^(2^l bitrev_{n-1-l}(s)) for the
 // 2^(n-1-l) position pairs of the level-l codeword.  Both x (for the encoder's butterflies) and
-// 1/(2x) (for folding) are kept on the device in Montgomery form, levels concatenated.
+// 1/(2x) (for folding) are kept on the device, levels concatenated: x as the plain residue, 1/(2x) in Montgomery form.
 struct Domain {
   int n = 0;
   uint32_t *tw = nullptr, *tw_inv2 = nullptr;
@@ -45,7 +45,8 @@ __global__ __launch_bounds__(BLOCK) void twiddle_kernel(LevelOffsets lv, const u
   uint32_t s = (uint32_t)(gid - lv.off[l]);
   uint32_t e = bitrev_dev(s, lv.n - 1 - l) << l;  // exponent of w_n, below 2^(n-1)
   // mont_mul of two Montgomery-form values is the Montgomery form of the product
-  tw[gid] = mont_mul(pw[e & 4095], pw[4096 + (e >> 12)]);
+  // (the encoder multiplies in double precision and takes the plain residue, the fold the Montgomery form)
+  tw[gid] = mont_mul(mont_mul(pw[e & 4095], pw[4096 + (e >> 12)]), 1);
   tw_inv2[gid] = mont_mul(pw_inv[e & 4095], pw_inv[4096 + (e >> 12)]);
 }
 
@@ -107,60 +108,91 @@ static int get_domain(int n, Domain **out) {
 //
 // Inside the tile the stages run four at a time in registers: a thread gathers the 16 elements that
 // differ in the four stage bits, does the 32 butterflies, and scatters them back, so LDS and the
-// workgroup barrier are touched once per four stages.  LDS words are padded by one per 32 so that
+// workgroup barrier are touched once per four stages.  The tile is padded by one element per 16 so that
 // the strided gathers fall on distinct banks.
-// A tile is 2^12 words, 16 per thread: a domain of 2^24 takes three passes (6 + 5 + 12 stages) with
-// global segments of at least 64 words.  The passes are bound by the butterflies' instructions (a
-// Montgomery product and two modular additions each, plus the LDS traffic), not by their bytes: tiles
-// of 2^14 words, which need two passes only, measured slower (338 us against 295 us for both columns
-// of 2^24).
+// A tile is 2^12 elements, 16 per thread: a domain of 2^24 takes three passes (6 + 5 + 12 stages) with
+// global segments of at least 64 words.
+// The butterflies run in double precision (field.hpp), whose fused multiply-add issues at four times the rate of
+// a 32-bit integer multiply: a product by a twiddle is six operations and leaves a residue within about p/2 of
+// zero, and the sum and the difference that follow are one operation each with no reduction, exact as long as
+// the values stay integers below 2^53: a tile's elements start below p and grow by less than 0.57 p per stage,
+// so after a pass's twelve stages at most they are below 8 p, and a product with a twiddle below 2^65.  The tile
+// in LDS therefore holds doubles; a pass ends by writing canonical residues.  The passes are bound by their
+// instructions all the same (the vector units about three quarters busy, some 330 instructions per thread and
+// round of four stages): both columns of 2^24 take 64 + 56 + 92 us, against 300 us with Montgomery products.
 constexpr int NTT_TILE_BITS = 12;
 constexpr int NTT_BLOCK = 256;
 constexpr int NTT_MAX_UPPER_STAGES = 7;  // per pass above the last: segments of 2^(12-7) words at least
-__device__ __forceinline__ uint32_t ntt_pad(uint32_t e) { return e + (e >> 5); }
+static_assert(NTT_TILE_BITS <= 12, "a pass's stages, the bound on the lazily reduced values");
+__device__ __forceinline__ uint32_t ntt_pad(uint32_t e) { return e + (e >> 4); }
+constexpr uint32_t ntt_lds_bytes(int tile_bits) {
+  return (((uint32_t)1 << tile_bits) + ((uint32_t)1 << tile_bits >> 4) + 1) * 8;
+}
 
-// R stages d_lo .. d_lo + R - 1 of the pass (stage d pairs tile indices differing in bit cbits + d)
-template <int R>
-__device__ __forceinline__ void ntt_round(uint32_t *lds, uint32_t tile, int cbits, int d_lo, int b_lo, int b_hi,
-                                          uint64_t top, const uint32_t *tw, const LevelOffsets &lv) {
+// R stages d_lo .. d_lo + R - 1 of the pass (stage d pairs tile indices differing in bit cbits + d).  A thread
+// takes groups of 2^R elements, its number of groups known at compile time for a FULL tile (2^NTT_TILE_BITS): the
+// twiddles of all its groups are then fetched before the first butterfly, one wait for memory per round where a
+// loop over the groups has one per group.  (Deriving a group's 2^R - 1 twiddles from one table entry, by squarings
+// and products with fixed roots of unity, was measured: the passes are bound by their instructions, and fourteen
+// more products per thirty-two butterflies cost more than the fetches.)
+template <int R, bool FULL>
+__device__ __forceinline__ void ntt_round(double *lds, uint32_t tile, int cbits, int d_lo, int b_lo, int b_hi,
+                                          uint64_t top, const uint32_t *__restrict__ tw, const LevelOffsets &lv) {
+  constexpr int GROUPS = FULL ? ((1 << NTT_TILE_BITS) >> R) / NTT_BLOCK : 1;
   const int p = cbits + d_lo;
-  for (uint32_t g = threadIdx.x; g < (tile >> R); g += NTT_BLOCK) {
-    const uint32_t upper = g >> p, e_base = (upper << (p + R)) | (g & ((1u << p) - 1));
-    uint32_t v[1 << R], t[(1 << R) - 1];
+  // a FULL tile's rounds have p = 0 or p >= 4 (a pass above the last keeps 2^cbits >= 32 consecutive indices, the
+  // last one runs its twelve stages four at a time): a group's padded positions are then evenly spaced
+  const uint32_t spacing = (1u << p) + ((1u << p) >> 4);
+  for (uint32_t g0 = threadIdx.x; g0 < (tile >> R); g0 += GROUPS * NTT_BLOCK) {
+    uint32_t t[GROUPS][(1 << R) - 1];
     // the twiddles of stage d_lo + s: 2^(R-1-s) of them, index (top | mid above the stage bit)
 #pragma unroll
-    for (int s = R - 1; s >= 0; s--) {
-      const int b = b_lo + d_lo + s;
-      const uint32_t *level = tw + lv.off[b] + ((top << (b_hi - b)) | ((uint64_t)upper << (R - 1 - s)));
+    for (int it = 0; it < GROUPS; it++) {
+      const uint32_t upper = (g0 + it * NTT_BLOCK) >> p;
 #pragma unroll
-      for (int jh = 0; jh < (1 << (R - 1 - s)); jh++) t[(1 << (R - 1 - s)) - 1 + jh] = level[jh];
-    }
+      for (int s = R - 1; s >= 0; s--) {
+        const int b = b_lo + d_lo + s;
+        const uint32_t *level = tw + lv.off[b] + ((top << (b_hi - b)) | ((uint64_t)upper << (R - 1 - s)));
 #pragma unroll
-    for (int j = 0; j < (1 << R); j++) v[j] = lds[ntt_pad(e_base | ((uint32_t)j << p))];
-#pragma unroll
-    for (int s = R - 1; s >= 0; s--) {
-#pragma unroll
-      for (int jh = 0; jh < (1 << (R - 1 - s)); jh++) {
-        const uint32_t x = t[(1 << (R - 1 - s)) - 1 + jh];
-#pragma unroll
-        for (int jl = 0; jl < (1 << s); jl++) {
-          const int j = (jh << (s + 1)) | jl;
-          uint32_t a = v[j], tc = mont_mul(x, v[j + (1 << s)]);
-          v[j] = fadd(a, tc);
-          v[j + (1 << s)] = fsub(a, tc);
-        }
+        for (int jh = 0; jh < (1 << (R - 1 - s)); jh++) t[it][(1 << (R - 1 - s)) - 1 + jh] = level[jh];
       }
     }
 #pragma unroll
-    for (int j = 0; j < (1 << R); j++) lds[ntt_pad(e_base | ((uint32_t)j << p))] = v[j];
+    for (int it = 0; it < GROUPS; it++) {
+      const uint32_t g = g0 + it * NTT_BLOCK, upper = g >> p, e_base = (upper << (p + R)) | (g & ((1u << p) - 1));
+      double *const group = lds + ntt_pad(e_base);
+      auto at = [&](int j) -> double & { return FULL ? group[j * spacing] : lds[ntt_pad(e_base | ((uint32_t)j << p))]; };
+      double v[1 << R];
+#pragma unroll
+      for (int j = 0; j < (1 << R); j++) v[j] = at(j);
+#pragma unroll
+      for (int s = R - 1; s >= 0; s--) {
+#pragma unroll
+        for (int jh = 0; jh < (1 << (R - 1 - s)); jh++) {
+          const double x = (double)t[it][(1 << (R - 1 - s)) - 1 + jh];
+#pragma unroll
+          for (int jl = 0; jl < (1 << s); jl++) {
+            const int j = (jh << (s + 1)) | jl;
+            const double a = v[j], tc = f_mul(x, v[j + (1 << s)]);
+            v[j] = a + tc;
+            v[j + (1 << s)] = a - tc;
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < (1 << R); j++) at(j) = v[j];
+    }
   }
 }
 
-__global__ __launch_bounds__(NTT_BLOCK) void ntt_pass_kernel(const uint32_t *in, uint32_t *out, int n, int b_hi,
-                                                             int b_lo, int tile_bits, const uint32_t *tw,
-                                                             LevelOffsets lv, int first, uint64_t in_stride,
-                                                             uint64_t out_stride) {
-  extern __shared__ uint32_t lds[];  // 2^tile_bits words plus one per 32
+// FULL: the tile is 2^NTT_TILE_BITS words and `in`, `out` and the columns' strides are multiples of 16 bytes: a
+// thread moves its sixteen words as four vectors of four consecutive ones (a segment of consecutive indices is a
+// multiple of four long, or the tile is one segment), all four fetches in flight at once.
+template <bool FULL>
+__global__ __launch_bounds__(NTT_BLOCK) __attribute__((amdgpu_waves_per_eu(5, 8))) void ntt_pass_kernel(
+    const uint32_t *in, uint32_t *out, int n, int b_hi, int b_lo, int tile_bits,
+    const uint32_t *__restrict__ tw, LevelOffsets lv, int first, uint64_t in_stride, uint64_t out_stride) {
+  extern __shared__ double lds[];  // 2^tile_bits elements plus one per 16
   const int S = b_hi - b_lo + 1, cbits = tile_bits - S;
   const uint32_t tile = 1u << tile_bits, C = 1u << cbits;
   in += (uint64_t)blockIdx.y * in_stride;
@@ -169,27 +201,49 @@ __global__ __launch_bounds__(NTT_BLOCK) void ntt_pass_kernel(const uint32_t *in,
   const uint64_t top = blockIdx.x / chunks_per_top, chunk = blockIdx.x % chunks_per_top;
   const uint64_t base = (top << (b_hi + 1)) | (chunk << cbits);
   const uint64_t msg_mask = ((uint64_t)1 << (n - 1)) - 1;
-  for (uint32_t e = threadIdx.x; e < tile; e += NTT_BLOCK) {
-    uint64_t g = base | ((uint64_t)(e >> cbits) << b_lo) | (e & (C - 1));
-    lds[ntt_pad(e)] = first ? in[g & msg_mask] : in[g];
+  auto global_index = [&](uint32_t e) { return base | ((uint64_t)(e >> cbits) << b_lo) | (e & (C - 1)); };
+  if (FULL) {
+    uint4 w[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const uint64_t g = global_index(4 * (threadIdx.x + k * NTT_BLOCK));
+      w[k] = *reinterpret_cast<const uint4 *>(in + (first ? g & msg_mask : g));
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      double *at = lds + ntt_pad(4 * (threadIdx.x + k * NTT_BLOCK));  // (four elements never straddle a pad)
+      at[0] = (double)w[k].x, at[1] = (double)w[k].y, at[2] = (double)w[k].z, at[3] = (double)w[k].w;
+    }
+  } else {
+    for (uint32_t e = threadIdx.x; e < tile; e += NTT_BLOCK) {
+      const uint64_t g = global_index(e);
+      lds[ntt_pad(e)] = (double)(first ? in[g & msg_mask] : in[g]);
+    }
   }
   __syncthreads();
   for (int d_hi = S - 1; d_hi >= 0;) {
     const int R = d_hi + 1 < 4 ? d_hi + 1 : 4, d_lo = d_hi - R + 1;
     if (R == 4)
-      ntt_round<4>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
+      ntt_round<4, FULL>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
     else if (R == 3)
-      ntt_round<3>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
+      ntt_round<3, FULL>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
     else if (R == 2)
-      ntt_round<2>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
+      ntt_round<2, FULL>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
     else
-      ntt_round<1>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
+      ntt_round<1, FULL>(lds, tile, cbits, d_lo, b_lo, b_hi, top, tw, lv);
     __syncthreads();
     d_hi = d_lo - 1;
   }
-  for (uint32_t e = threadIdx.x; e < tile; e += NTT_BLOCK) {
-    uint64_t g = base | ((uint64_t)(e >> cbits) << b_lo) | (e & (C - 1));
-    out[g] = lds[ntt_pad(e)];
+  if (FULL) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const uint32_t e = 4 * (threadIdx.x + k * NTT_BLOCK);
+      const double *at = lds + ntt_pad(e);
+      *reinterpret_cast<uint4 *>(out + global_index(e)) =
+          make_uint4(f_canonical(at[0]), f_canonical(at[1]), f_canonical(at[2]), f_canonical(at[3]));
+    }
+  } else {
+    for (uint32_t e = threadIdx.x; e < tile; e += NTT_BLOCK) out[global_index(e)] = f_canonical(lds[ntt_pad(e)]);
   }
 }
 
@@ -217,13 +271,12 @@ int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_
   lv.levels = n - 1, lv.n = n;
   for (int l = 0; l < n - 1; l++) lv.off[l] = dom->off[l];
   int tile_bits = n - 1 < NTT_TILE_BITS ? n - 1 : NTT_TILE_BITS;  // a tile never spans two tops
-  const uint32_t lds_bytes = (((uint32_t)1 << tile_bits) + ((uint32_t)1 << tile_bits >> 5) + 1) * 4;
-  static bool lds_enabled = false;
-  if (!lds_enabled) {  // more than the default 64 KiB of dynamic LDS
-    EXH_HIP(hipFuncSetAttribute((const void *)ntt_pass_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                ((1 << NTT_TILE_BITS) + (1 << (NTT_TILE_BITS - 5)) + 1) * 4));
-    lds_enabled = true;
-  }
+  const uint32_t lds_bytes = ntt_lds_bytes(tile_bits);
+  // whole tiles whose words move four at a time: every address and stride a multiple of 16 bytes, segments of
+  // consecutive indices at least four long (a pass above the last has 2^(tile_bits - stages) >= 32 of them)
+  const bool full = tile_bits == NTT_TILE_BITS && (reinterpret_cast<uintptr_t>(d_messages) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(d_codewords) & 15) == 0;
+  static_assert(NTT_TILE_BITS - NTT_MAX_UPPER_STAGES >= 2, "segments of four words at least");
   // stages n-2 .. 0: the last pass takes the low tile_bits stages, earlier passes share the rest
   int b = n - 2;
   bool first = true;
@@ -239,9 +292,9 @@ int rs_encode_columns(const uint32_t *d_messages, int ncols, int c, uint32_t *d_
       b_lo = b - take + 1;
     }
     uint32_t grid = (uint32_t)(len >> tile_bits);
-    hipLaunchKernelGGL(ntt_pass_kernel, dim3(grid, ncols), dim3(NTT_BLOCK), lds_bytes, cx.stream,
-                       first ? d_messages : d_codewords, d_codewords, n, b, b_lo, tile_bits, dom->tw, lv, first ? 1 : 0,
-                       first ? len / 2 : len, len);
+    hipLaunchKernelGGL(full ? ntt_pass_kernel<true> : ntt_pass_kernel<false>, dim3(grid, ncols), dim3(NTT_BLOCK),
+                       lds_bytes, cx.stream, first ? d_messages : d_codewords, d_codewords, n, b, b_lo, tile_bits,
+                       dom->tw, lv, first ? 1 : 0, first ? len / 2 : len, len);
     first = false;
     b = b_lo - 1;
   }

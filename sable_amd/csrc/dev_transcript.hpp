@@ -143,7 +143,11 @@ __device__ inline void dev_absorb_words(RunB3S &s, const uint32_t *words, uint32
 // K <= 8 base-field challenges (CHALLENGE-BASE, src/transcript.lisp:159-172): squeeze 4 (missing + 4)
 // bytes, keep the 31-bit words below p, repeat until K are kept; each squeeze then absorbs "squeeze" and
 // the first min(32, n) bytes of its output (src/transcript.lisp:152-157).  OUT is in LDS.
-__device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out) {
+// `ready` is called by the whole wavefront as soon as the K challenges are in OUT: what follows (absorbing the last
+// squeeze's bytes, a compression when they fill the block) is the transcript's own bookkeeping, which whoever waits
+// for the challenge need not wait for.
+template <class F>
+__device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out, F ready) {
   const uint32_t lane = threadIdx.x & 63;
   uint32_t *stage = s.ring + 32;
   int have = 0;
@@ -161,14 +165,18 @@ __device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out) {
     else if (lane < 7 + fed)
       byte = (stage[(lane - 7) >> 2] >> (8 * ((lane - 7) & 3))) & 0xff;
     const uint32_t cand = lane < n / 4 ? stage[lane] & 0x7fffffffu : P;
-    rb3s_append_bytes(s, byte, 7 + fed);
     // the candidates below p, in order, as far as needed
     const uint64_t ok = __ballot(cand < P);
     const int rank = __popcll(ok & (((uint64_t)1 << lane) - 1));
     if (cand < P && have + rank < k) out[have + rank] = cand;
     have += __popcll(ok);
     __builtin_amdgcn_wave_barrier();
+    if (have >= k) ready();
+    rb3s_append_bytes(s, byte, 7 + fed);
   }
+}
+__device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out) {
+  dev_challenge(s, k, out, [] {});
 }
 
 }  // namespace exh

@@ -599,19 +599,22 @@ __device__ __forceinline__ void round_message(const uint32_t *sums, uint32_t nac
 }
 
 // the first wavefront's part: send the message, draw the challenge, log both (every lane the same steps)
+// With `publish` (an LDS word), the challenge times R is in e->r_mont and *publish = round + 1 as soon as it is
+// drawn, before the transcript absorbs the squeeze's bytes: the workgroup's other wavefronts wait for that word
+// instead of a barrier and begin the fold while this one finishes the transcript's bookkeeping.
 template <int D>
 __device__ __forceinline__ void transcript_step(RunB3S &tr, Ctrl *ctrl, uint32_t round, uint32_t points,
-                                                EpilogueLds *e, bool log = true) {
+                                                EpilogueLds *e, bool log = true, uint32_t *publish = nullptr) {
   const uint32_t tid = threadIdx.x;
   dev_absorb_words(tr, e->msg, points * D);
-  dev_challenge(tr, D, e->chal);
+  dev_challenge(tr, D, e->chal, [&] {
+    if (tid < (uint32_t)D) e->r_mont[tid] = to_mont(e->chal[tid]);
+    __builtin_amdgcn_wave_barrier();
+    if (publish && tid == 0) __hip_atomic_store(publish, round + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  });
   if (log)
     for (uint32_t o = tid; o < points * D; o += 64) ctrl->msg[round][o] = e->msg[o];
-  if (tid < (uint32_t)D) {
-    const uint32_t rm = to_mont(e->chal[tid]);
-    e->r_mont[tid] = rm;
-    if (log) ctrl->chal[round][tid] = e->chal[tid], ctrl->r_mont[tid] = rm;
-  }
+  if (log && tid < (uint32_t)D) ctrl->chal[round][tid] = e->chal[tid], ctrl->r_mont[tid] = e->r_mont[tid];
 }
 
 template <int D>
@@ -828,7 +831,9 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   __shared__ uint32_t sums[MAXACC * D];
   __shared__ EpilogueLds epi;
   __shared__ uint32_t c0s[MAXTAIL * MAXPTS * D];
+  __shared__ uint32_t ready_round;  // rounds whose challenge the first wavefront has published, counted from the proof's first
   const uint32_t tid = threadIdx.x, cap = args.capacity, G = gridDim.x, wg = blockIdx.x;
+  if (tid == 0) ready_round = 0;
   const uint32_t width = (uint32_t)d.nacc * D;
   if (args.ctrl->round != args.first_round) return;  // an earlier launch gave up: leave the count as it is
   RunB3S tr;
@@ -885,7 +890,7 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   auto fold_small = [&](const Ext<D> &r, uint32_t count) {
 #pragma unroll
     for (int t = 0; t < MAXT; t++)
-      if (t < d.T && (uint32_t)(t & 3) == wave) {
+      if (t < d.T && (uint32_t)((t + 1) & 3) == wave) {  // (the first wavefront, late from the transcript, last)
         for (uint32_t x = lane; x < count; x += 64) {
           const uint32_t *p = tail_tables + ((size_t)t * cap + 2 * x) * D;
           const Ext<D> folded = fold_ext<D>(load_ext<D>(p), load_ext<D>(p + D), r);
@@ -987,8 +992,15 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
     }
     {  // the message, the challenge, the fold
       round_message<D>(sums, (uint32_t)d.nacc, args.points, epi.mtilde, c0s + (size_t)jj * args.points * D, &epi);
-      if (tid < 64) transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi, wg == 0);
-      lds_barrier();
+      // the first wavefront publishes the challenge the moment it is drawn and finishes the transcript's step while
+      // the others, which wait for that word alone, are already folding
+      if (tid < 64) {
+        transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi, wg == 0, &ready_round);
+      } else {
+        while (__hip_atomic_load(&ready_round, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != args.first_round + jj + 1)
+          __builtin_amdgcn_s_sleep(1);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       Ext<D> r;
 #pragma unroll
       for (int c = 0; c < D; c++) r.c[c] = epi.r_mont[c];
