@@ -39,8 +39,8 @@ INT32_MUL_PEAK_PER_S = 256 * 4 * 64 / 4.7 * 2.4e9
 # the same counter reads for the plain copy kernel of `--workload copy`), and 32-bit integer multiply instructions
 # per lane and prove from the kernels' instruction streams times their trip counts (profiles/ holds both summaries).
 MEASURED = {
-    "kernel_sources_sha256": "25798b90bc808a00208308fa49982b309a94d1ff3b97bc27610242b52e854c0d",
-    "traffic": {("round_nodes_base", 24): 203430854, ("round_fold2_base", 24): 403997705},
+    "kernel_sources_sha256": "1613bf95a80d17178e51f2f030678ca66368cf43f4f3d37e2ec7c6b544cf17d0",
+    "traffic": {("round_nodes_base", 24): 203455684, ("round_fold2_base", 24): 403998986},
     "int32_mul_per_prove": 2063597568,
 }
 KERNEL_SOURCES = ["sumcheck_kernels.hpp", "field.hpp", "dev_transcript.hpp", "blake3.hpp", "stmtdesc.hpp"]
