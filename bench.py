@@ -201,12 +201,18 @@ def run_gkr(sa, steps, warmup, gold):
     wit = [sa.Table.upload(a) for a in wit_h]
     tab = [sa.Table.upload(a) for a in tab_h]
 
-    def step():
+    def one_after_the_other():
         tw, tt = sa.Transcript(g["witness_label"], d), sa.Transcript(g["table_label"], d)
         sa.prove_upper(tw, nw, 1, [tuple(wit)])
         sa.prove_upper(tt, nt, 1, [tuple(tab)])
         return tw, tt
 
+    def step():  # the two trees have a transcript each: proved side by side (exh_gkr_prove_upper_pair)
+        tw, tt = sa.Transcript(g["witness_label"], d), sa.Transcript(g["table_label"], d)
+        sa.prove_upper_pair((tw, nw, 1, [tuple(wit)]), (tt, nt, 1, [tuple(tab)]))
+        return tw, tt
+
+    dt_serial, _ = timed(sa, one_after_the_other, max(3, steps // 2), warmup)
     dt, (tw, tt) = timed(sa, step, steps, warmup)
     pinned = True
     for key, tr, n in (("witness", tw, nw), ("table", tt, nt)):
@@ -230,7 +236,8 @@ def run_gkr(sa, steps, warmup, gold):
 
     nbytes = alg(nw) + alg(nt)
     return {"workload": "LogUp-GKR: 2^22 int8-range lookups into a 2^16-entry table, witness tree n=22 + table tree "
-                        "n=16, F_p^4, prove-upper of both", "ms_per_step": 1e3 * dt, "lookups_per_s": (1 << nw) / dt,
+                        "n=16, F_p^4, prove-upper of both (side by side: two host threads, two streams)",
+            "ms_per_step": 1e3 * dt, "lookups_per_s": (1 << nw) / dt, "ms_per_step_one_after_the_other": 1e3 * dt_serial,
             "proof_bytes": len(tw.proof()) + len(tt.proof()), "proof_sha256": [sha(tw.proof()), sha(tt.proof())],
             "proof_is_the_cpu_oracles": pinned, "verifier_accepts": True,
             "timed_launches_per_step": sum(per for _, per, _ in by.values()),
@@ -463,8 +470,9 @@ def main():
                                                     "proof_is_the_cpu_oracles", "loop_hbm_fraction")}
             others[name]["roofline"] = r["roofline"]
         r = run_gkr(sa, k, 2, gold)
-        others["config4"] = {key: r[key] for key in ("workload", "ms_per_step", "lookups_per_s", "proof_sha256",
-                                                     "proof_is_the_cpu_oracles", "timed_launches_per_step", "roofline")}
+        others["config4"] = {key: r[key] for key in ("workload", "ms_per_step", "ms_per_step_one_after_the_other",
+                                                     "lookups_per_s", "proof_sha256", "proof_is_the_cpu_oracles",
+                                                     "timed_launches_per_step", "roofline")}
         r = run_commit(sa, k, 2, gold)
         others["config5"] = {key: r[key] for key in ("workload", "ms_per_step", "cap_sha256", "cap_is_the_cpu_oracles",
                                                      "roofline")}

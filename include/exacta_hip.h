@@ -14,7 +14,8 @@
  *   - every function returns EXH_OK or a negative status; exh_last_error() describes the last failure
  *     of the calling thread in the words of the reference's condition classes (src/conditions.lisp);
  *   - one context per process: every entry point takes one process-wide lock, so calls from several threads
- *     are safe and take turns (they never overlap on the device); handles are shared by all threads; every
+ *     are safe and take turns (they never overlap on the device; exh_gkr_prove_upper_pair overlaps its two
+ *     proofs itself); handles are shared by all threads; every
  *     call returns after its small result is on the host; nothing calls back into the host language.
  */
 #ifndef EXACTA_HIP_H

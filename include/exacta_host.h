@@ -75,6 +75,23 @@ int exh_stmt_evaluate(exh_stmt stmt, int degree_d, const uint32_t *table_values,
 int exh_gkr_prove_upper(exh_transcript tr, int n, int K, int lookups, const exh_table *leaves,
                         const uint8_t *label, uint64_t label_len, uint32_t *out_ri, uint32_t *out_rb,
                         uint32_t *out_cp, uint32_t *out_cq);
+/* Two PROVE-UPPER calls of the same meaning (:215-272), each with a transcript of its own (a lookup's witness
+   tree and its table tree, two lookup arguments...), run side by side: the second on a second host thread and a
+   second stream, with a workspace of its own.  Their sumchecks are chains of dependent rounds that leave most of
+   the device idle, so the pair takes about as long as the longer of the two.  Each tree's results and transcript
+   are what the single call gives (the two never touch each other's state); `status` receives each tree's own
+   result and the call returns the first that is not EXH_OK.  While launches are being timed (exh_profile_enable)
+   the two run one after the other. */
+typedef struct exh_gkr_tree {
+  exh_transcript tr;
+  int n, K, lookups;
+  const exh_table *leaves;
+  const uint8_t *label;
+  uint64_t label_len;
+  uint32_t *out_ri, *out_rb, *out_cp, *out_cq;
+  int status;
+} exh_gkr_tree;
+int exh_gkr_prove_upper_pair(exh_gkr_tree *first, exh_gkr_tree *second);
 /* VERIFY-UPPER, :91-145 */
 int exh_gkr_verify_upper(exh_transcript tr, int n, int K, int lookups, const uint8_t *label, uint64_t label_len,
                          uint32_t *out_roots, uint32_t *out_ri, uint32_t *out_rb, uint32_t *out_cp,

@@ -372,6 +372,35 @@ def prove_upper(tr, n, k, leaves, label="gkr"):
     return ri, rb, cp, cq
 
 
+class _GkrTree(C.Structure):
+    _fields_ = [("tr", C.c_uint64), ("n", C.c_int), ("K", C.c_int), ("lookups", C.c_int),
+                ("leaves", C.POINTER(C.c_uint64)), ("label", C.c_char_p), ("label_len", C.c_uint64),
+                ("out_ri", C.c_void_p), ("out_rb", C.c_void_p), ("out_cp", C.c_void_p), ("out_cq", C.c_void_p),
+                ("status", C.c_int)]
+
+
+def prove_upper_pair(first, second):
+    """Two prove-upper calls side by side (exh_gkr_prove_upper_pair): each argument is (tr, n, k, leaves) or
+    (tr, n, k, leaves, label) as for prove_upper, each with a transcript of its own.  Returns the two results."""
+    keep, trees, outs = [], [], []
+    for call in (first, second):
+        tr, n, k, leaves = call[:4]
+        label = _bytes(call[4] if len(call) > 4 else "gkr")
+        d = tr.degree
+        flat = [t for pq in leaves for t in pq]
+        L, lk = len(leaves), _block_bits(k)
+        ri, rb = np.zeros((max(n - 1, 0), d), np.uint32), np.zeros((max(lk, 0), d), np.uint32)
+        cp, cq = np.zeros((L, d), np.uint32), np.zeros((L, d), np.uint32)
+        handles = _handles(flat)
+        keep.append((handles, label, ri, rb, cp, cq))
+        address = lambda a: a.ctypes.data if a.size else None
+        trees.append(_GkrTree(tr.handle, n, k, L, C.cast(handles, C.POINTER(C.c_uint64)), label, len(label), address(ri),
+                              address(rb), address(cp), address(cq), 0))
+        outs.append((ri, rb, cp, cq))
+    check(load().exh_gkr_prove_upper_pair(C.byref(trees[0]), C.byref(trees[1])))
+    return outs[0], outs[1]
+
+
 def verify_upper(tr, n, k, lookups, label="gkr"):
     d = tr.degree
     lk = _block_bits(k)

@@ -4,6 +4,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <thread>
 
 #include "../../include/exacta_host.h"
 #include "commit.hpp"
@@ -705,6 +706,66 @@ int exh_gkr_prove_upper(exh_transcript h, int n, int K, int lookups, const exh_t
     }
   return gkr_prove_upper(*tr, n, K, lookups, ptrs.data(), std::string((const char *)label, label_len), out_ri, out_rb,
                          out_cp, out_cq);
+}
+
+namespace {
+struct TreeCall {
+  Transcript *tr = nullptr;
+  std::vector<const uint32_t *> ptrs;
+  std::string label;
+};
+int prepare_tree(const exh_gkr_tree &t, TreeCall *call) {
+  call->tr = tr_of(t.tr);
+  if (!call->tr) return E_PARAM;
+  std::vector<int> strides;
+  int status = gather_tables(t.leaves, 2 * t.lookups, call->tr->D, (uint64_t)t.K << t.n, &call->ptrs, &strides);
+  if (status) return status;
+  for (int s : strides)
+    if (s != call->tr->D) {
+      set_error("invalid-parameter: GKR leaves are extension elements");
+      return E_PARAM;
+    }
+  call->label.assign((const char *)t.label, t.label_len);
+  return OK;
+}
+int run_tree(const exh_gkr_tree &t, TreeCall &call) {
+  return gkr_prove_upper(*call.tr, t.n, t.K, t.lookups, call.ptrs.data(), call.label, t.out_ri, t.out_rb, t.out_cp,
+                         t.out_cq);
+}
+}  // namespace
+
+int exh_gkr_prove_upper_pair(exh_gkr_tree *first, exh_gkr_tree *second) {
+  ApiLock api_lock;
+  if (!first || !second || first->tr == second->tr) {
+    set_error("invalid-parameter: two trees, each with a transcript of its own");
+    return E_PARAM;
+  }
+  Context &main_context = ctx();
+  TreeCall a, b;
+  if ((first->status = prepare_tree(*first, &a))) return first->status;
+  if ((second->status = prepare_tree(*second, &b))) return second->status;
+  Context *side = nullptr;
+  int status = side_context(&side);
+  if (status) return status;
+  if (main_context.profiling) {  // (the timed launches are the library's own stream's)
+    first->status = run_tree(*first, a);
+    second->status = first->status ? first->status : run_tree(*second, b);
+    return first->status ? first->status : second->status;
+  }
+  std::string second_error;
+  main_context.share = side->share = 2;
+  std::thread worker([&] {
+    use_context(side);
+    second->status = hipSetDevice(side->device) == hipSuccess ? run_tree(*second, b) : E_DEVICE;
+    if (second->status) second_error = last_error();
+    use_context(nullptr);
+  });
+  first->status = run_tree(*first, a);
+  worker.join();
+  main_context.share = side->share = 1;
+  if (first->status) return first->status;
+  if (second->status) set_error(second_error);
+  return second->status;
 }
 
 int exh_gkr_verify_upper(exh_transcript h, int n, int K, int lookups, const uint8_t *label, uint64_t label_len,

@@ -5,8 +5,33 @@
 
 namespace exh {
 
-static Context g_ctx;
-Context &ctx() { return g_ctx; }
+static Context g_ctx, g_side;
+static thread_local Context *t_ctx = nullptr;
+Context &ctx() { return t_ctx ? *t_ctx : g_ctx; }
+void use_context(Context *c) { t_ctx = c; }
+
+static int pinned_buffer(Context &c) {
+  c.host_pinned_words = 1 << 16;
+  // coherent and mapped: a kernel writes a sumcheck's logs into it directly and the host polls for them
+  EXH_HIP(hipHostMalloc((void **)&c.host_pinned, c.host_pinned_words * 4, hipHostMallocMapped | hipHostMallocCoherent));
+  EXH_HIP(hipHostGetDevicePointer((void **)&c.host_pinned_dev, c.host_pinned, 0));
+  return OK;
+}
+
+int side_context(Context **out) {
+  int status = g_ctx.require();
+  if (status) return status;
+  Context &c = g_side;
+  if (!c.ready) {
+    EXH_HIP(hipStreamCreate(&c.stream));
+    if ((status = pinned_buffer(c))) return status;
+    c.device = g_ctx.device;
+    c.compute_units = g_ctx.compute_units;
+    c.ready = true;
+  }
+  *out = &c;
+  return OK;
+}
 
 int Arena::reserve(size_t need) {
   if (need <= bytes) return OK;
@@ -134,10 +159,10 @@ int ctx_init(int device) {
     return E_DEVICE;
   }
   EXH_HIP(hipStreamCreate(&c.stream));
-  c.host_pinned_words = 1 << 16;
-  // coherent and mapped: a kernel writes a sumcheck's logs into it directly and the host polls for them
-  EXH_HIP(hipHostMalloc((void **)&c.host_pinned, c.host_pinned_words * 4, hipHostMallocMapped | hipHostMallocCoherent));
-  EXH_HIP(hipHostGetDevicePointer((void **)&c.host_pinned_dev, c.host_pinned, 0));
+  {
+    int pinned_status = pinned_buffer(c);
+    if (pinned_status) return pinned_status;
+  }
   {  // the device address of the static scratch array, with this device current
     int scratch_status = dot_pairs_static_setup(device);
     if (scratch_status) return scratch_status;
@@ -148,8 +173,7 @@ int ctx_init(int device) {
   return OK;
 }
 
-void ctx_shutdown() {
-  Context &c = g_ctx;
+static void release_context(Context &c) {
   if (!c.ready) return;
   (void)hipStreamSynchronize(c.stream);
   c.prof_clear();
@@ -166,6 +190,11 @@ void ctx_shutdown() {
   (void)hipStreamDestroy(c.stream);
   c.stream = nullptr;
   c.ready = false;
+}
+
+void ctx_shutdown() {
+  release_context(g_side);
+  release_context(g_ctx);
 }
 
 }  // namespace exh

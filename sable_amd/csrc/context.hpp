@@ -81,10 +81,19 @@ struct Context {
   size_t host_pinned_words = 0;
   uint32_t *host_pinned_dev = nullptr;  // the same buffer as kernels address it
   uint32_t log_seq = 0;  // counts the control blocks that launches delivered to host_pinned themselves
+  // how many proofs are running side by side (see side_context): a grid whose workgroups wait for one another
+  // may take 1 / share of the device, so that the grids of all of them are resident together
+  int share = 1;
   int require();  // OK, or E_DEVICE with the reason when the library is not initialised
 };
 
+// The context of the calling thread: the library's own, unless the thread has been given another with
+// use_context.  The side context has a stream, workspace and pinned buffer of its own (no tables: handles belong to
+// the library's context), so that a second host thread can run a proof on it while the first runs one on the
+// library's; it is made on first use.
 Context &ctx();
+void use_context(Context *c);  // nullptr: back to the library's own
+int side_context(Context **out);
 int ctx_init(int device);
 void ctx_shutdown();
 

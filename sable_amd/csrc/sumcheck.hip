@@ -1,5 +1,7 @@
 // sumcheck.hip -- sumcheck session: weight tables, round launches, partial-sum reduction, folds.
 #include "sumcheck.hpp"
+
+#include <mutex>
 #include "rtc.hpp"
 #include <atomic>
 
@@ -145,8 +147,13 @@ static std::map<std::pair<std::string, int>, KernelSet> &registry() {
   static std::map<std::pair<std::string, int>, KernelSet> r;
   return r;
 }
-void register_kernels(const std::string &key, int D, KernelSet set) { registry()[{key, D}] = set; }
+static std::mutex g_registry_mutex;  // (proofs may run on two host threads: see side_context)
+void register_kernels(const std::string &key, int D, KernelSet set) {
+  std::lock_guard<std::mutex> lock(g_registry_mutex);
+  registry()[{key, D}] = set;
+}
 const KernelSet *find_kernels(const std::string &key, int D) {
+  std::lock_guard<std::mutex> lock(g_registry_mutex);
   auto it = registry().find({key, D});
   return it == registry().end() ? nullptr : &it->second;
 }
@@ -910,7 +917,9 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     uint64_t slice_max = SLICE_LDS_BYTES / ((uint64_t)T * 2 * D * 4);
     if (const char *cap = getenv("EXACTA_HIP_MAX_SLICE_PAIRS"))  // tests: keep more rounds on the streaming kernels
       slice_max = std::min<uint64_t>(slice_max, strtoull(cap, nullptr, 10));
-    const uint64_t grid_max = std::min<uint64_t>(256, c.compute_units > 0 ? c.compute_units : 1);
+    // (proofs running side by side share the device: each one's grid takes its part, a power of two)
+    const uint64_t grid_max =
+        std::min<uint64_t>(256, c.compute_units > 0 ? c.compute_units : 1) / (c.share > 1 ? 2 : 1);
     if (pow2 && n_pairs > tail_pairs(T, D) && n_pairs <= slice_max * grid_max) {
       int count = 0;
       while ((n_pairs >> count) > tail_pairs(T, D) && count < MAXTAIL && j + count < n) count++;
@@ -925,6 +934,8 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       if (count > 0 && grid > 1 && n_pairs / grid <= slice_max) {
         const uint32_t lds_bytes = (uint32_t)((uint64_t)T * (2 * n_pairs / grid) * D * 4);
         static std::map<std::pair<const void *, uint32_t>, int> asked;
+        static std::mutex asked_mutex;
+        std::lock_guard<std::mutex> asked_lock(asked_mutex);
         auto key = std::make_pair(generated ? (const void *)kernels : (const void *)(uintptr_t)D, lds_bytes);
         auto it = asked.find(key);
         if (it == asked.end()) {
@@ -932,7 +943,8 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
                                  : (D == 4 ? tail_interp_blocks_per_cu<4>(lds_bytes) : tail_interp_blocks_per_cu<8>(lds_bytes));
           it = asked.emplace(key, blocks).first;
         }
-        resident = it->second < 0 || (uint64_t)it->second * (uint64_t)std::max(c.compute_units, 1) >= grid;
+        resident = it->second < 0 ||
+                   (uint64_t)it->second * (uint64_t)std::max(c.compute_units, 1) / (uint64_t)std::max(c.share, 1) >= grid;
       }
       if (count > 0 && grid > 1 && n_pairs / grid <= slice_max && resident) {
         status = launch_tail(j, count, (uint32_t)grid, fold_due);

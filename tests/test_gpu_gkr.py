@@ -89,6 +89,51 @@ def test_the_chained_layers_and_the_host_driven_layers_send_the_same_bytes(n, lo
         p.free(), q.free()
 
 
+# two trees side by side (a second host thread, stream and workspace): each proof's bytes, outputs and final
+# transcript state are those of the call on its own; pairs of different sizes, both chained, one host-driven
+# (several blocks), both large enough for the grids of slices that must share the device
+PAIRS = [((13, 1, 1, 4), (9, 1, 1, 4)), ((16, 1, 1, 4), (15, 1, 2, 4)), ((6, 3, 2, 4), (12, 1, 1, 4)),
+         ((7, 1, 1, 8), (3, 1, 1, 4)), ((17, 1, 1, 4), (17, 1, 1, 4))]
+
+
+@pytest.mark.parametrize("first,second", PAIRS)
+def test_two_trees_side_by_side_are_the_two_single_calls(first, second):
+    rng = np.random.default_rng(sum(first) + 3 * sum(second))
+    calls, alone = [], []
+    for which, (n, k, lookups, d) in enumerate((first, second)):
+        leaves = random_leaves(rng, lookups, n, k, d)
+        dev = [(sa.Table.upload(p), sa.Table.upload(q)) for p, q in leaves]
+        label = "tree-%d" % which
+        tr = sa.Transcript(label, d)
+        alone.append((tr, sa.prove_upper(tr, n, k, dev)))
+        calls.append((sa.Transcript(label, d), n, k, dev))
+    for _ in range(2):  # (the second time with the side context's buffers already there)
+        fresh = [(sa.Transcript("tree-%d" % which, c[0].degree),) + c[1:] for which, c in enumerate(calls)]
+        outs = sa.prove_upper_pair(fresh[0], fresh[1])
+        for (tr, want), call, got in zip(alone, fresh, outs):
+            assert call[0].proof() == tr.proof()
+            for a, b in zip(got, want):
+                assert same(a, b)
+    # the transcripts go on identically after the proofs
+    a = sa.Transcript("tree-0", calls[0][0].degree)
+    b = sa.Transcript("tree-0", calls[0][0].degree)
+    sa.prove_upper(a, *calls[0][1:])
+    sa.prove_upper_pair((b,) + calls[0][1:], (sa.Transcript("tree-1", calls[1][0].degree),) + calls[1][1:])
+    assert same(a.challenge(), b.challenge())
+    for c in calls:
+        for p, q in c[3]:
+            p.free(), q.free()
+
+
+def test_a_pair_needs_two_transcripts():
+    rng = np.random.default_rng(5)
+    leaves = random_leaves(rng, 1, 3, 1, 4)
+    dev = [(sa.Table.upload(p), sa.Table.upload(q)) for p, q in leaves]
+    tr = sa.Transcript("gkr-test", 4)
+    with pytest.raises(sa.ExactaError):
+        sa.prove_upper_pair((tr, 3, 1, dev), (tr, 3, 1, dev))
+
+
 def test_verify_upper_rejects_forgeries():
     n, k, lookups, d = 3, 3, 2, 4
     rng = np.random.default_rng(9)
