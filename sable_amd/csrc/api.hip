@@ -752,6 +752,14 @@ int exh_gkr_prove_upper_pair(exh_gkr_tree *first, exh_gkr_tree *second) {
     second->status = first->status ? first->status : run_tree(*second, b);
     return first->status ? first->status : second->status;
   }
+  {  // what the library's stream still has to do (the second tree's leaves, perhaps) comes first on the other too
+    hipEvent_t queued;
+    EXH_HIP(hipEventCreateWithFlags(&queued, hipEventDisableTiming));
+    hipError_t recorded = hipEventRecord(queued, main_context.stream);
+    if (recorded == hipSuccess) recorded = hipStreamWaitEvent(side->stream, queued, 0);
+    (void)hipEventDestroy(queued);
+    EXH_HIP(recorded);
+  }
   std::string second_error;
   main_context.share = side->share = 2;
   std::thread worker([&] {

@@ -38,8 +38,8 @@ struct Arena {
 
 // Device buffers that are reused instead of returned to the driver: tables and per-proof buffers are
 // allocated and freed around every call, and hipMalloc / hipFree cost more than the kernels between
-// them.  Everything runs on the library's one stream, so a buffer given out again is safe to write
-// as soon as the earlier work queued on it has run: no wait on release.
+// them.  Everything a context does runs on its one stream and every context has a pool of its own, so a
+// buffer given out again is safe to write as soon as the earlier work queued on it has run: no wait on release.
 struct Pool {
   std::multimap<size_t, void *> idle;  // by size
   std::map<void *, size_t> sizes;      // every buffer the pool owns, live or idle
