@@ -112,14 +112,15 @@ static int get_domain(int n, Domain **out) {
 // the strided gathers fall on distinct banks.
 // A tile is 2^12 elements, 16 per thread: a domain of 2^24 takes three passes (6 + 5 + 12 stages) with
 // global segments of at least 64 words.
-// The butterflies run in double precision (field.hpp), whose fused multiply-add issues at four times the rate of
-// a 32-bit integer multiply: a product by a twiddle is six operations and leaves a residue within about p/2 of
-// zero, and the sum and the difference that follow are one operation each with no reduction, exact as long as
-// the values stay integers below 2^53: a tile's elements start below p and grow by less than 0.57 p per stage,
-// so after a pass's twelve stages at most they are below 8 p, and a product with a twiddle below 2^65.  The tile
-// in LDS therefore holds doubles; a pass ends by writing canonical residues.  The passes are bound by their
-// instructions all the same (the vector units about three quarters busy, some 330 instructions per thread and
-// round of four stages): both columns of 2^24 take 64 + 56 + 92 us, against 300 us with Montgomery products.
+// The butterflies run in double precision (field.hpp), eight instructions each where Montgomery arithmetic takes
+// about twenty (the multiplies issue at the same rate either way): a product by a twiddle is six operations and
+// leaves a residue within about p/2 of zero, and the sum and the difference that follow are one operation each
+// with no reduction, exact as long as the values stay integers below 2^53: a tile's elements start below p and
+// grow by less than 0.57 p per stage, so after a pass's twelve stages at most they are below 8 p, and a product
+// with a twiddle below 2^65.  The tile in LDS therefore holds doubles; a pass ends by writing canonical residues.
+// The passes are bound by their instructions all the same (some 330 per thread and round of four stages, the
+// vector units busy nine tenths of the time): both columns of 2^24 take 64 + 56 + 92 us, against 300 us with
+// Montgomery products and the tile fetched word by word.
 constexpr int NTT_TILE_BITS = 12;
 constexpr int NTT_BLOCK = 256;
 constexpr int NTT_MAX_UPPER_STAGES = 7;  // per pass above the last: segments of 2^(12-7) words at least
