@@ -31,6 +31,36 @@ __global__ __launch_bounds__(BLOCK) void gkr_reduce_kernel(const uint32_t *p, co
   store_ext<D>(qq + o * D, ext_mul_mont<D>(q0, q1r));
 }
 
+// The layers m_top .. 0 of one lookup's tree with one block, in one workgroup: layer m has 2^m <= BLOCK parents,
+// a thread takes one, and the workgroup's barrier stands between a layer's writes and the next one's reads.  (A
+// launch per layer is 4 us each for a few hundred products.)
+constexpr int REDUCE_TOP_LAYERS = 9;  // m_top <= 8: 256 parents
+struct ReduceTopArgs {
+  const uint32_t *p, *q;  // layer m_top + 1
+  uint32_t *pp[REDUCE_TOP_LAYERS], *qq[REDUCE_TOP_LAYERS];
+  int m_top;
+};
+template <int D>
+__global__ __launch_bounds__(BLOCK) void gkr_reduce_top_kernel(ReduceTopArgs a) {
+  static_assert((1 << (REDUCE_TOP_LAYERS - 1)) <= BLOCK, "a thread per parent");
+  const uint32_t *p = a.p, *q = a.q;
+  for (int m = a.m_top; m >= 0; m--) {
+    const uint32_t o = threadIdx.x, half = 1u << m;
+    if (o < half) {
+      Ext<D> p0 = load_ext<D>(p + o * D), p1 = load_ext<D>(p + (o + half) * D);
+      Ext<D> q0 = load_ext<D>(q + o * D), q1 = load_ext<D>(q + (o + half) * D);
+      Ext<D> q1r, q0r;
+#pragma unroll
+      for (int c = 0; c < D; c++) q1r.c[c] = mont_mul(q1.c[c], R2), q0r.c[c] = mont_mul(q0.c[c], R2);
+      store_ext<D>(a.pp[m] + o * D, ext_add<D>(ext_mul_mont<D>(p0, q1r), ext_mul_mont<D>(p1, q0r)));
+      store_ext<D>(a.qq[m] + o * D, ext_mul_mont<D>(q0, q1r));
+    }
+    __threadfence();
+    __syncthreads();
+    p = a.pp[m], q = a.qq[m];
+  }
+}
+
 int gkr_reduce_layer(int D, int K, int m, const uint32_t *p, const uint32_t *q, uint32_t *pp, uint32_t *qq) {
   Context &c = ctx();
   int status = c.require();
@@ -477,15 +507,30 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
   // one allocation holds every layer above the leaves: 2 L K (2^n - 1) entries
   if ((status = c.tree.reserve(((((uint64_t)K << n) - K) * 2 * L * D + 64) * 4))) return status;
   uint32_t *next = (uint32_t *)c.tree.ptr;
+  const int m_top = K == 1 ? std::min(n - 1, REDUCE_TOP_LAYERS - 1) : -1;  // these layers in one launch per lookup
   for (int m = n - 1; m >= 0; m--)
     for (int l = 0; l < L; l++) {
       uint64_t words = ((uint64_t)K << m) * D;
       uint32_t *pp = next, *qq = next + words;
       next += 2 * words;
-      if ((status = gkr_reduce_layer(D, K, m, layers[m + 1][2 * l], layers[m + 1][2 * l + 1], pp, qq))) return status;
+      if (m > m_top &&
+          (status = gkr_reduce_layer(D, K, m, layers[m + 1][2 * l], layers[m + 1][2 * l + 1], pp, qq)))
+        return status;
       layers[m][2 * l] = pp;
       layers[m][2 * l + 1] = qq;
     }
+  for (int l = 0; l < L && m_top >= 0; l++) {
+    ReduceTopArgs a;
+    memset(&a, 0, sizeof(a));
+    a.p = layers[m_top + 1][2 * l], a.q = layers[m_top + 1][2 * l + 1], a.m_top = m_top;
+    for (int m = m_top; m >= 0; m--)
+      a.pp[m] = const_cast<uint32_t *>(layers[m][2 * l]), a.qq[m] = const_cast<uint32_t *>(layers[m][2 * l + 1]);
+    if (D == 4)
+      hipLaunchKernelGGL(gkr_reduce_top_kernel<4>, dim3(1), dim3(BLOCK), 0, c.stream, a);
+    else
+      hipLaunchKernelGGL(gkr_reduce_top_kernel<8>, dim3(1), dim3(BLOCK), 0, c.stream, a);
+    EXH_HIP(hipGetLastError());
+  }
   {  // one block: the layers chained on the device, one wait for the whole proof
     const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS"), *no_chain = getenv("EXACTA_HIP_NO_GKR_CHAIN");
     const bool off = (host_rounds && host_rounds[0] == '1') || (no_chain && no_chain[0] == '1');
