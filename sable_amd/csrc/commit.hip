@@ -125,6 +125,7 @@ constexpr int NTT_TILE_BITS = 12;
 constexpr int NTT_BLOCK = 256;
 constexpr int NTT_MAX_UPPER_STAGES = 7;  // per pass above the last: segments of 2^(12-7) words at least
 static_assert(NTT_TILE_BITS <= 12, "a pass's stages, the bound on the lazily reduced values");
+static_assert((1 << NTT_TILE_BITS) == 16 * NTT_BLOCK, "a thread moves a whole tile's sixteen words as four vectors");
 __device__ __forceinline__ uint32_t ntt_pad(uint32_t e) { return e + (e >> 4); }
 constexpr uint32_t ntt_lds_bytes(int tile_bits) {
   return (((uint32_t)1 << tile_bits) + ((uint32_t)1 << tile_bits >> 4) + 1) * 8;
