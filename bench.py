@@ -29,10 +29,16 @@ sys.path.insert(0, ROOT)
 from sable_amd import workloads as wl  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# The integer-multiply roofline's peak: one 32-bit multiply (v_mad_u64_u32, v_mul_lo_u32, v_mul_hi_u32) per lane
-# every 4.7 cycles of a SIMD's 16 lanes x 4, as measured with independent chains on this part at 2.4 GHz:
-# 256 CUs x 4 SIMDs x 64 lanes / 4.7 cycles x 2.4e9
-INT32_MUL_PEAK_PER_S = 256 * 4 * 64 / 4.7 * 2.4e9
+# The integer-multiply roofline's peak is measured by `--workload mulrate` (run_mulrate below; the issue-rate
+# kernel of sable_amd/csrc/issue_rate.hip): lanes x SIMDs x compute units x clock / cycles per wavefront instruction
+# of v_mad_u64_u32 with many wavefronts resident.  profiles/mulrate_kernel_stats.md holds the run this default is from.
+MULRATE_DEFAULT = {"cycles_per_wave_instruction": 4.7, "clock_ghz": 2.4, "compute_units": 256}
+
+
+def int32_mul_peak(rate=None):
+    r = rate or MULRATE_DEFAULT
+    return r["compute_units"] * 4 * 64 / r["cycles_per_wave_instruction"] * r["clock_ghz"] * 1e9
+
 
 # Figures that were measured on one version of the kernels and are only reported while the kernels' sources are
 # that version: HBM bytes per launch from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE, each scaled by what
@@ -373,6 +379,41 @@ def cpu_baseline(sa, n_one, n_all, best_of=7):
                 "reference off its base-field kernel, so its real time is higher)": "6.6 s"}}
 
 
+def run_mulrate(sa, iterations=4096):
+    """Issue rates of the VALU instructions the kernels are made of (the peak the integer-multiply figure is a
+    fraction of).  Per instruction: cycles per wavefront instruction and SIMD with
+    8 workgroups per compute unit of 8 independent chains (issue rate), with one wavefront per SIMD and 8 chains
+    (what a lone wavefront can issue), and with one wavefront per SIMD and one chain (dependent latency)."""
+    lib = sa.load()
+    rows = []
+    clock_khz, cus = C.c_int(), C.c_int()
+    for op in range(lib.exh_issue_rate_ops()):
+        row = {}
+        for key, chains, wg_per_cu in (("issue", 8, 8), ("lone_wave", 8, 1), ("dependent", 1, 1)):
+            name = C.create_string_buffer(64)
+            ms, ipw = C.c_float(), C.c_double()
+            # the compute-unit count comes back from the first call; 256 on this part
+            groups = wg_per_cu * (cus.value or 256)
+            sa.check(lib.exh_issue_rate(op, chains, groups, iterations, name, 64, C.byref(ms), C.byref(ipw),
+                                        C.byref(clock_khz), C.byref(cus)))
+            groups_now = wg_per_cu * cus.value
+            if groups_now != groups:  # first call on a part with another count: measure again at the right grid
+                sa.check(lib.exh_issue_rate(op, chains, groups_now, iterations, name, 64, C.byref(ms), C.byref(ipw),
+                                            C.byref(clock_khz), C.byref(cus)))
+            waves_per_simd = wg_per_cu  # a workgroup of 256 threads puts one wavefront on each of a unit's 4 SIMDs
+            cycles = ms.value * 1e-3 * clock_khz.value * 1e3 / (ipw.value * waves_per_simd)
+            row["instruction"] = name.value.decode()
+            row[key + "_cycles"] = round(cycles, 3)
+            row[key + "_ms"] = round(ms.value, 4)
+        rows.append(row)
+    mad = next(r for r in rows if r["instruction"] == "v_mad_u64_u32")
+    rate = {"cycles_per_wave_instruction": mad["issue_cycles"], "clock_ghz": clock_khz.value / 1e6,
+            "compute_units": cus.value}
+    return {"workload": "VALU issue rates: chains of one instruction, 256 threads per workgroup", "iterations": iterations,
+            "clock_khz": clock_khz.value, "compute_units": cus.value, "rates": rows,
+            "int32_mul_peak_per_s": int32_mul_peak(rate), "int32_mul_rate": rate}
+
+
 def run_copy(steps):
     """Calibration for the traffic counters: an elementwise kernel that reads 256 MiB and writes 256 MiB."""
     import torch
@@ -402,7 +443,8 @@ SEEDED = "synthetic (SplitMix64-seeded uniform field elements)"
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="config2",
-                    choices=["config1", "config2", "config3", "config4", "config5", "combine", "combine128", "copy"],
+                    choices=["config1", "config2", "config3", "config4", "config5", "combine", "combine128", "copy",
+                             "mulrate"],
                     help="config2 (default) is the headline; the others are the remaining configured workloads; "
                          "copy is the known-size kernel the traffic counters are calibrated on")
     ap.add_argument("--gpus", type=int, default=1)
@@ -439,6 +481,11 @@ def main():
         print(json.dumps(line("BaseFold commit ms (config 5)", res["ms_per_step"], "ms", False,
                               "u32 (Montgomery KoalaBear) + BLAKE3", SEEDED, res, steps, warmup)))
         return
+    if args.workload == "mulrate":
+        res = run_mulrate(sa)
+        print(json.dumps({"metric": "int32 multiply issue peak", "value": res["int32_mul_peak_per_s"],
+                          "unit": "32-bit multiplies/s (per lane)", "n_gpus": 1, "config": res}))
+        return
     if args.workload in ("combine", "combine128"):
         res = run_combine(sa, steps, warmup, 128 if args.workload == "combine128" else 2)
         print(json.dumps(line("combine-columns entries/s (config 5's columns)", res["column_entries_per_s"],
@@ -454,10 +501,12 @@ def main():
                "u32 (Montgomery KoalaBear, F_p^4 tower; exact integers in f64 for the first sweep's products)", SEEDED,
                res, steps, warmup)
     muls = MEASURED["int32_mul_per_prove"] if current and res["n"] == 24 else None
-    out["int32_mul"] = {"bound": "int32 multiply issue", "multiplies_per_step": muls, "peak": INT32_MUL_PEAK_PER_S,
+    rate = run_mulrate(sa, 1024)["int32_mul_rate"]  # measured in this run
+    peak = int32_mul_peak(rate)
+    out["int32_mul"] = {"bound": "int32 multiply issue", "multiplies_per_step": muls, "peak": peak, "peak_from": rate,
                         "unit": "32-bit multiplies/s (per lane)",
                         "achieved": muls / (res["ms_per_step"] * 1e-3) if muls else None,
-                        "frac": muls / (res["ms_per_step"] * 1e-3) / INT32_MUL_PEAK_PER_S if muls else None,
+                        "frac": muls / (res["ms_per_step"] * 1e-3) / peak if muls else None,
                         "note": "counts are from the kernels' instruction streams and go with one version of the "
                                 "sources (null when they have changed since)"}
     out["cpu_baseline"] = cpu_baseline(sa, args.cpu_n, min(args.cpu_n + 2, 24)) if args.cpu_n > 0 else None

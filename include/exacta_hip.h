@@ -70,6 +70,16 @@ int exh_profile_enable(int on);
 int exh_profile_count(void);
 int exh_profile_entry(int index, char *name, int name_cap, int *round, float *ms, uint64_t *alg_bytes);
 
+/* The second roofline's peak, measured (no counterpart in the reference): one launch of `workgroups` workgroups of
+   256 threads, every lane running `chains` (8: independent chains, the issue rate; 1: one dependent chain, the
+   latency a lone wavefront sees) of the VALU instruction number `op` (0 .. exh_issue_rate_ops() - 1; `name`
+   receives its mnemonic) for iterations * 8 links.  Out: the launch's duration, the machine instructions each
+   wavefront issued, the device's clock and compute units -- cycles per wavefront instruction and SIMD =
+   ms * clock / (instructions_per_wave * wavefronts per SIMD). */
+int exh_issue_rate_ops(void);
+int exh_issue_rate(int op, int chains, int workgroups, int iterations, char *name, int name_cap, float *ms,
+                   double *instructions_per_wave, int *clock_khz, int *compute_units);
+
 /* ---- tables: MAKE-TABLE and the read-back at the end of PROVE (src/sumcheck.lisp:61-70, 564-571) */
 int exh_table_upload(const uint32_t *host, uint64_t n_u32, int stride, exh_table *out);
 int exh_table_alloc(uint64_t n_u32, int stride, exh_table *out);

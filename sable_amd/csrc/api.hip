@@ -106,6 +106,24 @@ int exh_synchronize(void) {
   return OK;
 }
 
+// ---- issue-rate measurement (issue_rate.hip)
+int exh_issue_rate_ops(void) { return issue_rate_ops(); }
+int exh_issue_rate(int op, int chains, int workgroups, int iterations, char *name, int name_cap, float *ms,
+                   double *instructions_per_wave, int *clock_khz, int *compute_units) {
+  ApiLock api_lock;
+  const char *op_name = nullptr;
+  float t = 0;
+  int status = issue_rate(op, chains, workgroups, iterations, &op_name, &t, instructions_per_wave, clock_khz,
+                          compute_units);
+  if (status) return status;
+  if (ms) *ms = t;
+  if (name && name_cap > 0 && op_name) {
+    strncpy(name, op_name, name_cap - 1);
+    name[name_cap - 1] = 0;
+  }
+  return OK;
+}
+
 int exh_profile_enable(int on) {
   ApiLock api_lock;
   Context &c = ctx();

@@ -97,4 +97,9 @@ int side_context(Context **out);
 int ctx_init(int device);
 void ctx_shutdown();
 
+// issue_rate.hip: one timed launch of independent (or dependent) chains of one VALU instruction
+int issue_rate(int op, int chains, int workgroups, int iterations, const char **name, float *ms,
+               double *instructions_per_wave, int *clock_khz, int *compute_units);
+int issue_rate_ops();
+
 }  // namespace exh

@@ -98,6 +98,9 @@ __global__ __launch_bounds__(BLOCK) void halves_kernel(const uint32_t *v, uint32
 struct GkrChainState {
   DevB3S tr;                       // the transcript between launches
   uint32_t point[MAXROUNDS + 1][8];  // the next layer's eq point (canonical)
+  // sticky: a chained layer's sumcheck did not complete (a workgroup of a grid launch gave up, or the control
+  // block does not count the layer's rounds); the host reads it after its one wait and voids the proof
+  uint32_t failed;
 };
 
 constexpr int GLUE_MAXCONST = 8;  // constants of a layer statement the launch can form: a_l and a_l lambda, l < 4
@@ -156,6 +159,7 @@ __global__ __launch_bounds__(64) void gkr_glue_kernel(GlueArgs<D> a) {
     const int R = a.prev_rounds, mw = a.prev_points * D;
     uint32_t *log_msg = a.log, *log_chal = log_msg + R * mw, *log_fin = log_chal + R * D, *log_tt = log_fin + a.NT * D;
     if (a.close_kind == 2) {
+      if (lane == 0 && (a.prev_ctrl->gave_up != 0 || a.prev_ctrl->round != (uint32_t)R)) a.chain->failed = 1;
       for (int u = lane; u < R * mw; u += 64) log_msg[u] = a.prev_ctrl->msg[u / mw][u % mw];
       for (int u = lane; u < R * D; u += 64) {
         const uint32_t v = a.prev_ctrl->chal[u / D][u % D];
@@ -331,6 +335,14 @@ struct DeviceBuffers {  // frees what it allocated when the proof ends
 };
 
 
+// what the chain's sticky word means for the proof (host side)
+int chain_outcome(uint32_t failed) {
+  if (!failed) return OK;
+  set_error("device-error: a chained layer's sumcheck did not complete (a workgroup gave up waiting, or rounds are "
+            "missing); the proof is void");
+  return E_DEVICE;
+}
+
 // PROVE-UPPER's in-block layers with one block, chained on the device (see gkr_glue_kernel): every launch of every
 // layer's sumcheck is enqueued at once, the host waits once and reads the log.
 template <int D>
@@ -366,6 +378,8 @@ static int prove_upper_chained(Transcript &tr, int n, int L, const std::vector<s
   }
   const DevB3S first = device_state(tr);
   EXH_HIP(hipMemcpyAsync(&chain->tr, &first, sizeof(first), hipMemcpyHostToDevice, c.stream));
+  // (a fill kernel would do as well; the chain is never captured into a graph)
+  EXH_HIP(hipMemsetAsync(&chain->failed, 0, sizeof(chain->failed), c.stream));
   const std::vector<int> strides(NT, D);
   const std::vector<uint32_t> no_point((size_t)n * D, 0), no_consts((size_t)2 * L * D, 0);
   auto layer_tables = [&](int layer) {  // with one block the halves are views (LAYER-TABLES, src/gkr.lisp:199-206)
@@ -452,9 +466,12 @@ static int prove_upper_chained(Transcript &tr, int n, int L, const std::vector<s
   // ---- one wait, then the log
   std::vector<uint32_t> log(words);
   DevB3S last;
+  uint32_t failed = 0;
   EXH_HIP(hipMemcpyAsync(log.data(), d_log, words * 4, hipMemcpyDeviceToHost, c.stream));
   EXH_HIP(hipMemcpyAsync(&last, &chain->tr, sizeof(last), hipMemcpyDeviceToHost, c.stream));
+  EXH_HIP(hipMemcpyAsync(&failed, &chain->failed, sizeof(failed), hipMemcpyDeviceToHost, c.stream));
   EXH_HIP(hipStreamSynchronize(c.stream));
+  if ((status = chain_outcome(failed))) return status;
   // the messages as they were sent, recorded without hashing them again; the transcript takes the device's state
   uint64_t dims[2] = {2, (uint64_t)D};
   for (int l = 0; l < L; l++)

@@ -58,16 +58,18 @@ EXH_DESC_FN constexpr int node_slots(const Desc &d) {
 }
 
 // the launches per round of the base-field sweep for degree D and the slots each takes: the slots are split
-// evenly over launches of at most 10 (F_p^4) or 4 (F_p^8) slots, what two wavefronts per SIMD have the
-// registers for; no launches when the slot sums do not fit the accumulators' buffers
+// evenly over launches of at most NODES_CAP4 (F_p^4) or NODES_CAP8 (F_p^8) slots, what two wavefronts per SIMD
+// have the registers for at two registers a slot and coordinate; no launches when the slot sums do not fit the
+// accumulators' buffers
+constexpr int NODES_CAP4 = 20, NODES_CAP8 = 8;
 template <class Desc>
 EXH_DESC_FN constexpr int nodes_slots_per_pass(const Desc &d, int D) {
-  int slots = node_slots(d), cap = D == 4 ? 10 : 4, passes = (slots + cap - 1) / cap;
+  int slots = node_slots(d), cap = D == 4 ? NODES_CAP4 : NODES_CAP8, passes = (slots + cap - 1) / cap;
   return (slots + passes - 1) / passes;
 }
 template <class Desc>
 EXH_DESC_FN constexpr int nodes_launches(const Desc &d, int D) {
-  int slots = node_slots(d), cap = D == 4 ? 10 : 4;
+  int slots = node_slots(d), cap = D == 4 ? NODES_CAP4 : NODES_CAP8;
   return (slots + cap - 1) / cap;
 }
 

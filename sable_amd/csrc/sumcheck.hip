@@ -11,6 +11,7 @@
 
 #include "context.hpp"
 #include "hostfield.hpp"
+#include "interp.hpp"
 
 namespace exh {
 
@@ -105,43 +106,8 @@ __global__ __launch_bounds__(BLOCK) void reduce_partials_kernel(const uint32_t *
   }
 }
 
-// the interpreter's launchers
-template <int D>
-static void launch_interp(const RoundArgs<D> &a, const StmtDesc &d, bool in_base, bool fold, uint32_t grid,
-                          hipStream_t s) {
-  if (in_base && fold)
-    hipLaunchKernelGGL((round_kernel_interp<D, true, true>), dim3(grid), dim3(BLOCK), 0, s, a, d);
-  else if (in_base)
-    hipLaunchKernelGGL((round_kernel_interp<D, true, false>), dim3(grid), dim3(BLOCK), 0, s, a, d);
-  else if (fold)
-    hipLaunchKernelGGL((round_kernel_interp<D, false, true>), dim3(grid), dim3(BLOCK), 0, s, a, d);
-  else
-    hipLaunchKernelGGL((round_kernel_interp<D, false, false>), dim3(grid), dim3(BLOCK), 0, s, a, d);
-}
-
-template <int D>
-static void launch_tail_interp(const TailArgs<D> &a, const StmtDesc &d, uint32_t grid, hipStream_t s) {
-  static bool large_lds = false;
-  if (a.lds_bytes > TAIL_LDS_BYTES && !large_lds) {
-    (void)hipFuncSetAttribute((const void *)tail_kernel_interp<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              SLICE_LDS_BYTES);
-    large_lds = true;
-  }
-  hipLaunchKernelGGL((tail_kernel_interp<D>), dim3(grid), dim3(BLOCK), a.lds_bytes, s, a, d);
-}
-
-template <int D>
-static int tail_interp_blocks_per_cu(uint32_t lds_bytes) {
-  if (lds_bytes > TAIL_LDS_BYTES)
-    (void)hipFuncSetAttribute((const void *)tail_kernel_interp<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              SLICE_LDS_BYTES);
-  int blocks = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, (const void *)tail_kernel_interp<D>, BLOCK, lds_bytes) !=
-      hipSuccess)
-    return -1;
-  return blocks;
-}
-
+// the interpreter's launchers live in interp.hip (one translation unit per degree and kind: they are the
+// slowest kernels of the library to compile)
 // ------------------------------------------------------------------ registry of generated kernels
 static std::map<std::pair<std::string, int>, KernelSet> &registry() {
   static std::map<std::pair<std::string, int>, KernelSet> r;
@@ -162,6 +128,7 @@ const KernelSet *find_kernels(const std::string &key, int D) {
 // regions of the context's pinned host buffer (in words): per-round results | the session's eq point
 // and block weights | the device loop's constants | the device loop's logs and final tables
 constexpr uint32_t SLICE_GROUPS = 16;  // rows of totals per round of a grid launch of LDS-resident slices
+constexpr uint32_t ROUND_GROUPS = 32;  // rows of totals of a streaming round (its workgroups' atomics spread over them)
 constexpr size_t PIN_BEGIN = 16384, PIN_BEGIN_WORDS = 4096;
 constexpr size_t PIN_LOOP = PIN_BEGIN + PIN_BEGIN_WORDS, PIN_LOOP_WORDS = 12288;
 constexpr size_t PIN_DOWN = PIN_LOOP + PIN_LOOP_WORDS, PIN_DOWN_WORDS = 32768;
@@ -291,6 +258,14 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   words += words & 1;  // the 64-bit totals of the grid launch of slices: [MAXTAIL][SLICE_GROUPS][pstride]
   const uint64_t slice_totals_off = words;
   words += (uint64_t)2 * MAXTAIL * SLICE_GROUPS * pstride;
+  // the streaming rounds' own totals ([round][ROUND_GROUPS][pstride] 64-bit words) and arrival counters follow, so
+  // that the set-up kernel clears them all in one go
+  const uint64_t round_totals_off = words;
+  words += (uint64_t)2 * std::max(n, 1) * ROUND_GROUPS * pstride;
+  const uint64_t arrivals_off = words;
+  words += (uint64_t)std::max(n, 1) + 1;
+  words += words & 1;
+  zeroed_words = words - slice_totals_off;
   // mixed base / extension inputs: lift the base ones
   bool any_base = false, all_base = true;
   for (int t = 0; t < T; t++) {
@@ -313,6 +288,8 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   d_partials = base + partial_off;
   d_sums = d_partials + partial_rows * (uint64_t)pstride;
   d_slice_totals = reinterpret_cast<unsigned long long *>(base + slice_totals_off);
+  d_round_totals = reinterpret_cast<unsigned long long *>(base + round_totals_off);
+  d_arrivals = base + arrivals_off;
   d_ctrl = reinterpret_cast<Ctrl *>(base + ctrl_off);
   d_mtilde = base + mt_off;
   d_c0 = base + c0_off;
@@ -428,7 +405,7 @@ int SumcheckSession::launch_setup() {
   memcpy(&eqt, setup.eqt, sizeof(eqt));
   // a session whose first round fits the one-workgroup launch never takes the grid launch
   uint32_t *zero = reinterpret_cast<uint32_t *>(d_slice_totals);
-  uint64_t zero_words = size / 2 > tail_pairs(st.T(), D) ? (uint64_t)2 * MAXTAIL * SLICE_GROUPS * pstride : 0;
+  uint64_t zero_words = size / 2 > tail_pairs(st.T(), D) ? zeroed_words : 0;
   const uint32_t zero_grid = (uint32_t)((zero_words + 4 * BLOCK - 1) / (4 * BLOCK));  // four words a thread
   bool cleared = false;
   if (setup.total_eq) {
@@ -486,9 +463,26 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   a.pstride = s.pstride;
   a.double_fold = double_fold ? 1 : 0;
   if (s.device_loop) a.ctrl = s.d_ctrl;
+  uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
+  const bool own_epilogue = do_sums && s.device_loop && s.st.nacc > 0;
+  if (own_epilogue) {
+    // as many rows of totals as the elected workgroup's polls and scratch cover
+    const uint32_t width = (uint32_t)s.st.nacc * D;
+    uint32_t groups = 1;
+    while (groups * 2 <= ROUND_GROUPS && groups * 2 <= grid && groups * 2 * width <= MAXPTS * MAXACC * 8 &&
+           groups * 2 * width <= (uint32_t)TOTALS_POLLS * BLOCK)
+      groups *= 2;
+    a.totals = s.d_round_totals + (size_t)j * ROUND_GROUPS * s.pstride;
+    a.arrivals = s.d_arrivals + j;
+    a.groups = groups, a.points = (uint32_t)s.points, a.spin_limit = 200000;
+    a.mtilde = s.d_mtilde, a.c0 = s.d_c0 + (size_t)j * s.points * D;
+    if (!s.slice_totals_clear) {  // no set-up kernel cleared them
+      EXH_HIP(hipMemsetAsync(a.totals, 0, (size_t)ROUND_GROUPS * s.pstride * 8, c.stream));
+      EXH_HIP(hipMemsetAsync(a.arrivals, 0, 4, c.stream));
+    }
+  }
   if (fold && !s.device_loop)
     for (int k = 0; k < D; k++) a.r_mont[k] = to_mont(s.pending_r[k]);
-  uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
   {
     // bytes this launch must move: every table read once, the folded tables written once
     uint64_t in_words = (double_fold ? 8 : fold ? 4 : 2) * n_pairs * (s.cur_base ? 1 : D),
@@ -505,7 +499,7 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   else
     launch_interp<D>(a, s.desc, s.cur_base, fold, grid, c.stream);
   c.prof_end();
-  if (do_sums && s.device_loop) {
+  if (do_sums && s.device_loop && !own_epilogue) {
     EpilogueArgs e;
     e.partials = s.d_partials, e.nblocks = grid, e.pstride = s.pstride, e.nacc = (uint32_t)s.st.nacc;
     e.points = (uint32_t)s.points, e.mtilde = s.d_mtilde, e.c0 = s.d_c0 + (size_t)j * s.points * D, e.ctrl = s.d_ctrl;
@@ -556,17 +550,10 @@ static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs) {
   while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > s.max_grid) ppt *= 2;
   a.pairs_per_thread = ppt;
   a.deferred = (uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits) ? 1 : 0;
-  a.partials = s.d_partials;
-  a.pstride = s.pstride;
   uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
-  for (int pass = 0; pass < s.kernels->nodes_passes; pass++) {
-    c.prof_begin("round_nodes_base", 0, (uint64_t)T * 16 * n_pairs);
-    s.kernels->launch_nodes(&a, pass, grid, c.stream);
-    c.prof_end();
-  }
-  NodesEpilogueArgs e;
-  memset(&e, 0, sizeof(e));
-  e.e.partials = s.d_partials, e.e.nblocks = grid, e.e.pstride = s.pstride, e.e.nacc = (uint32_t)s.st.nacc;
+  // the two rounds' epilogue, run by the last workgroup of the last pass (see RoundTotals)
+  NodesEpilogueArgs &e = a.epi;
+  e.e.partials = nullptr, e.e.nblocks = grid, e.e.pstride = s.pstride, e.e.nacc = (uint32_t)s.st.nacc;
   e.e.points = (uint32_t)s.points, e.e.mtilde = s.d_mtilde, e.e.c0 = s.d_c0;
   e.e.ctrl = s.d_ctrl;
   e.eq1 = s.has_eq ? s.d_weights + (size_t)2 * D : nullptr;  // the eq factors lead the arena: (w_v, 1 - w_v) per variable
@@ -576,12 +563,26 @@ static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs) {
     for (int k = 0; k < s.desc.nev[g]; k++) e.ev[g][k] = (uint8_t)s.desc.ev[g][k];
   }
   fill_inv_den(e.inv_den);
-  c.prof_begin("epilogue", 0, 0);
-  if (D == 4)
-    hipLaunchKernelGGL(nodes_epilogue_kernel<4>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
-  else
-    hipLaunchKernelGGL(nodes_epilogue_kernel<8>, dim3(1), dim3(EPI_BLOCK), 0, c.stream, e);
-  c.prof_end();
+  {
+    const uint32_t width = (uint32_t)s.node_slots_n * D;
+    uint32_t groups = 1;
+    while (groups * 2 <= ROUND_GROUPS && groups * 2 <= grid && groups * 2 * width <= MAXPTS * MAXACC * 8 &&
+           groups * 2 * width <= (uint32_t)TOTALS_POLLS * BLOCK)
+      groups *= 2;
+    a.totals.totals = s.d_round_totals;  // round 0's region
+    a.totals.arrivals = s.d_arrivals;
+    a.totals.groups = groups, a.totals.pstride = s.pstride, a.totals.spin_limit = 200000;
+    a.passes = (uint32_t)s.kernels->nodes_passes;
+    if (!s.slice_totals_clear) {  // no set-up kernel cleared them
+      EXH_HIP(hipMemsetAsync(a.totals.totals, 0, (size_t)ROUND_GROUPS * s.pstride * 8, c.stream));
+      EXH_HIP(hipMemsetAsync(a.totals.arrivals, 0, 4, c.stream));
+    }
+  }
+  for (int pass = 0; pass < s.kernels->nodes_passes; pass++) {
+    c.prof_begin("round_nodes_base", 0, (uint64_t)T * 16 * n_pairs);
+    s.kernels->launch_nodes(&a, pass, grid, c.stream);
+    c.prof_end();
+  }
   EXH_HIP(hipGetLastError());
   return OK;
 }

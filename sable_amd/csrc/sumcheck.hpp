@@ -50,6 +50,9 @@ struct SumcheckSession {
   uint32_t *d_partials = nullptr, *d_sums = nullptr, *d_lifted = nullptr;
   unsigned long long *d_slice_totals = nullptr;  // the totals of the grid launch of slices
   bool slice_totals_clear = false;               // cleared by the session's set-up kernel and not used since
+  unsigned long long *d_round_totals = nullptr;  // the streaming rounds' totals, a region per round
+  uint32_t *d_arrivals = nullptr;                // and their arrival counters
+  uint64_t zeroed_words = 0;                     // what the set-up kernel clears: all three
   uint32_t *host_log = nullptr;                  // set around the loop's last launch: where it delivers the logs
   uint32_t host_flag_at = 0, host_seq = 0;
   uint64_t max_grid = 0;

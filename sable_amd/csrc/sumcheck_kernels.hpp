@@ -61,7 +61,26 @@ struct RoundArgs {
   Ctrl *ctrl;                // device-driven rounds: the fold challenge is read from here (else null)
   uint32_t pstride;          // words per workgroup partial (a power of two >= nacc * D)
   uint32_t double_fold;      // base tables, folded by challenges 0 and 1 at once (8 entries -> 2 per pair)
+  // device-driven rounds: the round's sums meet in counted totals and the last workgroup to arrive sends the
+  // message and draws the challenge itself (see RoundTotals); totals null: one partial row per workgroup
+  unsigned long long *totals;  // [groups][pstride], zero before the launch
+  uint32_t *arrivals;          // workgroups that have added their sums, zero before the launch
+  uint32_t groups, points, spin_limit;
+  const uint32_t *mtilde, *c0;  // the round's message map and constant terms
 };
+
+// How the workgroups of a streaming launch finish a round without another launch.  Every workgroup adds its sums
+// into the totals of its group (workgroup w: group w % groups) with integer atomics that also count the
+// contribution in the word's top 16 bits, then takes a ticket; the workgroup with the last ticket polls the words
+// until each carries its group's full count -- the data travels inside the atomics, so no fence is needed and
+// nobody reads memory another workgroup wrote with plain stores -- and goes on to the message, the transcript step
+// and the next challenge, which the next launch reads from the control block.
+struct RoundTotals {
+  unsigned long long *totals;
+  uint32_t *arrivals;
+  uint32_t groups, pstride, spin_limit;
+};
+constexpr int TOTALS_POLLS = 8;  // words a thread of the elected workgroup polls: groups * width <= 8 * BLOCK
 
 // The rounds below 2^18 pairs, with the tables resident in LDS: no global memory round trip separates a
 // round's sums, its transcript step and its fold.  With one workgroup (the last rounds) everything
@@ -633,6 +652,70 @@ __device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums,
   }
 }
 
+// All threads of the workgroup call with its sums (canonical, `width` words) in `mine` (LDS).  True in the one
+// workgroup that arrived last, which then holds the sums over all workgroups in `sums` (LDS, width words);
+// *ok is false when a word did not complete within the spin limit.  scratch: groups * width words of LDS.
+// A launch may add only the words [add_first, add_first + add_count) (the passes of the base-field sweep share one
+// set of totals, a pass per range of words); the workgroup whose ticket is last_ticket is the elected one.
+__device__ __forceinline__ bool add_and_elect(const RoundTotals &rt, const uint32_t *mine, uint32_t width,
+                                              uint32_t *scratch, uint32_t *sums, bool *ok, uint32_t add_first,
+                                              uint32_t add_count, uint32_t last_ticket) {
+  __shared__ uint32_t ticket;
+  const uint32_t tid = threadIdx.x, wg = blockIdx.x, G = gridDim.x, NG = rt.groups;
+  for (uint32_t o = add_first + tid; o < add_first + add_count; o += blockDim.x)
+    __hip_atomic_fetch_add(rt.totals + (size_t)(wg % NG) * rt.pstride + o, ((unsigned long long)1 << 48) + mine[o],
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) ticket = __hip_atomic_fetch_add(rt.arrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  *ok = true;
+  if (ticket != last_ticket) return false;
+  // every word this thread answers for is requested before any is looked at (one trip to memory for all), from a
+  // clamped address so that no load hangs on a condition
+  const uint32_t nwords = NG * width;
+  unsigned long long v[TOTALS_POLLS];
+  uint32_t pending = 0;
+#pragma unroll
+  for (int k = 0; k < TOTALS_POLLS; k++)
+    if (tid + k * blockDim.x < nwords) pending |= 1u << k;
+  uint32_t polls = 0;
+  int complete = 1;
+  while (pending) {
+#pragma unroll
+    for (int k = 0; k < TOTALS_POLLS; k++) {
+      const uint32_t u = tid + k * blockDim.x, at = u < nwords ? u : 0;
+      v[k] = __hip_atomic_load(rt.totals + (size_t)(at / width) * rt.pstride + at % width, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int k = 0; k < TOTALS_POLLS; k++) {
+      const uint32_t u = tid + k * blockDim.x, g = u / width;
+      const uint32_t expect = (G - g + NG - 1) / NG;  // workgroups w < G with w % NG == g
+      if (((pending >> k) & 1u) && (uint32_t)(v[k] >> 48) == expect) {
+        scratch[u] = f_canonical((double)(v[k] & (((unsigned long long)1 << 48) - 1)));  // exact below 2^53
+        pending &= ~(1u << k);
+      }
+    }
+    if (pending) {
+      if (++polls > rt.spin_limit) {
+        complete = 0;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  if (!__syncthreads_and(complete)) {
+    *ok = false;
+    return true;
+  }
+  for (uint32_t o = tid; o < width; o += blockDim.x) {
+    uint32_t t = 0;
+    for (uint32_t g = 0; g < NG; g++) t = fadd(t, scratch[g * width + o]);
+    sums[o] = t;
+  }
+  __syncthreads();
+  return true;
+}
+
 // One workgroup's share of a round: pairs [block * tile, (block + 1) * tile) with tile = BLOCK *
 // pairs_per_thread, folded first when FOLD, summed into the workgroup's partial row.
 template <int D>
@@ -641,6 +724,11 @@ struct RoundShape {
   uint64_t n_pairs;
   uint32_t low_bits, pairs_per_thread;
   bool deferred, do_sums;
+  // device-driven rounds (totals non-null): see RoundTotals
+  RoundTotals totals;
+  uint32_t points;
+  const uint32_t *mtilde, *c0;
+  Ctrl *ctrl;
 };
 
 template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false, bool GENERATED = false>
@@ -707,14 +795,58 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
 
   __shared__ uint32_t lds[BLOCK / 64][MAXACC * D];
   __shared__ uint32_t sums[MAXACC * D];
+  // a device-driven round: what the elected workgroup's serial part reads from memory (the transcript's state, the
+  // message map, the constant terms) is requested by every workgroup here, ahead of the reduction that hides the
+  // trip; the one elected later finds it in its LDS
+  constexpr int PRE = (MAXPTS * MAXACC * 8 + BLOCK - 1) / BLOCK;
+  uint32_t pre_map[PRE], pre_c0 = 0, pre_state = 0, pre_round = 0;
+  if (sh.totals.totals) {
+    const uint32_t map_words = sh.points * (uint32_t)d.nacc * D;
+#pragma unroll
+    for (int k = 0; k < PRE; k++) {
+      const uint32_t u = tid + k * BLOCK;
+      pre_map[k] = sh.mtilde[u < map_words ? u : 0];
+    }
+    pre_c0 = sh.c0[tid < sh.points * D ? tid : 0];
+    pre_state = reinterpret_cast<const uint32_t *>(&sh.ctrl->tr)[tid < sizeof(DevB3S) / 4 ? tid : 0];
+    pre_round = sh.ctrl->round;
+  }
   block_sums<D, false>(d, acc, lds, sums);
+  Ext<D> s;
   if (tid < (uint32_t)d.nacc) {
-    Ext<D> s;
 #pragma unroll
     for (int c = 0; c < D; c++) s.c[c] = sums[tid * D + c];
     if (sh.deferred) s = ext_mul_mont<D>(s, load_ext<D>(sh.high + (tile_start >> sh.low_bits) * D));
-    store_ext<D>(partial_row + tid * D, s);
   }
+  if (!sh.totals.totals) {
+    if (tid < (uint32_t)d.nacc) store_ext<D>(partial_row + tid * D, s);
+    return;
+  }
+  // the device-driven round: totals, and in the last workgroup to arrive the message and the challenge
+  __shared__ EpilogueLds epi;
+  __syncthreads();
+  if (tid < (uint32_t)d.nacc) {
+#pragma unroll
+    for (int c = 0; c < D; c++) sums[tid * D + c] = s.c[c];
+  }
+  {
+    const uint32_t map_words = sh.points * (uint32_t)d.nacc * D;
+#pragma unroll
+    for (int k = 0; k < PRE; k++)
+      if (tid + k * BLOCK < map_words) epi.mtilde[tid + k * BLOCK] = pre_map[k];
+    if (tid < sh.points * D) epi.c0[tid] = pre_c0;
+    if (tid < sizeof(DevB3S) / 4) epi.state[tid] = pre_state;
+    if (tid == 0) epi.round = pre_round;
+  }
+  __syncthreads();
+  bool ok;
+  const uint32_t width = (uint32_t)d.nacc * D;
+  if (!add_and_elect(sh.totals, sums, width, epi.prod, sums, &ok, 0, width, gridDim.x - 1)) return;
+  if (!ok) {
+    if (tid == 0) __hip_atomic_store(&sh.ctrl->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
+  round_epilogue<D>(sh.ctrl, sums, (uint32_t)d.nacc, sh.points, epi.mtilde, epi.c0, &epi, true);
 }
 
 template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false, bool GENERATED = false>
@@ -726,7 +858,8 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
     for (int c = 0; c < D; c++) r0.c[c] = to_mont(args.ctrl->chal[0][c]), r1.c[c] = args.ctrl->r_mont[c];
     BindWeights<D> bw = bind_weights<D>(r0, r1);
     RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
-                     args.do_sums != 0};
+                     args.do_sums != 0, RoundTotals{args.totals, args.arrivals, args.groups, args.pstride, args.spin_limit},
+                     args.points, args.mtilde, args.c0, args.ctrl};
     round_core<D, true, true, Desc, true, GENERATED>(d, args.in, args.out, sh, r, blockIdx.x,
                                           args.partials + (uint64_t)blockIdx.x * args.pstride, &bw);
     return;
@@ -737,7 +870,8 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
     for (int c = 0; c < D; c++) r.c[c] = rp[c];
   }
   RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
-                   args.do_sums != 0};
+                   args.do_sums != 0, RoundTotals{args.totals, args.arrivals, args.groups, args.pstride, args.spin_limit},
+                   args.points, args.mtilde, args.c0, args.ctrl};
   round_core<D, IN_BASE, FOLD, Desc, false, GENERATED>(d, args.in, args.out, sh, r, blockIdx.x,
                                args.partials + (uint64_t)blockIdx.x * args.pstride);
 }
@@ -1078,14 +1212,167 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
 //                       being the one factor round 0's weights have beyond round 1's.
 // All products are base-field; no folded table is written; round 2 folds twice.  A launch covers the slots
 // [PASS * SPP, (PASS + 1) * SPP) so the accumulators stay in registers.
+// The epilogue of that sweep, both rounds by one workgroup: slot sums -> round 0's accumulator sums -> its
+// message, through the transcript, to r0 -> the Lagrange basis at r0 -> round 1's accumulator sums -> its
+// message and r1.  The statement's shape comes as run-time arrays.
+struct NodesEpilogueArgs {
+  EpilogueArgs e;            // c0 points at round 0's rows, round 1's follow
+  const uint32_t *eq1;       // eq(w1, 1) and eq(w1, 0) as two elements, Montgomery form; null: both weights 1
+  uint32_t groups, slots;
+  uint32_t deg[MAXG], nev[MAXG];
+  uint8_t ev[MAXG][MAXEV];
+  uint32_t inv_den[(MAXDEG + 1) * (MAXDEG + 1)];  // [deg][m]: 1 / prod_{q != m, q <= deg} (m - q), Montgomery form
+};
+
 template <int D>
 struct NodesArgs {
   const uint32_t *in[MAXT];  // base tables
   const uint32_t *low, *high;
-  uint32_t *partials;        // [gridDim.x][pstride]: slot s at word s * D
   uint64_t n_pairs;          // pairs of round 1: four base entries each
-  uint32_t low_bits, pairs_per_thread, deferred, pstride;
+  uint32_t low_bits, pairs_per_thread, deferred;
+  // the slot sums of all passes meet in one set of counted totals (slot s at word s * D), and the last workgroup
+  // of the last pass to arrive runs the two rounds' epilogue itself (see RoundTotals)
+  RoundTotals totals;
+  uint32_t passes;
+  NodesEpilogueArgs epi;
 };
+
+// A 64-bit accumulator of 32 x 32-bit products kept below p 2^32 by a conditional subtraction of p from its high
+// word after every product: acc < p 2^32, the product of a canonical weight and a residue below 2^32 is below
+// p 2^32 as well, so the sum is below 2^64, and min(hi, hi - p) brings it back (hi < p: hi - p wraps above hi).
+// Eight registers per slot at F_p^4 where the 96-bit form takes twelve, for one more (cheap) instruction per word.
+__device__ __forceinline__ void lazy_mad(uint64_t &acc, uint32_t w, uint32_t v) {
+  acc = (uint64_t)w * v + acc;
+  const uint32_t hi = (uint32_t)(acc >> 32);
+  acc = ((uint64_t)umin32(hi, hi - P) << 32) | (uint32_t)acc;
+}
+__device__ __forceinline__ uint32_t lazy_reduce(uint64_t acc) {
+  Acc96 a;
+  a.lo = acc, a.hi = 0;
+  return acc_reduce(a);
+}
+
+// the LDS of the two rounds' epilogue
+template <int D>
+struct NodesEpilogueLds {
+  uint32_t slot_sums[MAXACC * D];
+  uint32_t sums[MAXACC * D];
+  uint32_t basis[(MAXDEG + 1) * (MAXDEG + 1) * D];  // [deg][node]: Lagrange basis at r0, Montgomery form
+  // the statement's shape: indexed by lane-dependent values out of the kernel's arguments, every access would be
+  // a load from memory with the next one waiting behind it
+  uint32_t s_deg[MAXG], s_nev[MAXG], s_inv_den[(MAXDEG + 1) * (MAXDEG + 1)];
+  uint8_t s_ev[MAXG][MAXEV];
+  EpilogueLds epi;
+};
+
+// everything the epilogue reads from memory, into LDS (all threads call; a barrier must follow before use)
+template <int D>
+__device__ __forceinline__ void nodes_epilogue_stage(const NodesEpilogueArgs &args, NodesEpilogueLds<D> &L) {
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x, points = args.e.points, nacc = args.e.nacc;
+  if (tid < MAXG) L.s_deg[tid] = args.deg[tid], L.s_nev[tid] = args.nev[tid];
+  if (tid < MAXG * MAXEV) L.s_ev[tid / MAXEV][tid % MAXEV] = args.ev[tid / MAXEV][tid % MAXEV];
+  if (tid < (MAXDEG + 1) * (MAXDEG + 1)) L.s_inv_den[tid] = args.inv_den[tid];
+  if (tid < sizeof(DevB3S) / 4) L.epi.state[tid] = reinterpret_cast<const uint32_t *>(&args.e.ctrl->tr)[tid];
+  for (uint32_t u = tid; u < points * nacc * D; u += nthreads) L.epi.mtilde[u] = args.e.mtilde[u];
+  for (uint32_t u = tid; u < points * D; u += nthreads) L.epi.c0[u] = args.e.c0[u];
+}
+
+// from the slot sums (L.slot_sums) to both rounds' messages and challenges; all threads of the workgroup call
+template <int D>
+__device__ __forceinline__ void nodes_epilogue_body(const NodesEpilogueArgs &args, NodesEpilogueLds<D> &L) {
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x, points = args.e.points, nacc = args.e.nacc;
+  EpilogueLds &epi = L.epi;
+  auto slot = [&](uint32_t index) {
+    Ext<D> v;
+#pragma unroll
+    for (int c = 0; c < D; c++) v.c[c] = L.slot_sums[index * D + c];
+    return v;
+  };
+  auto row_of = [&](uint32_t g, uint32_t x) {  // the index of X among group g's points, or nev
+    uint32_t at = L.s_nev[g];
+    for (uint32_t e = 0; e < L.s_nev[g]; e++)
+      if (L.s_ev[g][e] == x) at = e;
+    return at;
+  };
+  // accumulator tid is point e of group g, whose slots start at `base` (every thread finds its own, so that the
+  // accumulators' sums below run side by side on the lanes of one wavefront)
+  uint32_t g = 0, e = 0, base = 0;
+  bool mine = false;
+  {
+    uint32_t a = 0;
+    for (uint32_t k = 0; k < args.groups && !mine; k++) {
+      const uint32_t nev = L.s_nev[k];
+      if (tid < a + nev) {
+        g = k, e = tid - a, mine = true;
+      } else {
+        a += nev;
+        base += nev * (L.s_deg[k] + 1) + (row_of(k, 1) < nev ? 0 : nev);
+      }
+    }
+  }
+  // ---- round 0: accumulator (g, e) = eq(w1, 0) * slot(X1 = 0, node ev_e) + eq(w1, 1) * slot(X1 = 1, node ev_e)
+  if (mine) {
+    const uint32_t deg = L.s_deg[g], nev = L.s_nev[g], row0 = row_of(g, 0), row1 = row_of(g, 1);
+    const uint32_t node = L.s_ev[g][e];
+    Ext<D> at0 = slot(base + row0 * (deg + 1) + node);
+    Ext<D> at1 = row1 < nev ? slot(base + row1 * (deg + 1) + node) : slot(base + nev * (deg + 1) + e);
+    if (args.eq1) {
+      at1 = ext_mul_mont<D>(at1, load_ext<D>(args.eq1));
+      at0 = ext_mul_mont<D>(at0, load_ext<D>(args.eq1 + D));
+    }
+    const Ext<D> total = ext_add<D>(at0, at1);
+#pragma unroll
+    for (int c = 0; c < D; c++) L.sums[tid * D + c] = total.c[c];
+  }
+  __syncthreads();
+  round_message<D>(L.sums, nacc, points, epi.mtilde, epi.c0, &epi);
+  RunB3S tr;
+  if (tid < 64) {
+    rb3s_load(tr, epi.ring, reinterpret_cast<const DevB3S *>(epi.state));
+    transcript_step<D>(tr, args.e.ctrl, 0, points, &epi);
+  }
+  __syncthreads();
+  // ---- round 1: the basis of nodes 0..deg at r0, L_m = prod_{q != m} (r0 - q) / (m - q)
+  for (uint32_t u = tid; u < points * D; u += nthreads) epi.c0[u] = args.e.c0[points * D + u];
+  if (tid < (MAXDEG + 1) * (MAXDEG + 1)) {
+    const uint32_t deg = tid / (MAXDEG + 1), m = tid % (MAXDEG + 1);
+    if (deg >= 1 && m <= deg) {
+      Ext<D> r0, acc = ext_lift<D>(R1);  // 1 in Montgomery form
+#pragma unroll
+      for (int c = 0; c < D; c++) r0.c[c] = epi.r_mont[c];
+      for (uint32_t q = 0; q <= deg; q++) {
+        if (q == m) continue;
+        Ext<D> f = r0;
+        f.c[0] = fsub(f.c[0], to_mont(q));  // (r0 - q) R
+        acc = ext_mul_mont<D>(acc, f);
+      }
+      acc = ext_scale_mont<D>(acc, L.s_inv_den[tid]);
+#pragma unroll
+      for (int c = 0; c < D; c++) L.basis[tid * D + c] = acc.c[c];
+    }
+  }
+  __syncthreads();
+  // accumulator (g, e) = sum over nodes of basis * slot
+  if (mine) {
+    const uint32_t deg = L.s_deg[g];
+    Ext<D> total = ext_zero<D>();
+    for (uint32_t m = 0; m <= deg; m++) {
+      Ext<D> lb;
+#pragma unroll
+      for (int c = 0; c < D; c++) lb.c[c] = L.basis[(deg * (MAXDEG + 1) + m) * D + c];
+      total = ext_add<D>(total, ext_mul_mont<D>(lb, slot(base + e * (deg + 1) + m)));
+    }
+#pragma unroll
+    for (int c = 0; c < D; c++) L.sums[tid * D + c] = total.c[c];
+  }
+  __syncthreads();
+  round_message<D>(L.sums, nacc, points, epi.mtilde, epi.c0, &epi);
+  if (tid < 64) {
+    transcript_step<D>(tr, args.e.ctrl, 1, points, &epi);
+    rb3s_store(tr, &args.e.ctrl->tr);
+    if (tid == 0) args.e.ctrl->round = 2;
+  }
+}
 
 // the slot sums: lines and products in double precision (field.hpp), weighted sums in integers
 template <int D, int PASS, int SPP, class Desc>
@@ -1097,15 +1384,15 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
   const uint32_t tid = threadIdx.x;
   const uint64_t tile = (uint64_t)BLOCK * args.pairs_per_thread, tile_start = (uint64_t)blockIdx.x * tile;
   const uint64_t low_mask = ((uint64_t)1 << args.low_bits) - 1;
-  // the weighted sums themselves are integer: one 32 x 32 -> 64 multiply-add per word into 96 bits (twelve
-  // registers a slot where two exact double sums would take sixteen); up to 2^32 terms below 2^63 fit
-  Acc96 acc[SPP][D];
+  // the weighted sums themselves are integer: one 32 x 32 -> 64 multiply-add per word into a lazily reduced
+  // 64-bit sum (lazy_mad)
+  uint64_t acc[SPP][D];
 #pragma unroll
   for (int a = 0; a < SPP; a++)
 #pragma unroll
-    for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
+    for (int c = 0; c < D; c++) acc[a][c] = 0;
 
-  // the loads run PREFETCH pairs ahead of the arithmetic: few waves fit beside 16 registers per slot
+  // the loads run PREFETCH pairs ahead of the arithmetic: few waves fit beside the accumulators
   constexpr int PREFETCH = 2;
   uint4 ahead[PREFETCH][MAXT];
   Ext<D> wahead[PREFETCH];
@@ -1196,7 +1483,9 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
                     for (int j = 1; j < MAXDEG; j++)
                       if (j < d.deg[g]) prod = f_mul(prod, val[j]);
                     if (d.deg[g] == 1) prod = f_reduce(prod);
-                    ext_scale_acc<D>(acc[slot - PASS * SPP], we, f_residue32(prod));
+                    const uint32_t pv = f_residue32(prod);
+#pragma unroll
+                    for (int c = 0; c < D; c++) lazy_mad(acc[slot - PASS * SPP][c], we.c[c], pv);
                   }
 #pragma unroll
                   for (int j = 0; j < MAXDEG; j++)
@@ -1215,7 +1504,9 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
   // the workgroup's sums of this launch's slots, HIGH applied once when deferred
   constexpr int WORDS = SPP * D, CHUNKS = (WORDS + 31) / 32;
   __shared__ uint32_t lds[BLOCK / 64][CHUNKS * 32];
+  __shared__ NodesEpilogueLds<D> L;
   const uint32_t lane = tid & 63, wave = tid >> 6;
+  nodes_epilogue_stage<D>(args.epi, L);  // (the loads' trip hides behind the reduction below)
   {  // the wavefront's sums, 32 words at a time by the transposing reduction
     uint32_t idx = 0;
 #pragma unroll
@@ -1224,14 +1515,16 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
     for (int first = 0; first < WORDS; first += 32) {
       const uint32_t total = wave_sums_transposed<32>([&](int k) -> uint32_t {
         const int o = first + k;
-        return o < WORDS ? acc_reduce(acc[o / D][o % D]) : 0u;
+        return o < WORDS ? lazy_reduce(acc[o / D][o % D]) : 0u;
       });
       if (lane < 32) lds[wave][first + idx] = total;
     }
   }
   __syncthreads();
   const int total = node_slots(d);
-  if (tid < SPP && PASS * SPP + (int)tid < total) {
+  const bool mine = tid < SPP && PASS * SPP + (int)tid < total;
+  Ext<D> sum = ext_zero<D>();
+  if (mine) {
     // The sums above are of w * (the plain product of the group's factors); the integer kernels' products
     // carry 1/R per multiplication, which the epilogue's constants expect: times R^(1 - degree) here.
     int base = 0, deg = 1;
@@ -1241,7 +1534,6 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
     }
     uint32_t fix = R1;  // mont_mul(v, fix) = v R^(1 - degree)
     for (int q = 1; q < deg; q++) fix = mont_mul(fix, 1u);
-    Ext<D> sum;
 #pragma unroll
     for (int c = 0; c < D; c++) {
       uint32_t v = lds[0][tid * D + c];
@@ -1250,131 +1542,23 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
       sum.c[c] = mont_mul(v, fix);
     }
     if (args.deferred) sum = ext_mul_mont<D>(sum, load_ext<D>(args.high + (tile_start >> args.low_bits) * D));
-    store_ext<D>(args.partials + (uint64_t)blockIdx.x * args.pstride + (PASS * SPP + tid) * D, sum);
   }
-}
-
-// The epilogue of that sweep, both rounds in one workgroup: slot sums -> round 0's accumulator sums -> its
-// message, through the transcript, to r0 -> the Lagrange basis at r0 -> round 1's accumulator sums -> its
-// message and r1.  The statement's shape comes as run-time arrays.
-struct NodesEpilogueArgs {
-  EpilogueArgs e;            // c0 points at round 0's rows, round 1's follow
-  const uint32_t *eq1;       // eq(w1, 1) and eq(w1, 0) as two elements, Montgomery form; null: both weights 1
-  uint32_t groups, slots;
-  uint32_t deg[MAXG], nev[MAXG];
-  uint8_t ev[MAXG][MAXEV];
-  uint32_t inv_den[(MAXDEG + 1) * (MAXDEG + 1)];  // [deg][m]: 1 / prod_{q != m, q <= deg} (m - q), Montgomery form
-};
-
-template <int D>
-__global__ __launch_bounds__(EPI_BLOCK) void nodes_epilogue_kernel(NodesEpilogueArgs args) {
-  __shared__ uint32_t scratch[EPI_BLOCK];
-  __shared__ uint32_t slot_sums[MAXACC * D];
-  __shared__ uint32_t sums[MAXACC * D];
-  __shared__ uint32_t basis[(MAXDEG + 1) * (MAXDEG + 1) * D];  // [deg][node]: Lagrange basis at r0, Montgomery form
-  __shared__ EpilogueLds epi;
-  const uint32_t tid = threadIdx.x, ps = args.e.pstride, points = args.e.points, nacc = args.e.nacc;
-  // the statement's shape into LDS first: indexed by lane-dependent values out of the kernel's arguments, every
-  // access would be a load from memory with the next one waiting behind it
-  __shared__ uint32_t s_deg[MAXG], s_nev[MAXG], s_inv_den[(MAXDEG + 1) * (MAXDEG + 1)];
-  __shared__ uint8_t s_ev[MAXG][MAXEV];
-  if (tid < MAXG) s_deg[tid] = args.deg[tid], s_nev[tid] = args.nev[tid];
-  if (tid < MAXG * MAXEV) s_ev[tid / MAXEV][tid % MAXEV] = args.ev[tid / MAXEV][tid % MAXEV];
-  if (tid < (MAXDEG + 1) * (MAXDEG + 1)) s_inv_den[tid] = args.inv_den[tid];
-  if (tid < sizeof(DevB3S) / 4) epi.state[tid] = reinterpret_cast<const uint32_t *>(&args.e.ctrl->tr)[tid];
-  for (uint32_t u = tid; u < points * nacc * D; u += EPI_BLOCK) epi.mtilde[u] = args.e.mtilde[u];
-  for (uint32_t u = tid; u < points * D; u += EPI_BLOCK) epi.c0[u] = args.e.c0[u];
-  sum_partials(args.e.partials, args.e.nblocks, ps, args.slots * D, scratch, slot_sums);
-  auto slot = [&](uint32_t index) {
-    Ext<D> v;
-#pragma unroll
-    for (int c = 0; c < D; c++) v.c[c] = slot_sums[index * D + c];
-    return v;
-  };
-  auto row_of = [&](uint32_t g, uint32_t x) {  // the index of X among group g's points, or nev
-    uint32_t at = s_nev[g];
-    for (uint32_t e = 0; e < s_nev[g]; e++)
-      if (s_ev[g][e] == x) at = e;
-    return at;
-  };
-  // accumulator tid is point e of group g, whose slots start at `base` (every thread finds its own, so that the
-  // accumulators' sums below run side by side on the lanes of one wavefront)
-  uint32_t g = 0, e = 0, base = 0;
-  bool mine = false;
-  {
-    uint32_t a = 0;
-    for (uint32_t k = 0; k < args.groups && !mine; k++) {
-      const uint32_t nev = s_nev[k];
-      if (tid < a + nev) {
-        g = k, e = tid - a, mine = true;
-      } else {
-        a += nev;
-        base += nev * (s_deg[k] + 1) + (row_of(k, 1) < nev ? 0 : nev);
-      }
-    }
-  }
-  // ---- round 0: accumulator (g, e) = eq(w1, 0) * slot(X1 = 0, node ev_e) + eq(w1, 1) * slot(X1 = 1, node ev_e)
+  // the slot sums of all workgroups and passes, and in the last workgroup of the last pass both rounds' epilogue
   if (mine) {
-    const uint32_t deg = s_deg[g], nev = s_nev[g], row0 = row_of(g, 0), row1 = row_of(g, 1);
-    const uint32_t node = s_ev[g][e];
-    Ext<D> at0 = slot(base + row0 * (deg + 1) + node);
-    Ext<D> at1 = row1 < nev ? slot(base + row1 * (deg + 1) + node) : slot(base + nev * (deg + 1) + e);
-    if (args.eq1) {
-      at1 = ext_mul_mont<D>(at1, load_ext<D>(args.eq1));
-      at0 = ext_mul_mont<D>(at0, load_ext<D>(args.eq1 + D));
-    }
-    const Ext<D> total = ext_add<D>(at0, at1);
 #pragma unroll
-    for (int c = 0; c < D; c++) sums[tid * D + c] = total.c[c];
+    for (int c = 0; c < D; c++) L.sums[(PASS * SPP + tid) * D + c] = sum.c[c];
   }
   __syncthreads();
-  round_message<D>(sums, nacc, points, epi.mtilde, epi.c0, &epi);
-  RunB3S tr;
-  if (tid < 64) {
-    rb3s_load(tr, epi.ring, reinterpret_cast<const DevB3S *>(epi.state));
-    transcript_step<D>(tr, args.e.ctrl, 0, points, &epi);
+  const int here = total - PASS * SPP < SPP ? total - PASS * SPP : SPP;  // slots of this pass
+  bool ok;
+  if (!add_and_elect(args.totals, L.sums, (uint32_t)total * D, L.epi.prod, L.slot_sums, &ok, (uint32_t)(PASS * SPP * D),
+                     (uint32_t)(here > 0 ? here : 0) * D, args.passes * gridDim.x - 1))
+    return;
+  if (!ok) {
+    if (tid == 0) __hip_atomic_store(&args.epi.e.ctrl->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
   }
-  __syncthreads();
-  // ---- round 1: the basis of nodes 0..deg at r0, L_m = prod_{q != m} (r0 - q) / (m - q)
-  for (uint32_t u = tid; u < points * D; u += EPI_BLOCK) epi.c0[u] = args.e.c0[points * D + u];
-  if (tid < (MAXDEG + 1) * (MAXDEG + 1)) {
-    const uint32_t deg = tid / (MAXDEG + 1), m = tid % (MAXDEG + 1);
-    if (deg >= 1 && m <= deg) {
-      Ext<D> r0, acc = ext_lift<D>(R1);  // 1 in Montgomery form
-#pragma unroll
-      for (int c = 0; c < D; c++) r0.c[c] = epi.r_mont[c];
-      for (uint32_t q = 0; q <= deg; q++) {
-        if (q == m) continue;
-        Ext<D> f = r0;
-        f.c[0] = fsub(f.c[0], to_mont(q));  // (r0 - q) R
-        acc = ext_mul_mont<D>(acc, f);
-      }
-      acc = ext_scale_mont<D>(acc, s_inv_den[tid]);
-#pragma unroll
-      for (int c = 0; c < D; c++) basis[tid * D + c] = acc.c[c];
-    }
-  }
-  __syncthreads();
-  // accumulator (g, e) = sum over nodes of basis * slot
-  if (mine) {
-    const uint32_t deg = s_deg[g];
-    Ext<D> total = ext_zero<D>();
-    for (uint32_t m = 0; m <= deg; m++) {
-      Ext<D> lb;
-#pragma unroll
-      for (int c = 0; c < D; c++) lb.c[c] = basis[(deg * (MAXDEG + 1) + m) * D + c];
-      total = ext_add<D>(total, ext_mul_mont<D>(lb, slot(base + e * (deg + 1) + m)));
-    }
-#pragma unroll
-    for (int c = 0; c < D; c++) sums[tid * D + c] = total.c[c];
-  }
-  __syncthreads();
-  round_message<D>(sums, nacc, points, epi.mtilde, epi.c0, &epi);
-  if (tid < 64) {
-    transcript_step<D>(tr, args.e.ctrl, 1, points, &epi);
-    rb3s_store(tr, &args.e.ctrl->tr);
-    if (tid == 0) args.e.ctrl->round = 2;
-  }
+  nodes_epilogue_body<D>(args.epi, L);
 }
 
 // a kernel generated for one statement: S::d is its descriptor, known at compile time
