@@ -286,6 +286,66 @@ def run_commit(sa, steps, warmup, gold):
             "roofline_by_time": by_time(by)[:8]}
 
 
+def run_basefold(sa, steps, warmup, gold):
+    """Config 5's second half: BASEFOLD (src/pcs.lisp:581-657) of the F_p^8 combination H of the two committed
+    columns at nv = 23 -- 18 fold rounds of the message table and the codeword, 8 oracle trees over the folded
+    codewords (their caps through the transcript), the final table, grinding, 6 queries' openings.  Timed: the two
+    combine-columns launches (H from the columns, its codeword from the committed codewords) and the prove.
+    Resident before the timed region: the columns and their codewords (what PCS-COMMIT left)."""
+    cm = wl.COMMIT
+    c, ncols = cm["c"], cm["ncols"]
+    cols = sa.Table.random(cm["seed"], ncols << c)
+    cf = splitmix_field(cm["coefficient_seed"], ncols * 8).reshape(ncols, 8)
+    rr = splitmix_field(cm["point_seed"], c * 8).reshape(c, 8)
+    cw = sa.encode(cols, ncols, c)
+    h0 = sa.combine_columns(cols, ncols, cf)
+    v = sa.hypercube_sum(sa.Statement("t0", ["t0"]), c, [h0], 8, eq=rr)
+    h0.free()
+
+    def step():
+        h = sa.combine_columns(cols, ncols, cf)
+        cwh = sa.combine_columns(cw, ncols, cf)
+        tr = sa.Transcript(cm["open_label"], 4)
+        sa.basefold_prove(tr, c, rr, v, h, grind_bits=cm["grind_bits"], queries=cm["queries"], codeword=cwh)
+        h.free(), cwh.free()
+        return tr
+
+    dt, tr = timed(sa, step, steps, warmup)
+    proof = tr.proof()
+    want = gold.get("config5", {}).get("basefold", {}).get("proof_sha256")
+    if want is not None and sha(proof) != want:
+        sys.exit("bench.py: the timed BaseFold proof differs from the CPU oracle's")
+    by = launches(sa, step, max(2, min(steps, 5)))
+    for t in (cols, cw):
+        t.free()
+    # algorithmic bytes: the two combinations (columns and codewords read, H and its codeword written); per round i
+    # the table of 2^(23-i) EXT8s read and its fold written with the next round's sums taken in the same pass, the
+    # codeword of 2^(24-i) EXT8s read and its fold written; per oracle level its codeword read, leaf digests and
+    # node levels written and read
+    nv, fl = c, c - 5
+    ext = 32
+    nbytes = ncols * (4 << c) + (ext << c) + ncols * (4 << (c + 1)) + (ext << (c + 1))
+    nbytes += ext << nv  # round 0 reads H
+    for i in range(fl):
+        nbytes += (ext << (nv - i)) + (ext << (nv - i - 1))  # fold of the table
+        if i + 1 < fl:
+            nbytes += (ext << (nv + 1 - i)) + (ext << (nv - i))  # fold of the codeword
+        l = i + 1
+        if 2 <= l < fl and l % 2 == 0:
+            leaves = (1 << (nv - i)) // 4
+            nbytes += (ext << (nv - i)) + 32 * leaves + 64 * (leaves - 1) + 32 * (leaves - 1)
+    total_ms = sum(avg * per for avg, per, _ in by.values())
+    return {"workload": "BaseFold opening of config 5: combine-columns of the 2 committed columns (2^23) and of their "
+                        "codewords (2^24) into F_p^8, then basefold at nv = 23 (18 fold rounds, 8 oracle trees, 6 queries)",
+            "ms_per_step": 1e3 * dt, "proof_bytes": len(proof), "proof_sha256": sha(proof),
+            "proof_is_the_cpu_oracles": want is not None, "kernel_ms_per_step": total_ms,
+            "timed_launches_per_step": sum(per for _, per, _ in by.values()),
+            "roofline": {"bound": "hbm", "kernel": "combine-columns x 2 + basefold (whole opening)",
+                         "achieved": nbytes / dt / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS, "alg_bytes": nbytes, "traffic": None},
+            "roofline_by_time": by_time(by)[:10]}
+
+
 def run_combine(sa, steps, warmup, ncols=2):
     """combine-columns at config 5's shape: the committed columns of 2^23 base values into the table of 2^23
     EXT8s that BaseFold opens (src/pcs.lisp:434-441)."""
@@ -443,8 +503,8 @@ SEEDED = "synthetic (SplitMix64-seeded uniform field elements)"
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="config2",
-                    choices=["config1", "config2", "config3", "config4", "config5", "combine", "combine128", "copy",
-                             "mulrate"],
+                    choices=["config1", "config2", "config3", "config4", "config5", "basefold", "combine", "combine128",
+                             "copy", "mulrate"],
                     help="config2 (default) is the headline; the others are the remaining configured workloads; "
                          "copy is the known-size kernel the traffic counters are calibrated on")
     ap.add_argument("--gpus", type=int, default=1)
@@ -480,6 +540,11 @@ def main():
         res = run_commit(sa, steps, warmup, gold)
         print(json.dumps(line("BaseFold commit ms (config 5)", res["ms_per_step"], "ms", False,
                               "u32 (Montgomery KoalaBear) + BLAKE3", SEEDED, res, steps, warmup)))
+        return
+    if args.workload == "basefold":
+        res = run_basefold(sa, steps, warmup, gold)
+        print(json.dumps(line("BaseFold opening ms (config 5, nv = 23)", res["ms_per_step"], "ms", False,
+                              "u32 (Montgomery KoalaBear, F_p^8) + BLAKE3", SEEDED, res, steps, warmup)))
         return
     if args.workload == "mulrate":
         res = run_mulrate(sa)
@@ -525,6 +590,10 @@ def main():
         r = run_commit(sa, k, 2, gold)
         others["config5"] = {key: r[key] for key in ("workload", "ms_per_step", "cap_sha256", "cap_is_the_cpu_oracles",
                                                      "roofline")}
+        r = run_basefold(sa, k, 2, gold)
+        others["config5"]["basefold"] = {key: r[key] for key in ("workload", "ms_per_step", "proof_sha256",
+                                                                 "proof_is_the_cpu_oracles", "kernel_ms_per_step",
+                                                                 "timed_launches_per_step", "roofline")}
         out["other_configs"] = others
     print(json.dumps(out))
 

@@ -105,6 +105,13 @@ int exh_pcs_commit(exh_transcript tr, exh_table columns, int ncols, int c, exh_t
 int exh_basefold_prove(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, exh_table h,
                        int grind_bits, int queries, uint64_t *out_qs, uint32_t *out_challenges,
                        uint32_t *out_final);
+/* The same with ENCODE-EXT of h (src/pcs.lisp:569-575, 2^(nv+1) EXT8s on the device) supplied by the caller:
+   encoding is linear, so when h is COMBINE-COLUMNS of committed columns its codeword is exh_combine_columns of
+   their committed codewords with the same coefficients, and BASEFOLD's eight transforms (src/pcs.lisp:598-600)
+   are not repeated.  The proof is the same bytes. */
+int exh_basefold_prove_encoded(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, exh_table h,
+                               exh_table codeword, int grind_bits, int queries, uint64_t *out_qs,
+                               uint32_t *out_challenges, uint32_t *out_final);
 int exh_basefold_verify(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits,
                         int queries, uint64_t *out_qs);
 

@@ -504,14 +504,21 @@ def pcs_commit(tr, columns, ncols, c):
     return Table(hc.value, ncols << (c + 1), 1), Table(hl.value, (2 * nleaves - 1) * 8, 8)
 
 
-def basefold_prove(tr, nv, rr, v, h, grind_bits=4, queries=6):
+def basefold_prove(tr, nv, rr, v, h, grind_bits=4, queries=6, codeword=None):
+    """basefold of the table h (2^nv EXT8s); codeword: encode-ext of h as a Table of 2^(nv+1) EXT8s when the caller
+    has it (the combination of the committed codewords), else it is encoded inside."""
     rr, v = _u32(rr).reshape(-1, 8), _u32(v)
     fl = max(0, nv - 5)
     qs = np.zeros(queries, np.uint64)
     chal = np.zeros((max(fl, 1), 8), np.uint32)
     final = np.zeros((1 << (nv - fl), 8), np.uint32)
-    check(load().exh_basefold_prove(tr.h, nv, _p(rr), _p(v), C.c_uint64(h.handle), grind_bits, queries,
-                                    qs.ctypes.data_as(u64p), _p(chal), _p(final)))
+    if codeword is None:
+        check(load().exh_basefold_prove(tr.h, nv, _p(rr), _p(v), C.c_uint64(h.handle), grind_bits, queries,
+                                        qs.ctypes.data_as(u64p), _p(chal), _p(final)))
+    else:
+        check(load().exh_basefold_prove_encoded(tr.h, nv, _p(rr), _p(v), C.c_uint64(h.handle),
+                                                C.c_uint64(codeword.handle), grind_bits, queries,
+                                                qs.ctypes.data_as(u64p), _p(chal), _p(final)))
     return [int(q) for q in qs], chal[:fl], final
 
 

@@ -1082,6 +1082,20 @@ int exh_basefold_prove(exh_transcript h, int nv, const uint32_t *rr, const uint3
   }
   return basefold_prove(*tr, nv, rr, v, dt->ptr, grind_bits, queries, out_qs, out_chal, out_final);
 }
+int exh_basefold_prove_encoded(exh_transcript h, int nv, const uint32_t *rr, const uint32_t *v, exh_table table,
+                               exh_table codeword, int grind_bits, int queries, uint64_t *out_qs, uint32_t *out_chal,
+                               uint32_t *out_final) {
+  ApiLock api_lock;
+  Transcript *tr = tr_of(h);
+  DeviceTable *dt = table_of(table), *dc = table_of(codeword);
+  if (!tr || !dt || !dc) return E_PARAM;
+  if (nv < 1 || nv > 23 || dt->stride != 8 || dt->n_u32 != ((uint64_t)8 << nv) || dc->stride != 8 ||
+      dc->n_u32 != ((uint64_t)16 << nv)) {
+    set_error("invalid-parameter: BaseFold takes 2^nv EXT8s and their codeword of 2^(nv+1) EXT8s, 1 <= nv <= 23");
+    return E_PARAM;
+  }
+  return basefold_prove(*tr, nv, rr, v, dt->ptr, grind_bits, queries, out_qs, out_chal, out_final, dc->ptr);
+}
 
 int exh_basefold_verify(exh_transcript h, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,
                         uint64_t *out_qs) {

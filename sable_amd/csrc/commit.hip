@@ -6,12 +6,14 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <map>
 #include <vector>
 
 #include "blake3.hpp"
 #include "context.hpp"
 #include "hostfield.hpp"
+#include "sumcheck.hpp"
 #include "sumcheck_kernels.hpp"
 
 namespace exh {
@@ -607,8 +609,8 @@ static int cap_level_of(uint64_t leaves) {  // src/pcs.lisp:57-59
 // Every level of the tree at d_levels (leaves first), a few launches of up to nine levels each; the
 // leaf digests are computed by the first launch (leaves 1: ncols codewords, 2: an oracle codeword) or
 // already there (0).  A single leaf (no node above it) is hashed by the same kernel's bottom step.
-static int merkle_tree_device(uint32_t *d_levels, uint64_t nleaves, int leaves, const uint32_t *cw, int ncols,
-                              uint64_t cw_len, uint8_t *cap, uint64_t *cap_rows) {
+static int merkle_tree_launch(uint32_t *d_levels, uint64_t nleaves, int leaves, const uint32_t *cw, int ncols,
+                              uint64_t cw_len, uint64_t *cap_rows, uint64_t *cap_off_words) {
   Context &c = ctx();
   uint32_t *level = d_levels;
   uint64_t n = nleaves;
@@ -623,12 +625,15 @@ static int merkle_tree_device(uint32_t *d_levels, uint64_t nleaves, int leaves, 
     int height = 0;
     for (uint64_t v = n; v > 1 && height < 9; v >>= 1) height++;
     uint32_t grid = (uint32_t)((n / 2 + BLOCK - 1) / BLOCK);
+    c.prof_begin(leaves == 1 ? "merkle_leaves" : leaves == 2 ? "merkle_oracle_leaves" : "merkle_levels", 0,
+                 (leaves == 1 ? (uint64_t)ncols * 16 * n : leaves == 2 ? 128 * n : 0) + 64 * n);
     if (leaves == 1)
       hipLaunchKernelGGL(subtree_kernel<1>, dim3(grid), dim3(BLOCK), 0, c.stream, level, n, height, cw, ncols, cw_len);
     else if (leaves == 2)
       hipLaunchKernelGGL(subtree_kernel<2>, dim3(grid), dim3(BLOCK), 0, c.stream, level, n, height, cw, ncols, cw_len);
     else
       hipLaunchKernelGGL(subtree_kernel<0>, dim3(grid), dim3(BLOCK), 0, c.stream, level, n, height, cw, ncols, cw_len);
+    c.prof_end();
     leaves = 0;
     for (int s = 0; s < height; s++) {
       level += 8 * n;
@@ -637,6 +642,15 @@ static int merkle_tree_device(uint32_t *d_levels, uint64_t nleaves, int leaves, 
   }
   EXH_HIP(hipGetLastError());
   *cap_rows = nleaves >> lc;
+  *cap_off_words = cap_off;
+  return OK;
+}
+static int merkle_tree_device(uint32_t *d_levels, uint64_t nleaves, int leaves, const uint32_t *cw, int ncols,
+                              uint64_t cw_len, uint8_t *cap, uint64_t *cap_rows) {
+  Context &c = ctx();
+  uint64_t cap_off = 0;
+  int status = merkle_tree_launch(d_levels, nleaves, leaves, cw, ncols, cw_len, cap_rows, &cap_off);
+  if (status) return status;
   EXH_HIP(hipMemcpyAsync(cap, d_levels + cap_off, 32 * *cap_rows, hipMemcpyDeviceToHost, c.stream));
   EXH_HIP(hipStreamSynchronize(c.stream));
   return OK;
@@ -1052,16 +1066,195 @@ int open_queries_device(const uint32_t *d_codewords, int ncols, int c, const uin
   return OK;
 }
 
+// ------------------------------------------------------------------ BASEFOLD's rounds
+// The sumcheck of eq(rr, x) Phi(x) never needs the eq table or its folds.  After i rounds the folded eq table is
+// prf_i eq(rr[i..], .) with prf_i = prod_{j<i} eq1(r_j, x_j), so with E = eq(rr[i+1..], .) over the pairs k,
+//   DOT-PAIRS(tt, et, 0) = prf_i (1 - r_i) h0,  h0 = sum_k E[k] tt[2k]
+//   DOT-PAIRS(tt, et, 1) = prf_i r_i h1,        h1 = sum_k E[k] tt[2k+1]
+//   DOT-PAIRS(tt, et, 2) = prf_i (2 r_i - (1 - r_i)) (2 h1 - h0)
+// (src/pcs.lisp:473-483, 607-612): the same field elements, from two weighted sums of the message table with split
+// weights E[k] = LOW[k mod |LOW|] HIGH[k div |LOW|] as in the sumcheck prover (src/sumcheck.lisp:37-49).
+//
+// One launch per round does both of the round's passes over memory: its first workgroups fold the message table
+// by the last challenge (FOLD-TABLE, src/field.lisp:365-370) and take h0, h1 of the folded table in the same
+// pass; the others fold the codeword (RS:FOLD, src/rs.lisp:93-101).  The sums meet in counted totals (RoundTotals)
+// and the last summing workgroup to arrive writes them into pinned host memory and raises a flag there, so the
+// host neither copies nor waits on the stream: it polls the flag while the codeword's workgroups still run.
+struct BfStepArgs {
+  // the message table's part: workgroups [0, tt_blocks)
+  const uint32_t *tt_in;  // 4 entries per pair when folding, else 2
+  uint32_t *tt_out;       // the folded table (fold)
+  const uint32_t *low, *high;
+  uint64_t n_pairs;  // pairs after the fold
+  uint32_t low_bits, pairs_per_thread, fold, do_sums, tt_blocks;
+  uint32_t r_mont[8];
+  RoundTotals totals;
+  // 17 64-bit words in pinned host memory, each (host_seq << 32 | value): h0, h1, then 1 when the totals never
+  // completed.  Every word says itself that it has arrived, so no fence orders them: a release at system scope
+  // writes back the whole L2 of the elected workgroup's XCD, which the fold's stores of the other workgroups keep
+  // dirty (measured: 90 us per round)
+  unsigned long long *host_out;
+  uint32_t host_seq;
+  // the codeword's part: workgroups [tt_blocks, gridDim.x)
+  const uint32_t *cw_in, *tw_inv2;
+  uint32_t *cw_out;
+  uint64_t cw_m;  // elements after the fold
+};
+
+template <bool FOLD>
+__global__ __launch_bounds__(BLOCK) void bf_step_kernel(BfStepArgs a) {
+  const uint32_t tid = threadIdx.x;
+  Ext<8> r;
+#pragma unroll
+  for (int c = 0; c < 8; c++) r.c[c] = a.r_mont[c];
+  if (blockIdx.x >= a.tt_blocks) {  // pair (a, b) at twiddle x: f0 = (a + b)/2, f1 = (a - b)/(2x), f0 + r (f1 - f0)
+    const uint64_t s = (uint64_t)(blockIdx.x - a.tt_blocks) * BLOCK + tid;
+    if (s >= a.cw_m) return;
+    const Ext<8> x = load_ext<8>(a.cw_in + 2 * s * 8), y = load_ext<8>(a.cw_in + (2 * s + 1) * 8);
+    const Ext<8> f0 = ext_scale_mont<8>(ext_add<8>(x, y), mont_mul(INV2, R2));
+    const Ext<8> f1 = ext_scale_mont<8>(ext_sub<8>(x, y), a.tw_inv2[s]);
+    store_ext<8>(a.cw_out + s * 8, ext_add<8>(f0, ext_mul_mont<8>(r, ext_sub<8>(f1, f0))));
+    return;
+  }
+  const uint64_t tile = (uint64_t)BLOCK * a.pairs_per_thread, tile_start = (uint64_t)blockIdx.x * tile;
+  const uint64_t low_mask = ((uint64_t)1 << a.low_bits) - 1;
+  Acc96 acc[2][8];
+#pragma unroll
+  for (int q = 0; q < 2; q++)
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc_zero(acc[q][c]);
+  // a pair's words are requested one pair ahead of its arithmetic (Q quads per pair: 8 when folding, else 4)
+  constexpr int Q = FOLD ? 8 : 4;
+  uint4 raw[Q], ahead[Q];
+  Ext<8> w = ext_zero<8>(), w_ahead = ext_zero<8>();
+  auto fetch = [&](uint64_t i, uint4 *q, Ext<8> &wq) {
+    const uint4 *p = reinterpret_cast<const uint4 *>(a.tt_in) + (uint64_t)Q * i;
+#pragma unroll
+    for (int j = 0; j < Q; j++) q[j] = p[j];
+    if (a.do_sums) wq = load_ext<8>(a.low + (i & low_mask) * 8);
+  };
+  if (tile_start + tid < a.n_pairs) fetch(tile_start + tid, raw, w);
+  for (uint32_t k = 0; k < a.pairs_per_thread; k++) {
+    const uint64_t i = tile_start + (uint64_t)k * BLOCK + tid;
+    if (i >= a.n_pairs) break;
+    const bool more = k + 1 < a.pairs_per_thread && i + BLOCK < a.n_pairs;
+    if (more) fetch(i + BLOCK, ahead, w_ahead);
+    Ext<8> lo, hi;
+    if constexpr (FOLD) {
+      lo = fold_ext<8>(ext_from_quads<8>(raw), ext_from_quads<8>(raw + 2), r);
+      hi = fold_ext<8>(ext_from_quads<8>(raw + 4), ext_from_quads<8>(raw + 6), r);
+      store_ext<8>(a.tt_out + 2 * i * 8, lo);
+      store_ext<8>(a.tt_out + (2 * i + 1) * 8, hi);
+    } else {
+      lo = ext_from_quads<8>(raw), hi = ext_from_quads<8>(raw + 2);
+    }
+    if (a.do_sums) {
+      ext_mul_acc<8>(acc[0], lo, w);  // (the weight second: its tripled wrap coefficients serve both products)
+      ext_mul_acc<8>(acc[1], hi, w);
+    }
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < Q; j++) raw[j] = ahead[j];
+      w = w_ahead;
+    }
+  }
+  if (!a.do_sums) return;
+  __shared__ uint32_t lds[BLOCK / 64][16];
+  __shared__ uint32_t mine[16], sums[16];
+  __shared__ uint32_t scratch[TOTALS_POLLS * BLOCK];
+#pragma unroll
+  for (int q = 0; q < 2; q++)
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+      const uint32_t v = wave_sum(acc_reduce(acc[q][c]));
+      if ((tid & 63) == 0) lds[tid >> 6][q * 8 + c] = v;
+    }
+  __syncthreads();
+  if (tid < 2) {  // a workgroup's pairs share one HIGH weight (the tile is |LOW| pairs)
+    Ext<8> t;
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+      uint32_t v = lds[0][tid * 8 + c];
+#pragma unroll
+      for (int w = 1; w < BLOCK / 64; w++) v = fadd(v, lds[w][tid * 8 + c]);
+      t.c[c] = v;
+    }
+    // times HIGH / R, then times R: the plain product
+    t = ext_mul_mont<8>(t, load_ext<8>(a.high + (tile_start >> a.low_bits) * 8));
+#pragma unroll
+    for (int c = 0; c < 8; c++) mine[tid * 8 + c] = mont_mul(t.c[c], R2);
+  }
+  __syncthreads();
+  bool ok;
+  if (!add_and_elect(a.totals, mine, 16, scratch, sums, &ok, 0, 16, a.tt_blocks - 1, a.tt_blocks)) return;
+  if (tid < 17) {
+    const uint32_t value = tid < 16 ? (ok ? sums[tid] : 0u) : (ok ? 0u : 1u);
+    __hip_atomic_store(a.host_out + tid, ((unsigned long long)a.host_seq << 32) | value, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+// `words` words from device memory into pinned host memory as 64-bit words (seq << 32 | value), each its own flag
+__global__ __launch_bounds__(BLOCK) void deliver_kernel(const uint32_t *src, uint32_t words, unsigned long long *host_dst,
+                                                        uint32_t seq) {
+  for (uint32_t u = threadIdx.x; u < words; u += BLOCK)
+    __hip_atomic_store(host_dst + u, ((unsigned long long)seq << 32) | src[u], __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// segments of 8 words from anywhere in device memory, side by side into out
+__global__ __launch_bounds__(BLOCK) void gather8_kernel(const uint32_t *const *src, uint32_t count, uint32_t *out) {
+  const uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid >= (uint64_t)count * 8) return;
+  out[gid] = src[gid / 8][gid % 8];
+}
+
+__global__ __launch_bounds__(BLOCK) void zero_words_kernel(uint32_t *p, uint64_t words) {
+  const uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+  if (gid < words) p[gid] = 0;
+}
+
+// the host's side of such words in pinned memory: true once all n carry seq (their low halves then go to out);
+// false when the stream ran dry without them
+static bool await_words(Context &c, const volatile unsigned long long *w, size_t n, uint32_t seq, uint32_t *out) {
+  auto all_there = [&]() {
+    for (size_t u = n; u-- > 0;)
+      if ((uint32_t)(w[u] >> 32) != seq) return false;
+    return true;
+  };
+  uint32_t spins = 0;
+  bool there = false;
+  while (!(there = all_there())) {
+    if ((++spins & 1023) == 0 && hipStreamQuery(c.stream) != hipErrorNotReady) break;
+  }
+  if (!there) {
+    (void)hipStreamSynchronize(c.stream);
+    if (!all_there()) return false;
+  }
+  std::atomic_thread_fence(std::memory_order_acquire);
+  for (size_t u = 0; u < n; u++) out[u] = (uint32_t)w[u];
+  return true;
+}
+
+// regions of the context's pinned host buffer BaseFold's rounds use (in 32-bit words): a slot of 17 64-bit words
+// per round, then a slot of 128 * 8 64-bit words per oracle cap
+constexpr size_t BF_PIN = 32768, BF_ROUND_SLOT = 40, BF_MAX_ROUNDS = 40, BF_CAP_SLOT = 2048, BF_MAX_ORACLES = 14;
+static_assert(BF_PIN + BF_MAX_ROUNDS * BF_ROUND_SLOT + BF_MAX_ORACLES * BF_CAP_SLOT <= 65536, "the pinned buffer");
+constexpr uint32_t BF_GROUPS = 32;  // rows of totals of a round's sums (16 words each)
+
 // BASEFOLD (src/pcs.lisp:581-657) over ncls size classes, ascending, the last one nv: class c's table d_h[k]
-// (2^c EXT8s) joins the message table and the codeword at level nv - c (:590-600, :635-639)
+// (2^c EXT8s) joins the message table and the codeword at level nv - c (:590-600, :635-639).  d_cws (optional, and
+// optional per class): the class's codeword ENCODE-EXT(H_c) (2^(c+1) EXT8s) when the caller has it already --
+// encoding is linear, so the codeword of a combination of committed columns is the same combination of their
+// committed codewords (COMBINE-COLUMNS over the codewords) -- else it is encoded here, coordinate by coordinate.
 int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, const uint32_t *const *d_hs,
                            const uint32_t *rr, const uint32_t *v, int grind_bits, int queries, uint64_t *out_qs,
-                           uint32_t *out_chal, uint32_t *out_final) {
+                           uint32_t *out_chal, uint32_t *out_final, const uint32_t *const *d_cws) {
   Context &c = ctx();
   int status = c.require();
   if (status) return status;
-  if (ncls < 1 || cls[ncls - 1] != nv || queries < 1) {
-    set_error("invalid-parameter: basefold takes its classes in ascending order, the largest being nv");
+  if (ncls < 1 || cls[ncls - 1] != nv || queries < 1 || nv > 30) {
+    set_error("invalid-parameter: basefold takes its classes in ascending order, the largest being nv <= 30");
     return E_PARAM;
   }
   for (int k = 0; k < ncls; k++)
@@ -1073,19 +1266,36 @@ int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, con
   const int fl = nv - 5 > 0 ? nv - 5 : 0;
   const uint64_t len = (uint64_t)1 << nv;
   Owned mem;
-  uint32_t *tt = mem.alloc(len * 8), *tt2 = mem.alloc(len * 4 + 8), *et = mem.alloc(len * 8),
-           *et2 = mem.alloc(len * 4 + 8), *cw = mem.alloc(2 * len * 8), *cw2 = mem.alloc(len * 8);
-  uint32_t *cols = mem.alloc(len * 8), *cwcols = mem.alloc(2 * len * 8);
+  // the folded message tables ping-pong between two buffers (the class's own table is read in round 0 and never
+  // written); so do the folded codewords, except that a level with an oracle tree keeps a buffer of its own
+  uint32_t *tt_a = mem.alloc(len * 4 + 8), *tt_b = mem.alloc(len * 2 + 8);
+  uint32_t *cw_b = mem.alloc(len * 8), *cw_c = mem.alloc(len * 4 + 8);
+  uint32_t *cw0 = nullptr, *cols = nullptr, *cwcols = nullptr;
+  const bool given = d_cws && d_cws[ncls - 1];
+  if (!given) {
+    cw0 = mem.alloc(2 * len * 8), cols = mem.alloc(len * 8), cwcols = mem.alloc(2 * len * 8);
+    if (!cw0 || !cols || !cwcols) return E_NOMEM;
+  } else if (ncls > 1) {  // the joining classes add their codewords into the working one
+    cols = mem.alloc(len * 4), cwcols = mem.alloc(len * 8);
+    if (!cols || !cwcols) return E_NOMEM;
+  }
   const uint32_t max_grid = 1024;
   uint32_t *partials = mem.alloc((uint64_t)max_grid * 24 + 24), *factors = mem.alloc((uint64_t)nv * 16 + 16);
-  if (!tt || !tt2 || !et || !et2 || !cw || !cw2 || !cols || !cwcols || !partials || !factors) return E_NOMEM;
+  if (!tt_a || !tt_b || !cw_b || !cw_c || !partials || !factors) return E_NOMEM;
   uint32_t *sums = partials + (uint64_t)max_grid * 24;
-  uint32_t grid_len = (uint32_t)((len + BLOCK - 1) / BLOCK);
-  // tt = H, cw = ENCODE-EXT(H), et = eq-table(rr)
-  EXH_HIP(hipMemcpyAsync(tt, d_h, len * 32, hipMemcpyDeviceToDevice, c.stream));
-  hipLaunchKernelGGL(split_coords_kernel, dim3(grid_len), dim3(BLOCK), 0, c.stream, d_h, cols, len);
-  if ((status = rs_encode_columns(cols, 8, nv, cwcols))) return status;
-  hipLaunchKernelGGL(join_coords_kernel, dim3(2 * grid_len), dim3(BLOCK), 0, c.stream, cwcols, cw, 2 * len);
+  const uint32_t grid_len = (uint32_t)((len + BLOCK - 1) / BLOCK);
+  // cw = ENCODE-EXT(H) unless given
+  const uint32_t *cw = given ? d_cws[ncls - 1] : cw0;
+  if (!given) {
+    hipLaunchKernelGGL(split_coords_kernel, dim3(grid_len), dim3(BLOCK), 0, c.stream, d_h, cols, len);
+    if ((status = rs_encode_columns(cols, 8, nv, cwcols))) return status;
+    hipLaunchKernelGGL(join_coords_kernel, dim3(2 * grid_len), dim3(BLOCK), 0, c.stream, cwcols, cw0, 2 * len);
+  }
+  // ---- the rounds' split weights: round i sums over the pairs k of variables i+1 .. nv-1; LOW covers a workgroup's
+  // tile, HIGH the rest
+  std::vector<int> low_bits(std::max(fl, 1), 0);
+  std::vector<uint64_t> low_off(std::max(fl, 1), 0), high_off(std::max(fl, 1), 0);
+  uint32_t *weights = nullptr;
   {
     std::vector<uint32_t> f((size_t)nv * 16);
     for (int b = 0; b < nv; b++)
@@ -1094,8 +1304,31 @@ int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, con
         f[((size_t)b * 2) * 8 + k] = to_mont(r);
         f[((size_t)b * 2 + 1) * 8 + k] = to_mont(fsub(k == 0 ? 1u : 0u, r));
       }
-    EXH_HIP(hipMemcpy(factors, f.data(), f.size() * 4, hipMemcpyHostToDevice));
-    hipLaunchKernelGGL(eq8_kernel, dim3(grid_len), dim3(BLOCK), 0, c.stream, factors, nv, et, len);
+    EXH_HIP(hipMemcpyAsync(factors, f.data(), f.size() * 4, hipMemcpyHostToDevice, c.stream));
+    EXH_HIP(hipStreamSynchronize(c.stream));  // `f` is pageable
+    if (fl > BF_MAX_ROUNDS || 2 * fl > 64) {
+      set_error("invalid-parameter: basefold rounds beyond the buffers");
+      return E_PARAM;
+    }
+    std::vector<int> first, bits;
+    std::vector<uint64_t> off;
+    uint64_t pos = 0;
+    for (int i = 0; i < fl; i++) {
+      const int rest = nv - 1 - i;  // variables of the pairs
+      // (tiles of 2^10 to 2^12 pairs, at least a thousand of them while the table is that large: long tiles in few
+      // workgroups trail their loads one after another, short ones pay the reduction and the atomics per tile)
+      low_bits[i] = std::min(rest, std::min(std::max(rest - 10, 10), 12));
+      low_off[i] = pos, first.push_back(i + 1), bits.push_back(low_bits[i]), off.push_back(pos);
+      pos += (uint64_t)1 << low_bits[i];
+      high_off[i] = pos, first.push_back(i + 1 + low_bits[i]), bits.push_back(rest - low_bits[i]), off.push_back(pos);
+      pos += (uint64_t)1 << (rest - low_bits[i]);
+    }
+    if (fl > 0) {
+      weights = mem.alloc(pos * 8);
+      if (!weights) return E_NOMEM;
+      if ((status = eq_tables_launch(8, (int)first.size(), first.data(), bits.data(), off.data(), factors, nv, weights)))
+        return status;
+    }
   }
   EXH_HIP(hipGetLastError());
   Domain *dom;
@@ -1108,7 +1341,7 @@ int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, con
   hf::E ysum = hf::zero(8);
   for (int k = 0; k + 1 < ncls; k++) {
     const uint64_t clen = (uint64_t)1 << cls[k], n_pairs = clen / 2;
-    uint32_t *eqc = et2;  // the eq table of the point's tail (at most half of et2's room)
+    uint32_t *eqc = tt_a;  // the eq table of the point's tail (at most half of the buffer's room)
     hipLaunchKernelGGL(eq8_kernel, dim3((uint32_t)((clen + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, c.stream,
                        factors + (size_t)(nv - cls[k]) * 16, cls[k], eqc, clen);
     uint32_t grid = (uint32_t)std::min<uint64_t>((n_pairs + BLOCK - 1) / BLOCK, max_grid);
@@ -1120,22 +1353,88 @@ int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, con
     yc[k] = hf::add(hf::from(dots, 8), hf::from(dots + 8, 8));  // even entries' products + odd entries' products
     ysum = hf::add(ysum, yc[k]);
   }
+  // ---- the rounds' totals (cleared by a kernel: callers may record this path) and the pinned slots
+  const uint64_t total_words = (uint64_t)std::max(fl, 1) * BF_GROUPS * 16 * 2 + std::max(fl, 1) + 1;
+  uint32_t *totals_mem = mem.alloc(total_words + (total_words & 1));
+  if (!totals_mem) return E_NOMEM;
+  hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)((total_words + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, c.stream,
+                     totals_mem, total_words);
+  uint32_t *arrivals = totals_mem + (uint64_t)std::max(fl, 1) * BF_GROUPS * 16 * 2;
+  volatile uint32_t *pin = c.host_pinned + BF_PIN;
+  uint32_t *pin_dev = c.host_pinned_dev + BF_PIN;
+  if (++c.log_seq == 0) ++c.log_seq;  // (a word of an earlier proof carries an earlier number)
+  const uint32_t seq = c.log_seq;
+
   std::vector<OracleTree> oracles;
+  const uint32_t *tt = d_h;  // the table the next step reads
+  uint32_t x[8] = {0};
+  // the launch of round i: fold the table by x (the challenge of round i - 1) when i > 0, sum round i's h0, h1;
+  // with_cw: fold the codeword of level i - 1 as well, into cw_out
+  auto launch_step = [&](int i, bool fold, bool do_sums, uint32_t *cw_out) -> int {
+    BfStepArgs a;
+    memset(&a, 0, sizeof(a));
+    const uint64_t entries = fold ? len >> i : len >> i;  // entries of the table summed (after the fold)
+    (void)entries;
+    const uint64_t n_pairs = (len >> i) / 2;
+    a.tt_in = tt, a.fold = fold ? 1 : 0, a.do_sums = do_sums ? 1 : 0, a.n_pairs = n_pairs;
+    if (fold) a.tt_out = (tt == tt_a) ? tt_b : tt_a;
+    uint32_t tile = 1;
+    if (do_sums) {
+      a.low = weights + low_off[i] * 8, a.high = weights + high_off[i] * 8, a.low_bits = (uint32_t)low_bits[i];
+      tile = (uint32_t)1 << low_bits[i];  // |LOW| pairs: one HIGH weight per workgroup
+    } else {
+      tile = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(n_pairs, 1), 4 * BLOCK);
+    }
+    a.pairs_per_thread = std::max<uint32_t>(1, tile / BLOCK);
+    a.tt_blocks = n_pairs ? (uint32_t)((n_pairs + tile - 1) / tile) : 0;
+    for (int k = 0; k < 8; k++) a.r_mont[k] = to_mont(x[k]);
+    if (do_sums) {
+      uint32_t groups = 1;
+      while (groups * 2 <= BF_GROUPS && groups * 2 <= a.tt_blocks) groups *= 2;
+      a.totals.totals = reinterpret_cast<unsigned long long *>(totals_mem) + (uint64_t)i * BF_GROUPS * 16;
+      a.totals.arrivals = arrivals + i;
+      a.totals.groups = groups, a.totals.pstride = 16, a.totals.spin_limit = 200000;
+      a.host_out = reinterpret_cast<unsigned long long *>(pin_dev + (size_t)i * BF_ROUND_SLOT), a.host_seq = seq;
+    }
+    uint32_t cw_blocks = 0;
+    if (cw_out) {
+      const uint64_t m = (len >> (i - 1));  // elements of the folded codeword: half of level i - 1's 2^(nv + 2 - i)
+      a.cw_in = cw, a.cw_out = cw_out, a.cw_m = m, a.tw_inv2 = dom->tw_inv2 + dom->off[i - 1];
+      cw_blocks = (uint32_t)((m + BLOCK - 1) / BLOCK);
+    }
+    if (a.tt_blocks + cw_blocks == 0) return OK;
+    c.prof_begin("basefold_step", i, (fold ? 3 : 2) * n_pairs * 32 * (do_sums || fold ? 1 : 0) + (cw_out ? 3 * a.cw_m * 32 : 0));
+    if (fold)
+      hipLaunchKernelGGL(bf_step_kernel<true>, dim3(a.tt_blocks + cw_blocks), dim3(BLOCK), 0, c.stream, a);
+    else
+      hipLaunchKernelGGL(bf_step_kernel<false>, dim3(a.tt_blocks + cw_blocks), dim3(BLOCK), 0, c.stream, a);
+    c.prof_end();
+    EXH_HIP(hipGetLastError());
+    if (fold) tt = a.tt_out;
+    if (cw_out) cw = cw_out;
+    return OK;
+  };
+  if (fl > 0 && (status = launch_step(0, false, true, nullptr))) return status;
+  size_t cap_slots = 0;
   for (int i = 0; i < fl; i++) {
-    uint64_t cur = len >> i, n_pairs = cur / 2;
-    uint32_t grid = (uint32_t)std::min<uint64_t>((n_pairs + BLOCK - 1) / BLOCK, max_grid);
-    hipLaunchKernelGGL(dot_pairs_kernel, dim3(grid), dim3(BLOCK), 0, c.stream, tt, et, n_pairs, partials);
-    hipLaunchKernelGGL(sum_columns_kernel, dim3(24), dim3(BLOCK), 0, c.stream, partials, grid, 24u, sums);
+    // ---- the round's message from h0, h1
+    uint32_t hh[17];
+    if (!await_words(c, reinterpret_cast<const volatile unsigned long long *>(pin + (size_t)i * BF_ROUND_SLOT), 17, seq,
+                     hh) ||
+        hh[16]) {
+      set_error("device-error: a basefold round's sums did not arrive");
+      return E_DEVICE;
+    }
+    const hf::E h0 = hf::from(hh, 8), h1 = hf::from(hh + 8, 8);
+    const hf::E ri = hf::from(rr + 8 * (size_t)i, 8), one_r = hf::sub(hf::lift(1, 8), ri);
+    const hf::E eqx[3] = {one_r, ri, hf::sub(hf::scale(ri, 2), one_r)};
+    const hf::E hx[3] = {h0, h1, hf::sub(hf::scale(h1, 2), h0)};
     uint32_t ev[24];
-    EXH_HIP(hipMemcpyAsync(ev, sums, 96, hipMemcpyDeviceToHost, c.stream));
-    EXH_HIP(hipStreamSynchronize(c.stream));
-    if (ncls > 1) {  // the classes still to join: a = prf * ysum times (1 - r_i, r_i, 2 r_i - (1 - r_i)), :607-612
-      const hf::E ri = hf::from(rr + 8 * (size_t)i, 8), a = hf::mul(prf, ysum), one_r = hf::sub(hf::lift(1, 8), ri);
-      const hf::E eqx[3] = {one_r, ri, hf::sub(hf::scale(ri, 2), one_r)};
-      for (int parity = 0; parity < 3; parity++) {
-        hf::E t = hf::add(hf::from(ev + 8 * parity, 8), hf::mul(a, eqx[parity]));
-        memcpy(ev + 8 * parity, t.data(), 32);
-      }
+    const hf::E a_term = ncls > 1 ? hf::mul(prf, ysum) : hf::zero(8);  // the classes still to join, :607-612
+    for (int parity = 0; parity < 3; parity++) {
+      hf::E t = hf::mul(hf::mul(prf, eqx[parity]), hx[parity]);
+      if (ncls > 1) t = hf::add(t, hf::mul(a_term, eqx[parity]));
+      memcpy(ev + 8 * parity, t.data(), 32);
     }
     uint64_t dims[2] = {3, 8};
     if ((status = tr.send(ev, 2, dims, nullptr))) return status;
@@ -1143,55 +1442,97 @@ int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, con
       set_error("verification-failure: pcs: basefold sumcheck round " + std::to_string(i) + " failed");
       return E_REJECT;
     }
-    uint32_t x[8];
     tr.challenge(8, x);
     if (out_chal) memcpy(out_chal + 8 * i, x, 32);
     claim = hf::lagrange({hf::from(ev, 8), hf::from(ev + 8, 8), hf::from(ev + 16, 8)}, hf::from(x, 8));
     prf = hf::mul(prf, hf::eq1(hf::from(rr + 8 * i, 8), hf::from(x, 8)));
-    RoundArgs<8> a;
-    memset(&a, 0, sizeof(a));
-    for (int k = 0; k < 8; k++) a.r_mont[k] = to_mont(x[k]);
-    uint32_t gfold = (uint32_t)((n_pairs + BLOCK - 1) / BLOCK);
-    hipLaunchKernelGGL(fold_table_kernel<8>, dim3(gfold), dim3(BLOCK), 0, c.stream, tt, tt2, n_pairs, a);
-    hipLaunchKernelGGL(fold_table_kernel<8>, dim3(gfold), dim3(BLOCK), 0, c.stream, et, et2, n_pairs, a);
-    std::swap(tt, tt2);
-    std::swap(et, et2);
-    if ((status = rs_fold_launch(8, cur, dom->tw_inv2 + dom->off[i], cw, x, cw2))) return status;
-    std::swap(cw, cw2);
-    int l = i + 1;
-    if (l >= 2 && l < fl && l % 2 == 0) {  // an oracle tree over the folded codeword
+    // ---- level l: fold the table and the codeword by x; an oracle tree over the folded codeword; the joins
+    const int l = i + 1;
+    const uint64_t cur = len >> i;  // elements of the folded codeword
+    const bool oracle = l >= 2 && l < fl && l % 2 == 0;
+    bool joins = false;
+    for (int k = 0; k + 1 < ncls; k++) joins = joins || nv - cls[k] == l;
+    uint32_t *cw_out = nullptr;
+    if (l < fl) {  // (the last level's codeword is never looked at)
+      if (oracle) {
+        if (oracles.size() >= BF_MAX_ORACLES) {
+          set_error("invalid-parameter: basefold oracle levels beyond the buffers");
+          return E_PARAM;
+        }
+        cw_out = mem.alloc(cur * 8);
+        if (!cw_out) return E_NOMEM;
+      } else {
+        cw_out = (cw == cw_b) ? cw_c : cw_b;
+        if (cur * 8 > (cw_out == cw_b ? len * 8 : len * 4)) cw_out = cw_b;  // (only level 1 needs the larger one)
+      }
+    }
+    // the next round's sums ride on the fold unless a class joins in between
+    const bool more = l < fl;
+    if ((status = launch_step(l, true, more && !joins, cw_out))) return status;
+    if (oracle) {  // an oracle tree over the folded codeword, its cap to the host behind a flag
       OracleTree o;
       o.level = l;
       o.cw_len = cur;
       o.nleaves = cur / 4;
       o.lc = cap_level_of(o.nleaves);
-      o.cw = mem.alloc(cur * 8);
+      o.cw = cw_out;
       o.levels = mem.alloc((2 * o.nleaves) * 8);
-      if (!o.cw || !o.levels) return E_NOMEM;
-      EXH_HIP(hipMemcpyAsync(o.cw, cw, cur * 32, hipMemcpyDeviceToDevice, c.stream));
-      std::vector<uint8_t> cap(32 * 128);
-      uint64_t rows = 0;
-      if ((status = merkle_tree_device(o.levels, o.nleaves, 2, o.cw, 1, o.cw_len, cap.data(), &rows))) return status;
+      if (!o.levels) return E_NOMEM;
+      uint64_t rows = 0, cap_off = 0;
+      if ((status = merkle_tree_launch(o.levels, o.nleaves, 2, o.cw, 1, o.cw_len, &rows, &cap_off))) return status;
+      const size_t cap_at = BF_MAX_ROUNDS * BF_ROUND_SLOT + cap_slots * BF_CAP_SLOT;
+      hipLaunchKernelGGL(deliver_kernel, dim3(1), dim3(BLOCK), 0, c.stream, o.levels + cap_off, (uint32_t)(8 * rows),
+                         reinterpret_cast<unsigned long long *>(pin_dev + cap_at), seq);
+      EXH_HIP(hipGetLastError());
+      cap_slots++;
+      std::vector<uint32_t> cap_words(8 * rows);
+      if (!await_words(c, reinterpret_cast<const volatile unsigned long long *>(pin + cap_at), 8 * rows, seq,
+                       cap_words.data())) {
+        set_error("device-error: a basefold oracle's cap did not arrive");
+        return E_DEVICE;
+      }
+      std::vector<uint8_t> cap(32 * rows);
+      memcpy(cap.data(), cap_words.data(), 32 * rows);
       if ((status = tr.send_bytes(cap.data(), (int64_t)(32 * rows), nullptr))) return status;
       oracles.push_back(o);
     }
-    for (int k = 0; k + 1 < ncls; k++)  // the classes that join at this level, :635-639
-      if (nv - cls[k] == l) {
-        const uint64_t clen = (uint64_t)1 << cls[k];
-        const uint32_t gl = (uint32_t)((clen + BLOCK - 1) / BLOCK);
-        scale_add_launch<8>(tt, d_hs[k], tt, clen, one8);
-        hipLaunchKernelGGL(split_coords_kernel, dim3(gl), dim3(BLOCK), 0, c.stream, d_hs[k], cols, clen);
-        if ((status = rs_encode_columns(cols, 8, cls[k], cwcols))) return status;
-        hipLaunchKernelGGL(join_coords_kernel, dim3(2 * gl), dim3(BLOCK), 0, c.stream, cwcols, cw2, 2 * clen);
-        scale_add_launch<8>(cw, cw2, cw, 2 * clen, one8);
-        ysum = hf::sub(ysum, yc[k]);
-      }
+    if (joins) {
+      for (int k = 0; k + 1 < ncls; k++)  // the classes that join at this level, :635-639
+        if (nv - cls[k] == l) {
+          const uint64_t clen = (uint64_t)1 << cls[k];
+          const uint32_t gl = (uint32_t)((clen + BLOCK - 1) / BLOCK);
+          uint32_t *tt_w = const_cast<uint32_t *>(tt), *cw_w = const_cast<uint32_t *>(cw);  // folded: ours to write
+          scale_add_launch<8>(tt_w, d_hs[k], tt_w, clen, one8);
+          if (l < fl) {
+            const uint32_t *cwk = d_cws ? d_cws[k] : nullptr;
+            if (!cwk) {  // ENCODE-EXT of the class's table, into a buffer of its own
+              uint32_t *joined = mem.alloc(2 * clen * 8);
+              if (!joined) return E_NOMEM;
+              hipLaunchKernelGGL(split_coords_kernel, dim3(gl), dim3(BLOCK), 0, c.stream, d_hs[k], cols, clen);
+              if ((status = rs_encode_columns(cols, 8, cls[k], cwcols))) return status;
+              hipLaunchKernelGGL(join_coords_kernel, dim3(2 * gl), dim3(BLOCK), 0, c.stream, cwcols, joined, 2 * clen);
+              cwk = joined;
+            }
+            if (oracle) {  // the oracle keeps the codeword it hashed: the sum goes to a buffer of its own
+              uint32_t *sum = mem.alloc(2 * clen * 8);
+              if (!sum) return E_NOMEM;
+              scale_add_launch<8>(cw, cwk, sum, 2 * clen, one8);
+              cw = sum;
+            } else {
+              scale_add_launch<8>(cw_w, cwk, cw_w, 2 * clen, one8);
+            }
+          }
+          ysum = hf::sub(ysum, yc[k]);
+        }
+      EXH_HIP(hipGetLastError());
+      if (more && (status = launch_step(l, false, true, nullptr))) return status;
+    }
   }
   // the final table in the clear, the final claim, grinding, the query positions
   uint64_t mlen = len >> fl;
   std::vector<uint32_t> m(mlen * 8);
+  EXH_HIP(hipMemcpyAsync(m.data(), tt, mlen * 32, hipMemcpyDeviceToHost, c.stream));
   EXH_HIP(hipStreamSynchronize(c.stream));
-  EXH_HIP(hipMemcpy(m.data(), tt, mlen * 32, hipMemcpyDeviceToHost));
   uint64_t dims[2] = {mlen, 8};
   if ((status = tr.send(m.data(), 2, dims, nullptr))) return status;
   if (out_final) memcpy(out_final, m.data(), mlen * 32);
@@ -1204,36 +1545,53 @@ int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, con
   std::vector<uint64_t> qs(queries);
   tr.challenge_bits(nv - 1, queries, qs.data());
   if (out_qs) memcpy(out_qs, qs.data(), 8 * (size_t)queries);
-  for (const OracleTree &o : oracles) {  // the oracle openings, recorded (src/pcs.lisp:651-655)
-    std::vector<uint64_t> leaf_off, path_off;
-    for (int q = 0; q < queries; q++) {
-      uint64_t li = qs[q] >> o.level;
-      for (int s = 0; s < 4; s++) leaf_off.push_back((4 * li + s) * 8);
-      uint64_t level_start = 0, n = o.nleaves, idx = li;
-      for (int d = 0; d < o.lc; d++) {
-        path_off.push_back((level_start + (idx ^ 1)) * 8);
-        level_start += n;
-        n /= 2;
-        idx >>= 1;
+  // ---- the oracle openings, recorded (src/pcs.lisp:651-655): every queried leaf's four symbols and every path's
+  // siblings of every oracle in one gather of 8-word segments and one copy back
+  if (!oracles.empty()) {
+    std::vector<const uint32_t *> segs;
+    for (const OracleTree &o : oracles)
+      for (int q = 0; q < queries; q++) {
+        const uint64_t li = qs[q] >> o.level;
+        for (int s = 0; s < 4; s++) segs.push_back(o.cw + (4 * li + s) * 8);
+        uint64_t level_start = 0, n = o.nleaves, idx = li;
+        for (int d = 0; d < o.lc; d++) {
+          segs.push_back(o.levels + (level_start + (idx ^ 1)) * 8);
+          level_start += n;
+          n /= 2;
+          idx >>= 1;
+        }
       }
+    const size_t nseg = segs.size();
+    uint32_t *d_ptrs = mem.alloc(nseg * 2 + 2), *d_out = mem.alloc(nseg * 8);
+    if (!d_ptrs || !d_out) return E_NOMEM;
+    std::vector<uint32_t> got(nseg * 8);
+    EXH_HIP(hipMemcpyAsync(d_ptrs, segs.data(), nseg * 8, hipMemcpyHostToDevice, c.stream));
+    hipLaunchKernelGGL(gather8_kernel, dim3((uint32_t)((nseg * 8 + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, c.stream,
+                       reinterpret_cast<const uint32_t *const *>(d_ptrs), (uint32_t)nseg, d_out);
+    EXH_HIP(hipGetLastError());
+    EXH_HIP(hipMemcpyAsync(got.data(), d_out, nseg * 32, hipMemcpyDeviceToHost, c.stream));
+    EXH_HIP(hipStreamSynchronize(c.stream));
+    size_t at = 0;
+    for (const OracleTree &o : oracles) {
+      std::vector<uint32_t> leaves((size_t)queries * 32);  // (Q, 8 rows, 4 symbols): row d holds coordinate d
+      std::vector<uint32_t> path;
+      for (int q = 0; q < queries; q++) {
+        for (int s = 0; s < 4; s++, at++)
+          for (int d = 0; d < 8; d++) leaves[((size_t)q * 8 + d) * 4 + s] = got[at * 8 + d];
+        for (int d = 0; d < o.lc; d++, at++) path.insert(path.end(), got.begin() + at * 8, got.begin() + at * 8 + 8);
+      }
+      uint64_t d3[3] = {(uint64_t)queries, 8, 4};
+      if ((status = tr.send(leaves.data(), 3, d3, nullptr, false))) return status;
+      if ((status = tr.send_bytes((const uint8_t *)path.data(), (int64_t)path.size() * 4, nullptr, false))) return status;
     }
-    std::vector<uint32_t> syms, path;
-    if ((status = gather_to_host(o.cw, leaf_off, 8, &syms))) return status;
-    if ((status = gather_to_host(o.levels, path_off, 8, &path))) return status;
-    std::vector<uint32_t> leaves((size_t)queries * 32);  // (Q, 8 rows, 4 symbols): row d holds coordinate d
-    for (int q = 0; q < queries; q++)
-      for (int d = 0; d < 8; d++)
-        for (int s = 0; s < 4; s++) leaves[((size_t)q * 8 + d) * 4 + s] = syms[((size_t)q * 4 + s) * 8 + d];
-    uint64_t d3[3] = {(uint64_t)queries, 8, 4};
-    if ((status = tr.send(leaves.data(), 3, d3, nullptr, false))) return status;
-    if ((status = tr.send_bytes((const uint8_t *)path.data(), (int64_t)path.size() * 4, nullptr, false))) return status;
   }
   return OK;
 }
 
 int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
-                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final) {
-  return basefold_prove_classes(tr, nv, 1, &nv, &d_h, rr, v, grind_bits, queries, out_qs, out_chal, out_final);
+                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final, const uint32_t *d_cw) {
+  return basefold_prove_classes(tr, nv, 1, &nv, &d_h, rr, v, grind_bits, queries, out_qs, out_chal, out_final,
+                                d_cw ? &d_cw : nullptr);
 }
 
 // The final opening over several size classes, one key per class, each a unit of its own with its own tree:
@@ -1251,7 +1609,7 @@ int pcs_open(Transcript &tr, int nv, int nkeys, const OpenClass *keys, const uin
   }
   Owned mem;
   std::vector<int> cls(nkeys);
-  std::vector<const uint32_t *> hs(nkeys);
+  std::vector<const uint32_t *> hs(nkeys), cws(nkeys, nullptr);
   for (int k = 0; k < nkeys; k++) {
     cls[k] = keys[k].c;
     if (keys[k].c < 1 || keys[k].c > 30 || keys[k].ncols < 1) {
@@ -1263,10 +1621,20 @@ int pcs_open(Transcript &tr, int nv, int nkeys, const OpenClass *keys, const uin
     if ((status = combine_columns_device(8, keys[k].d_columns, keys[k].ncols, (uint64_t)1 << keys[k].c, keys[k].coef, h)))
       return status;
     hs[k] = h;
+    // ENCODE-EXT of the combined column by the encoder's linearity: the same combination of the committed
+    // codewords (2^(c+1) symbols per column), no transform
+    if (keys[k].d_codewords) {
+      uint32_t *cwk = mem.alloc(((uint64_t)16) << keys[k].c);
+      if (!cwk) return E_NOMEM;
+      if ((status = combine_columns_device(8, keys[k].d_codewords, keys[k].ncols, (uint64_t)2 << keys[k].c,
+                                           keys[k].coef, cwk)))
+        return status;
+      cws[k] = cwk;
+    }
   }
   std::vector<uint64_t> qs(queries > 0 ? queries : 1);
   if ((status = basefold_prove_classes(tr, nv, nkeys, cls.data(), hs.data(), rr, v, grind_bits, queries, qs.data(),
-                                       nullptr, nullptr)))
+                                       nullptr, nullptr, cws.data())))
     return status;
   if (out_qs) memcpy(out_qs, qs.data(), 8 * (size_t)queries);
   for (int k = 0; k < nkeys; k++) {

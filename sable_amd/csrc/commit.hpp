@@ -36,14 +36,18 @@ int merkle_commit_columns(const uint32_t *d_codewords, int ncols, int c, uint32_
 // siblings up to the cap level (out_paths: count * depth * 32 bytes); leaves: count leaf indices below 2^(c-1)
 int open_queries_device(const uint32_t *d_codewords, int ncols, int c, const uint32_t *d_levels, const uint64_t *leaves,
                         int count, uint32_t *out_leaves, uint8_t *out_paths, int *out_depth);
+// d_cw (optional): ENCODE-EXT of the table (2^(nv+1) EXT8s on the device) when the caller has it already -- by the
+// encoder's linearity the same combination of the committed codewords as the table is of the committed columns
 int basefold_prove(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, const uint32_t *d_h, int grind_bits,
-                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final);
+                   int queries, uint64_t *out_qs, uint32_t *out_chal, uint32_t *out_final,
+                   const uint32_t *d_cw = nullptr);
 int basefold_verify(Transcript &tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits, int queries,
                     uint64_t *out_qs);
 // BASEFOLD over several size classes (ascending, the last one nv): class c's table d_hs[k] joins at level nv - c
+// d_cws (optional): per class its codeword as for basefold_prove, or null entries
 int basefold_prove_classes(Transcript &tr, int nv, int ncls, const int *cls, const uint32_t *const *d_hs,
                            const uint32_t *rr, const uint32_t *v, int grind_bits, int queries, uint64_t *out_qs,
-                           uint32_t *out_chal, uint32_t *out_final);
+                           uint32_t *out_chal, uint32_t *out_final, const uint32_t *const *d_cws = nullptr);
 // one key of the final opening: a size class, a unit of its own with its own tree
 struct OpenClass {
   int c = 0, ncols = 0;

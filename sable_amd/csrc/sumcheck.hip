@@ -396,6 +396,35 @@ int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out) {
   return OK;
 }
 
+// Eq tables over ranges of a point's variables, one launch: table k covers the variables [first[k], first[k] +
+// bits[k]) and lands at d_out + off[k] * D (2^bits[k] elements); d_factors holds (r_v R, (1 - r_v) R) per variable,
+// 2 n_vars D words.  At most 64 tables.  Enqueued on the context's stream; nothing is waited for.
+int eq_tables_launch(int D, int count, const int *first, const int *bits, const uint64_t *off,
+                     const uint32_t *d_factors, int n_vars, uint32_t *d_out) {
+  Context &c = ctx();
+  if (count < 1 || count > 64 || n_vars > MAXROUNDS || (D != 4 && D != 8)) {
+    set_error("invalid-parameter: eq tables (at most 64 tables over at most 48 variables)");
+    return E_PARAM;
+  }
+  EqTables eqt;
+  memset(&eqt, 0, sizeof(eqt));
+  eqt.count = count;
+  uint64_t total = 0;
+  for (int k = 0; k < count; k++) {
+    eqt.off[k] = off[k], eqt.first[k] = first[k], eqt.bits[k] = bits[k];
+    total += (uint64_t)1 << bits[k];
+  }
+  const uint32_t grid = (uint32_t)((total + BLOCK - 1) / BLOCK);
+  if (D == 4)
+    hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors,
+                       (uint32_t)(2 * n_vars * D), d_out, total, nullptr, (uint64_t)0);
+  else
+    hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, d_factors,
+                       (uint32_t)(2 * n_vars * D), d_out, total, nullptr, (uint64_t)0);
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
 static uint64_t tail_pairs(int T, int D);
 
 int SumcheckSession::launch_setup() {

@@ -26,6 +26,9 @@ struct KernelSet {  // the launchers generated for one statement and one degree 
 };
 // EQ-TABLE of k coordinates (canonical, host) into 2^k elements of device memory
 int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out);
+// eq tables over ranges of a point's variables in one launch (see sumcheck.hip)
+int eq_tables_launch(int D, int count, const int *first, const int *bits, const uint64_t *off,
+                     const uint32_t *d_factors, int n_vars, uint32_t *d_out);
 void register_kernels(const std::string &key, int D, KernelSet set);
 const KernelSet *find_kernels(const std::string &key, int D);
 

@@ -657,11 +657,12 @@ __device__ __forceinline__ void round_epilogue(Ctrl *ctrl, const uint32_t *sums,
 // *ok is false when a word did not complete within the spin limit.  scratch: groups * width words of LDS.
 // A launch may add only the words [add_first, add_first + add_count) (the passes of the base-field sweep share one
 // set of totals, a pass per range of words); the workgroup whose ticket is last_ticket is the elected one.
+// G: the workgroups that add to every word (the launch's grid, or the part of it that sums).
 __device__ __forceinline__ bool add_and_elect(const RoundTotals &rt, const uint32_t *mine, uint32_t width,
                                               uint32_t *scratch, uint32_t *sums, bool *ok, uint32_t add_first,
-                                              uint32_t add_count, uint32_t last_ticket) {
+                                              uint32_t add_count, uint32_t last_ticket, uint32_t G) {
   __shared__ uint32_t ticket;
-  const uint32_t tid = threadIdx.x, wg = blockIdx.x, G = gridDim.x, NG = rt.groups;
+  const uint32_t tid = threadIdx.x, wg = blockIdx.x, NG = rt.groups;
   for (uint32_t o = add_first + tid; o < add_first + add_count; o += blockDim.x)
     __hip_atomic_fetch_add(rt.totals + (size_t)(wg % NG) * rt.pstride + o, ((unsigned long long)1 << 48) + mine[o],
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -841,7 +842,7 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
   __syncthreads();
   bool ok;
   const uint32_t width = (uint32_t)d.nacc * D;
-  if (!add_and_elect(sh.totals, sums, width, epi.prod, sums, &ok, 0, width, gridDim.x - 1)) return;
+  if (!add_and_elect(sh.totals, sums, width, epi.prod, sums, &ok, 0, width, gridDim.x - 1, gridDim.x)) return;
   if (!ok) {
     if (tid == 0) __hip_atomic_store(&sh.ctrl->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
@@ -1552,7 +1553,7 @@ __device__ __forceinline__ void nodes_body(const Desc &d, const NodesArgs<D> &ar
   const int here = total - PASS * SPP < SPP ? total - PASS * SPP : SPP;  // slots of this pass
   bool ok;
   if (!add_and_elect(args.totals, L.sums, (uint32_t)total * D, L.epi.prod, L.slot_sums, &ok, (uint32_t)(PASS * SPP * D),
-                     (uint32_t)(here > 0 ? here : 0) * D, args.passes * gridDim.x - 1))
+                     (uint32_t)(here > 0 ? here : 0) * D, args.passes * gridDim.x - 1, gridDim.x))
     return;
   if (!ok) {
     if (tid == 0) __hip_atomic_store(&args.epi.e.ctrl->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -138,6 +138,29 @@ def test_basefold_matches_the_oracle(nv):
     t.free()
 
 
+@pytest.mark.parametrize("nv", [6, 11])
+def test_basefold_from_the_committed_codewords_matches_the_oracle(nv):
+    """The table is combine-columns of three committed columns; its codeword is handed over as the same combination
+    of their committed codewords (encoding is linear) instead of being encoded again: the oracle's bytes."""
+    rng = np.random.default_rng(100 + nv)
+    ncols = 3
+    cols = rng.integers(0, P, (ncols, 1 << nv), dtype=np.uint32)
+    cf = rng.integers(0, P, (ncols, 8), dtype=np.uint32)
+    rr = rng.integers(0, P, (nv, 8), dtype=np.uint32)
+    h = orc.combine_columns(cols, cf)
+    v = orc.mle_eval(h, rr, 8)
+    otr = orc.Transcript("bf", 4)
+    want = orc.basefold_prove(otr, nv, rr, v, h)
+    t = sa.Table.upload(cols.reshape(-1))
+    cw = sa.encode(t, ncols, nv)
+    th, tcw = sa.combine_columns(t, ncols, cf), sa.combine_columns(cw, ncols, cf)
+    tr = sa.Transcript("bf", 4)
+    got = sa.basefold_prove(tr, nv, rr, v, th, codeword=tcw)
+    assert tr.proof() == otr.proof() and got[0] == want[0]
+    for x in (t, cw, th, tcw):
+        x.free()
+
+
 def test_basefold_round_trip_beyond_the_oracle_sizes():
     """nv = 19 (the oracle stops near 12): the claim comes from the device's hypercube sum with eq = the
     point, the prover's own round checks pass, the verifier's BaseFold side accepts the proof (rounds, final

@@ -299,7 +299,14 @@ def test_basefold_config_at_full_size_against_the_oracles_digest(golden):
     assert sha(proof) == g["proof_sha256"], "config 5: the BaseFold proof at nv=23 differs from the oracle's"
     assert sa.basefold_verify(sa.Transcript(cm["open_label"], 4, proof=proof), c, rr, v, cm["grind_bits"],
                               cm["queries"]) == qs
-    for t in (cols, h):
+    # the same opening with the table's codeword taken from the commitment (the combination of the committed
+    # codewords, by the encoder's linearity) instead of eight transforms: the same bytes
+    cw = sa.encode(cols, ncols, c)
+    cwh = sa.combine_columns(cw, ncols, cf)
+    tr2 = sa.Transcript(cm["open_label"], 4)
+    qs2, _, _ = sa.basefold_prove(tr2, c, rr, v, h, grind_bits=cm["grind_bits"], queries=cm["queries"], codeword=cwh)
+    assert qs2 == qs and tr2.proof() == proof, "config 5: the opening from the committed codewords differs"
+    for t in (cols, h, cw, cwh):
         t.free()
 
 

@@ -21,6 +21,20 @@ def test_static_dot_pairs_matches_the_allocating_entry_point_twice_in_a_row():
         e.free(), v.free()
 
 
+def test_static_dot_pairs_matches_the_oracle_directly():
+    """Against the CPU oracle's dot-pairs itself (not only against the allocating entry point), after a larger call
+    has left its partial sums in the static array."""
+    from oracle import binding as orc
+    big_e, big_v = sa.Table.random(9701, 1 << 16, 8), sa.Table.random(9702, 1 << 16, 8)
+    sa.dot_pairs_static(big_e, big_v)
+    big_e.free(), big_v.free()
+    for length in (1 << 10, 6):
+        e, v = sa.Table.random(9600 + length, length, 8), sa.Table.random(9650 + length, length, 8)
+        he, hv = e.download().reshape(-1, 8), v.download().reshape(-1, 8)
+        assert np.array_equal(sa.dot_pairs_static(e, v), orc.dot_pairs(he, hv)), f"length {length}"
+        e.free(), v.free()
+
+
 def test_static_dot_pairs_refuses_what_it_cannot_hold():
     lib = sa.load()
     out = np.zeros((3, 8), np.uint32)
