@@ -155,10 +155,11 @@ int exh_combine_columns(exh_table columns, int ncols, uint64_t len, int degree_d
    of either by the round's challenge r (degree = the table's) -> a new table of half the length */
 int exh_dot_pairs(exh_table e, exh_table v, uint32_t *out);
 int exh_fold_table(exh_table table, const uint32_t *r, exh_table *out);
-/* exh_dot_pairs for callers that cannot allocate device memory while they run (code under HIP graph capture,
-   tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
-   arguments and result as exh_dot_pairs; the workgroups' partial sums live in a static 48 KiB device array that
-   each GPU holds until the process ends, and the call makes no hipMalloc, hipFree or other allocating call.
+/* exh_dot_pairs for callers that must not allocate device memory while they run (tight serving loops, harnesses
+   that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and result as exh_dot_pairs;
+   the workgroups' partial sums live in a static 48 KiB device array that each GPU holds until the process ends,
+   and the call makes no hipMalloc, hipFree or other allocating call.  Like every entry point it is synchronous
+   (it launches on the library's own stream and waits for its 24 words), so it cannot be recorded into a HIP graph.
    Tables of more than 2^26 EXT8s are refused (invalid-parameter).  Calls on one GPU share that GPU's array:
    calls that overlap on one GPU race. */
 int exh_dot_pairs_static(exh_table e, exh_table v, uint32_t *out);

@@ -289,6 +289,33 @@ def prove(tr, n, st, tables, eq=None, constants=None, label="sc", block_weights=
     return chal, finals, folded
 
 
+class ProveCall:
+    """`prove` with its arguments marshalled once: a host that proves the same statement over the same resident tables
+    again and again (a benchmark loop; an SBCL host holds its pinned vectors the same way) pays one foreign call per
+    proof instead of a dozen array conversions.  call(tr) -> (challenges, finals, folded) as `prove` returns them;
+    the arrays are the call's own and are overwritten by the next call."""
+
+    def __init__(self, n, st, tables, d, eq=None, constants=None, label="sc", block_weights=None, degree=None):
+        self.n, self.st, self.tables = n, st, list(tables)
+        self._eq, self._c, self._bw = _opt(eq, d), _consts(constants, d), _opt(block_weights, d)
+        self.K = len(self._bw) if self._bw is not None else 1
+        self.chal = np.zeros((n, d), np.uint32)
+        self.finals = np.zeros((len(tables), d), np.uint32)
+        self.folded = [np.zeros((self.K, d), np.uint32) for _ in tables]
+        self._fptr = (u32p * len(tables))(*[a.ctypes.data_as(u32p) for a in self.folded])
+        self._label = _bytes(label)
+        self._args = (C.c_int(n), C.c_uint64(st.handle), _handles(tables), C.c_int(len(tables)), _p(self._eq),
+                      _p(self._c), self._label, C.c_uint64(len(self._label)), _p(self._bw), C.c_int(self.K),
+                      C.c_int(-1 if degree is None else degree), _p(self.chal), _p(self.finals), self._fptr)
+        self._fn = load().exh_prove
+
+    def __call__(self, tr):
+        status = self._fn(C.c_uint64(tr.handle), *self._args)
+        if status:
+            check(status)
+        return self.chal, self.finals, self.folded
+
+
 def verify(tr, n, st, claim, eq=None, constants=None, blocks=1, label="sc", degree=None):
     d = tr.degree
     eqa, ca, claim = _opt(eq, d), _consts(constants, d), _u32(claim)

@@ -94,6 +94,9 @@ int exh_init(int device) {
 }
 void exh_shutdown(void) {
   ApiLock api_lock;
+  // a compilation still running is waited for here, so that a host that shuts the library down before it exits
+  // keeps its own exit handlers (the hard exit of rtc.cpp is for a process that ends without this call)
+  (void)rtc_idle(true);
   g_sessions.clear();
   ctx_shutdown();
 }
@@ -735,6 +738,10 @@ struct TreeCall {
 int prepare_tree(const exh_gkr_tree &t, TreeCall *call) {
   call->tr = tr_of(t.tr);
   if (!call->tr) return E_PARAM;
+  if (t.lookups < 1 || t.lookups > MAXT / 4 || t.n < 0 || t.n > 30 || t.K < 1 || !t.leaves) {
+    set_error("invalid-parameter: GKR shape (lookups, n, K, leaves)");
+    return E_PARAM;
+  }
   std::vector<int> strides;
   int status = gather_tables(t.leaves, 2 * t.lookups, call->tr->D, (uint64_t)t.K << t.n, &call->ptrs, &strides);
   if (status) return status;
@@ -747,8 +754,16 @@ int prepare_tree(const exh_gkr_tree &t, TreeCall *call) {
   return OK;
 }
 int run_tree(const exh_gkr_tree &t, TreeCall &call) {
-  return gkr_prove_upper(*call.tr, t.n, t.K, t.lookups, call.ptrs.data(), call.label, t.out_ri, t.out_rb, t.out_cp,
-                         t.out_cq);
+  try {  // (nothing may leave a thread's body as an exception: a proof of 2^22 leaves holds large host vectors)
+    return gkr_prove_upper(*call.tr, t.n, t.K, t.lookups, call.ptrs.data(), call.label, t.out_ri, t.out_rb, t.out_cp,
+                           t.out_cq);
+  } catch (const std::bad_alloc &) {
+    set_error("device-out-of-memory: host memory ran out during prove-upper");
+    return E_NOMEM;
+  } catch (const std::exception &e) {
+    set_error(std::string("device-error: prove-upper: ") + e.what());
+    return E_DEVICE;
+  }
 }
 }  // namespace
 
@@ -779,16 +794,30 @@ int exh_gkr_prove_upper_pair(exh_gkr_tree *first, exh_gkr_tree *second) {
     EXH_HIP(recorded);
   }
   std::string second_error;
-  main_context.share = side->share = 2;
-  std::thread worker([&] {
-    use_context(side);
-    second->status = hipSetDevice(side->device) == hipSuccess ? run_tree(*second, b) : E_DEVICE;
-    if (second->status) second_error = last_error();
-    use_context(nullptr);
-  });
-  first->status = run_tree(*first, a);
-  worker.join();
-  main_context.share = side->share = 1;
+  struct Shared {  // both proofs' grids take half the device while they run side by side; whole again on every way out
+    Context &one, &other;
+    Shared(Context &a, Context &b) : one(a), other(b) { one.share = other.share = 2; }
+    ~Shared() { one.share = other.share = 1; }
+  };
+  {
+    Shared shared(main_context, *side);
+    second->status = E_DEVICE;
+    std::thread worker;
+    try {
+      worker = std::thread([&] {
+        use_context(side);
+        second->status = hipSetDevice(side->device) == hipSuccess ? run_tree(*second, b) : E_DEVICE;
+        if (second->status) second_error = last_error();
+        use_context(nullptr);
+      });
+    } catch (const std::exception &e) {  // no second thread: one tree after the other
+      first->status = run_tree(*first, a);
+      second->status = first->status ? first->status : run_tree(*second, b);
+      return first->status ? first->status : second->status;
+    }
+    first->status = run_tree(*first, a);
+    worker.join();
+  }
   if (first->status) return first->status;
   if (second->status) set_error(second_error);
   return second->status;

@@ -224,6 +224,21 @@ void end_of_process(int status, void *) {
           if (t.joinable()) t.join();
   }
   if (compiling) {
+    // a short grace for a compilation about to end (the ordinary exit then goes on); beyond it the hard exit
+    for (int waited_ms = 0; waited_ms < 2000 && compiling; waited_ms += 50) {
+      std::this_thread::sleep_for(std::chrono::milliseconds(50));
+      compiling = false;
+      std::lock_guard<std::mutex> lock(g_mutex);
+      for (auto &kv : g_jobs)
+        if (kv.second->running.load() > 0) compiling = true;
+    }
+    if (!compiling) {
+      std::lock_guard<std::mutex> lock(g_mutex);
+      for (auto &kv : g_jobs)
+        for (std::thread &t : kv.second->threads)
+          if (t.joinable()) t.join();
+      return;
+    }
     fflush(nullptr);
     _exit(status);
   }

@@ -1054,7 +1054,9 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     volatile uint32_t *flag = reinterpret_cast<volatile uint32_t *>(down) + ctrl_words;
     uint32_t spins = 0;
     while (*flag != c.log_seq) {
-      if ((++spins & 1023) == 0 && hipStreamQuery(c.stream) == hipSuccess) break;
+      // (any answer but "not ready" ends the polling: a stream in an error state never raises the flag, and the
+      // wait below reports what happened)
+      if ((++spins & 1023) == 0 && hipStreamQuery(c.stream) != hipErrorNotReady) break;
     }
     if (*flag != c.log_seq) {
       EXH_HIP(hipStreamSynchronize(c.stream));
