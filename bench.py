@@ -185,6 +185,11 @@ def run_sumcheck(sa, name, steps, warmup, gold, n=None):
     streaming = {k: v for k, v in by.items() if k[0].startswith("round_")} or by
     (kname, kround), (avg_ms, per, kbytes) = max(streaming.items(), key=lambda kv: kv[1][0] * kv[1][1])
     achieved = kbytes / (avg_ms * 1e-3) / 1e9
+    note = None
+    if kname == "round_nodes_base":
+        note = ("the launch stands for rounds 0 and 1: its algorithmic bytes are the two reads of the base tables "
+                "those rounds' units take (round 0's sums, the read side of fold 1: T * 2^n * 8), shared among its "
+                "passes; a pass moves one read of them, which is what `traffic` measures")
     return {"workload": f"sumcheck prove of {cfg['form']}, eq mode, n={n}, {T} base tables of 2^{n}, F_p^{d}, BLAKE3 "
                         "transcript", "n": n, "tables": T, "extension": d, "degree": st.degree,
             "ms_per_step": 1e3 * dt, "entries_per_s": T * (1 << n) / dt, "proof_bytes": len(proof),
@@ -193,7 +198,7 @@ def run_sumcheck(sa, name, steps, warmup, gold, n=None):
             "loop_hbm_fraction": T * (1 << n) * (8 + 8 * d) / dt / (HBM_PEAK_GBS * 1e9),
             "roofline": {"bound": "hbm", "kernel": f"{kname} (round {kround})", "achieved": achieved,
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "avg_launch_ms": avg_ms,
-                         "launches_per_step": per, "alg_bytes_per_launch": kbytes, "traffic": None},
+                         "launches_per_step": per, "alg_bytes_per_launch": kbytes, "traffic": None, "note": note},
             "roofline_by_time": by_time(by)}
 
 

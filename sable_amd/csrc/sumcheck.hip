@@ -551,13 +551,19 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
 // [deg][m] = 1 / prod_{q != m, q <= deg} (m - q), in Montgomery form: the denominators of the Lagrange basis
 // over the nodes 0..deg
 static void fill_inv_den(uint32_t *out) {
-  for (int deg = 1; deg <= MAXDEG; deg++)
-    for (int m = 0; m <= deg; m++) {
-      uint32_t den = 1;
-      for (int q = 0; q <= deg; q++)
-        if (q != m) den = fmul(den, m > q ? (uint32_t)(m - q) : P - (uint32_t)(q - m));
-      out[deg * (MAXDEG + 1) + m] = to_mont(finv(den));
-    }
+  // computed once: forty-nine field inversions on the host are ten microseconds between two launches of a prove
+  static const std::vector<uint32_t> table = [] {
+    std::vector<uint32_t> t((MAXDEG + 1) * (MAXDEG + 1), 0);
+    for (int deg = 1; deg <= MAXDEG; deg++)
+      for (int m = 0; m <= deg; m++) {
+        uint32_t den = 1;
+        for (int q = 0; q <= deg; q++)
+          if (q != m) den = fmul(den, m > q ? (uint32_t)(m - q) : P - (uint32_t)(q - m));
+        t[deg * (MAXDEG + 1) + m] = to_mont(finv(den));
+      }
+    return t;
+  }();
+  memcpy(out, table.data(), table.size() * 4);
 }
 
 // Rounds 0 and 1 from one sweep of the base tables (nothing folded): the slot sums in as many launches as the
@@ -607,8 +613,11 @@ static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs) {
       EXH_HIP(hipMemsetAsync(a.totals.arrivals, 0, 4, c.stream));
     }
   }
+  // (the bytes the sweep is credited with when launches are timed: the two reads of the base tables it stands for,
+  // round 0's sums and the fold that would have produced round 1's tables, shared among its passes; a pass moves
+  // one read of them)
   for (int pass = 0; pass < s.kernels->nodes_passes; pass++) {
-    c.prof_begin("round_nodes_base", 0, (uint64_t)T * 16 * n_pairs);
+    c.prof_begin("round_nodes_base", 0, (uint64_t)T * 32 * n_pairs / (uint64_t)s.kernels->nodes_passes);
     s.kernels->launch_nodes(&a, pass, grid, c.stream);
     c.prof_end();
   }
