@@ -202,6 +202,40 @@ def run_sumcheck(sa, name, steps, warmup, gold, n=None):
             "roofline_by_time": by_time(by)}
 
 
+def run_domain(sa, steps, warmup, n=None):
+    """A statement wider than the table groups' kernels (workloads.SUMCHECK["domain"]): proved in one device-driven
+    session by the kernels of its direct form, which are compiled before the clock starts; the proof is verified and
+    compared with the one the same library gives when it deals the statement into parts (the way the parity tests
+    hold to the oracle's bytes), which is timed beside it."""
+    cfg, n, d, T, st, dev, eq, cv, step = sumcheck_setup(sa, "domain", n)
+    if not st.generate(d, wait=True):
+        sys.exit("bench.py: the kernels of the domain statement's direct form did not compile")
+    dt, (tr, finals) = timed(sa, step, steps, warmup)
+    proof, _ = sumcheck_checked(sa, "domain", n, d, st, dev, eq, cv, tr, finals, {})
+    by = launches(sa, step, max(2, min(steps, 5)))
+    os.environ["EXACTA_HIP_NO_DIRECT"] = "1"
+    try:
+        dt_parts, (tr_parts, _) = timed(sa, step, max(2, steps // 4), 1)
+    finally:
+        del os.environ["EXACTA_HIP_NO_DIRECT"]
+    if tr_parts.proof() != proof:
+        sys.exit("bench.py: the direct form's proof differs from the proof in parts")
+    for t in dev:
+        t.free()
+    nbytes = T * (1 << n) * (8 + 8 * d)
+    return {"workload": f"sumcheck prove of the toy domain's leaf-layer and zerocheck statement (41 table monomials, "
+                        f"degree {st.degree}), eq mode, n={n}, {T} base tables of 2^{n}, F_p^{d}, BLAKE3 transcript",
+            "n": n, "tables": T, "extension": d, "degree": st.degree, "ms_per_step": 1e3 * dt,
+            "ms_per_step_in_parts": 1e3 * dt_parts, "entries_per_s": T * (1 << n) / dt, "proof_bytes": len(proof),
+            "proof_sha256": sha(proof), "proof_is_the_parts_paths": True, "verifier_accepts": True,
+            "timed_launches_per_step": sum(per for _, per, _ in by.values()),
+            "loop_hbm_fraction": nbytes / dt / (HBM_PEAK_GBS * 1e9),
+            "roofline": {"bound": "hbm", "kernel": "whole round loop", "achieved": nbytes / dt / 1e9,
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / dt / 1e9 / HBM_PEAK_GBS,
+                         "alg_bytes": nbytes, "traffic": None},
+            "roofline_by_time": by_time(by)[:8]}
+
+
 # ------------------------------------------------------------------ config 4: LogUp-GKR
 def run_gkr(sa, steps, warmup, gold):
     g = wl.GKR
@@ -510,8 +544,8 @@ SEEDED = "synthetic (SplitMix64-seeded uniform field elements)"
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="config2",
-                    choices=["config1", "config2", "config3", "config4", "config5", "basefold", "combine", "combine128",
-                             "copy", "mulrate"],
+                    choices=["config1", "config2", "config3", "config4", "config5", "basefold", "domain", "combine",
+                             "combine128", "copy", "mulrate"],
                     help="config2 (default) is the headline; the others are the remaining configured workloads; "
                          "copy is the known-size kernel the traffic counters are calibrated on")
     ap.add_argument("--gpus", type=int, default=1)
@@ -536,6 +570,12 @@ def main():
         d = res["extension"]
         print(json.dumps(line(f"sumcheck table entries/s ({args.workload})", res["entries_per_s"], "table entries/s", True,
                               f"u32 (Montgomery KoalaBear, F_p^{d} tower)", SEEDED, res, steps, warmup)))
+        return
+    if args.workload == "domain":
+        res = run_domain(sa, steps, warmup, n)
+        print(json.dumps(line("sumcheck table entries/s (wide statement, direct form)", res["entries_per_s"],
+                              "table entries/s", True, "u32 (Montgomery KoalaBear, F_p^4 tower)", SEEDED, res, steps,
+                              warmup)))
         return
     if args.workload == "config4":
         res = run_gkr(sa, steps, warmup, gold)

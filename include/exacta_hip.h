@@ -57,7 +57,11 @@ int exh_stmt_has_generated_kernel(exh_stmt stmt, int degree_d);
    registered before the library's first compilation skipped).
    exh_stmt_generate asks for that compilation ahead of a proof, for round polynomials of the given header degree
    (-1: the statement's own).  Returns 1 when the kernels are in place, 0 while they compile (wait = 0), or
-   EXH_E_DEVICE with the compiler's log when the compilation failed; with wait != 0 it returns once it has ended. */
+   EXH_E_DEVICE with the compiler's log when the compilation failed; with wait != 0 it returns once it has ended.
+   A statement too wide for the table groups' kernels (more than 16 table monomials or 36 accumulators) gets the
+   kernels of its direct form instead, which evaluate the written form at every wire point (the role of
+   COMPILE-FORM, src/forms.lisp:144-186): with them exh_prove proves it in one device-driven session; without them
+   (not compiled yet, or EXACTA_HIP_NO_DIRECT=1) in parts proved in step, the same bytes. */
 int exh_stmt_generate(exh_stmt stmt, int degree_d, int degree, int wait);
 /* 1 when no compilation is running, 0 while one is; with wait != 0 it returns 1 once none is (a host that wants an
    orderly exit calls it before it ends: see above) */

@@ -48,7 +48,8 @@ int exh_transcript_message_count(exh_transcript tr, uint64_t *count);
 int exh_transcript_proof(exh_transcript tr, uint8_t *out, uint64_t cap, uint64_t *out_len);
 
 /* ---- sumcheck (src/sumcheck.lisp) */
-/* HYPERCUBE-SUM, :112-127: the honest claim, computed on the device */
+/* HYPERCUBE-SUM, :112-127: the honest claim, computed on the device (a statement wider than one kernel holds: the
+   sum of its parts' claims) */
 int exh_hypercube_sum(exh_stmt stmt, int degree_d, int n, const exh_table *tables, int n_tables,
                       const uint32_t *eq, const uint32_t *constants, uint32_t *out);
 /* PROVE, :512-571.  out_challenges: n * D; out_finals: n_tables * D; out_folded: NULL or n_tables

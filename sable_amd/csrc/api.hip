@@ -286,7 +286,12 @@ int exh_stmt_has_generated_kernel(exh_stmt stmt, int D) {
   Statement copy = *st;
   copy.plan(copy.degree > 1 ? copy.degree : 1);
   if (ctx().ready) (void)rtc_collect();
-  return find_kernels(copy.key(), D) ? 1 : 0;
+  if (find_kernels(copy.key(), D)) return 1;
+  StmtDesc desc;
+  Statement direct;  // a statement too wide for the table groups' kernels: those of its direct form
+  if ((copy.T() > MAXT || !make_desc(copy, &desc)) && make_direct(*st, copy.degree > 1 ? copy.degree : 1, &direct))
+    return find_kernels(direct.key(), D) ? 1 : 0;
+  return 0;
 }
 int exh_stmt_generate_idle(int wait) {
   ApiLock api_lock;
@@ -308,8 +313,16 @@ int exh_stmt_generate(exh_stmt stmt, int D, int degree, int wait) {
   if (find_kernels(copy.key(), D)) return 1;
   StmtDesc desc;
   if (copy.T() > MAXT || !make_desc(copy, &desc)) {
-    set_error("invalid-parameter: statement beyond the kernels' limits");
-    return E_PARAM;
+    // too wide for accumulators per table group: the kernels of its direct form, which evaluate the written
+    // form itself at every wire point
+    Statement direct;
+    if (!make_direct(*st, degree > 1 ? degree : 1, &direct) || !make_desc(direct, &desc)) {
+      set_error("invalid-parameter: statement beyond the kernels' limits");
+      return E_PARAM;
+    }
+    if (find_kernels(direct.key(), D)) return 1;
+    rtc_request(direct.key(), desc, D, direct_source(direct, desc, "RtStmt"));
+    return rtc_status(direct.key(), D, wait != 0);
   }
   rtc_request(copy.key(), desc, D);
   return rtc_status(copy.key(), D, wait != 0);
@@ -575,7 +588,10 @@ int exh_hypercube_sum(exh_stmt stmt, int D, int n, const exh_table *tables, int 
     return OK;
   }
   SumcheckSession s;
-  if ((status = s.begin(*st, D, n, ptrs.data(), strides.data(), eq, nullptr, 1, constants, -1, true))) return status;
+  status = s.begin(*st, D, n, ptrs.data(), strides.data(), eq, nullptr, 1, constants, -1, true);
+  if (status == E_PARAM && s.beyond_limits)
+    return hypercube_sum_wide(*st, D, n, ptrs.data(), strides.data(), eq, constants, out);
+  if (status) return status;
   uint32_t sums[16 * 8];
   if ((status = s.round_sums(sums))) return status;
   memcpy(out, sums, 4 * D);

@@ -448,6 +448,7 @@ static void choose_shape(Statement *st, int points) {
 }
 
 void Statement::plan(int points) {
+  if (direct) return;  // made for its wire points already
   if (planned_points == points) return;
   planned_points = points;
   choose_shape(this, points);
@@ -459,6 +460,7 @@ void Statement::plan_claim() {
 }
 
 std::string Statement::key() const {
+  if (direct) return direct_key;
   std::string k = "T" + std::to_string(T()) + ":";
   for (const Linear &l : linear) {
     k += "(";
@@ -505,6 +507,15 @@ bool make_desc(const Statement &st, StmtDesc *out) {
   StmtDesc d;
   memset(&d, 0, sizeof(d));
   d.T = st.T();
+  if (st.direct) {  // no groups: the wire points are the accumulators
+    if (d.T < 1 || d.T > MAXT || st.nacc > MAXEV || st.groups.size() != 1) return false;
+    d.nacc = st.nacc;
+    d.nev[0] = st.nacc;
+    for (int k = 0; k < st.nacc; k++) d.ev[0][k] = st.groups[0].evalx[(size_t)k];
+    d.maxx = st.groups[0].evalx.back();
+    *out = d;
+    return true;
+  }
   d.NV = (int)st.linear.size();
   if (d.T < 1 || d.NV > MAXV || d.T + d.NV > MAXT || st.nacc > MAXACC) return false;
   for (int v = 0; v < d.NV; v++) {
@@ -576,6 +587,241 @@ std::string desc_source(const StmtDesc &d, const std::string &name) {
   o << "},\n    {";
   for (int v = 0; v < MAXV; v++) o << d.vconst[v] << "u" << (v + 1 < MAXV ? "," : "");
   o << "}};\n};\n";
+  return o.str();
+}
+
+// ---- the direct form
+namespace {
+
+// One walk of the written form serves both the code and the constants: it numbers the constant slots in the order
+// it meets them, so the values are computed by the same walk with the constants at hand.
+struct DirectWalk {
+  const Statement &st;
+  std::ostringstream code;
+  int vars = 0, slots = 0;
+  bool failed = false;
+  std::map<std::string, std::string> seen;  // a subform's text -> the variable that holds it
+  // evaluation of the slots (when const_vals is set)
+  int D = 0;
+  const uint32_t *const_vals = nullptr;
+  std::vector<hf::E> values;
+
+  explicit DirectWalk(const Statement &s) : st(s) {}
+  int find(const std::vector<std::string> &names, const std::string &v) const {
+    auto it = std::find(names.begin(), names.end(), v);
+    return it == names.end() ? -1 : (int)(it - names.begin());
+  }
+  std::string text(const Node &n) const {
+    if (n.kind == Node::INT) return std::to_string(n.value);
+    if (n.kind == Node::VAR) return n.name;
+    std::string s = "(" + n.name;
+    for (auto &a : n.args) s += " " + text(*a);
+    return s + ")";
+  }
+  bool table_free(const Node &n) const {
+    if (n.kind == Node::INT) return true;
+    if (n.kind == Node::VAR) return find(st.tables, n.name) < 0;
+    if (n.name == "EXPT" && n.args.size() == 2 && n.args[1]->kind == Node::INT && n.args[1]->value == 0) return true;
+    for (auto &a : n.args)
+      if (!table_free(*a)) return false;
+    return true;
+  }
+  bool integer_only(const Node &n) const {  // no named constant: an integer mod p, a base-field scalar
+    if (n.kind == Node::INT) return true;
+    if (n.kind == Node::VAR) return false;
+    for (auto &a : n.args)
+      if (!integer_only(*a)) return false;
+    return true;
+  }
+  hf::E value(const Node &n) {  // of a table-free subform, at the constants
+    if (n.kind == Node::INT) return hf::lift((uint32_t)n.value, D);
+    if (n.kind == Node::VAR) {
+      int ci = find(st.constants, n.name);
+      if (ci < 0) {
+        failed = true;
+        return hf::zero(D);
+      }
+      return hf::from(const_vals + (size_t)ci * D, D);
+    }
+    if (n.name == "+" || n.name == "-") {
+      hf::E acc = hf::zero(D);
+      for (size_t i = 0; i < n.args.size(); i++) {
+        bool negate = n.name == "-" && (n.args.size() == 1 || i > 0);
+        acc = negate ? hf::sub(acc, value(*n.args[i])) : hf::add(acc, value(*n.args[i]));
+      }
+      return acc;
+    }
+    if (n.name == "*") {
+      hf::E acc = hf::lift(1, D);
+      for (auto &a : n.args) acc = hf::mul(acc, value(*a));
+      return acc;
+    }
+    if (n.name == "EXPT" && n.args.size() == 2 && n.args[1]->kind == Node::INT) {
+      hf::E acc = hf::lift(1, D), base = n.args[1]->value ? value(*n.args[0]) : hf::zero(D);
+      for (long long i = 0; i < n.args[1]->value; i++) acc = hf::mul(acc, base);
+      return acc;
+    }
+    failed = true;
+    return hf::zero(D);
+  }
+  // a constant slot for the sum (signs) or the product of table-free subforms
+  std::map<std::string, int> slot_of;        // a slot's text -> its number (a constant met again is the same slot)
+  std::map<int, std::string> slot_variable;  // slots already loaded into a variable
+  int slot(const std::vector<std::pair<const Node *, bool>> &items, bool product) {
+    std::string key = product ? "*" : "+";
+    for (auto &it : items) key += (it.second ? " -" : " +") + text(*it.first);
+    auto hit = slot_of.find(key);
+    if (hit != slot_of.end()) return hit->second;
+    slot_of[key] = slots;
+    if (const_vals) {
+      hf::E acc = product ? hf::lift(1, D) : hf::zero(D);
+      for (auto &it : items) {
+        hf::E v = value(*it.first);
+        acc = product ? hf::mul(acc, v) : (it.second ? hf::sub(acc, v) : hf::add(acc, v));
+      }
+      values.push_back(acc);
+    }
+    return slots++;
+  }
+  std::string fresh() { return "v" + std::to_string(vars++); }
+  std::string load_slot(int k) {
+    auto hit = slot_variable.find(k);
+    if (hit != slot_variable.end()) return hit->second;
+    std::string v = fresh();
+    code << "    const Ext<D> " << v << " = load_ext<D>(kc + " << k << " * D);\n";
+    slot_variable[k] = v;
+    return v;
+  }
+  // the variable holding the subform's value (Montgomery form)
+  std::string gen(const Node &n) {
+    if (table_free(n)) return load_slot(slot({{&n, false}}, false));
+    if (n.kind == Node::VAR) return "t[" + std::to_string(find(st.tables, n.name)) + "]";
+    const std::string key = text(n);
+    auto hit = seen.find(key);
+    if (hit != seen.end()) return hit->second;
+    std::string out;
+    if (n.name == "+" || n.name == "-") {
+      std::vector<std::pair<const Node *, bool>> consts;
+      for (size_t i = 0; i < n.args.size(); i++) {
+        const bool negate = n.name == "-" && (n.args.size() == 1 || i > 0);
+        if (table_free(*n.args[i])) {
+          consts.push_back({n.args[i].get(), negate});
+          continue;
+        }
+        const std::string a = gen(*n.args[i]);
+        const std::string v = fresh();
+        if (out.empty())
+          code << "    const Ext<D> " << v << " = " << (negate ? "ext_sub<D>(ext_zero<D>(), " + a + ")" : a) << ";\n";
+        else
+          code << "    const Ext<D> " << v << " = " << (negate ? "ext_sub<D>(" : "ext_add<D>(") << out << ", " << a << ");\n";
+        out = v;
+      }
+      if (!consts.empty()) {
+        const std::string k = load_slot(slot(consts, false)), v = fresh();
+        code << "    const Ext<D> " << v << " = ext_add<D>(" << out << ", " << k << ");\n";
+        out = v;
+      }
+    } else if (n.name == "*") {
+      std::vector<std::pair<const Node *, bool>> consts;
+      bool integers = true;
+      for (auto &arg : n.args) {
+        if (table_free(*arg)) {
+          consts.push_back({arg.get(), false});
+          integers = integers && integer_only(*arg);
+          continue;
+        }
+        const std::string a = gen(*arg);
+        if (out.empty()) {
+          out = a;
+          continue;
+        }
+        const std::string v = fresh();
+        code << "    const Ext<D> " << v << " = ext_mul_mont<D>(" << out << ", " << a << ");\n";
+        out = v;
+      }
+      if (!consts.empty()) {
+        const int k = slot(consts, true);
+        std::string v;
+        if (!integers) (void)load_slot(k);  // (its line comes before the product's)
+        v = fresh();
+        if (integers)  // a base-field scalar: its Montgomery form is the slot's first word
+          code << "    const Ext<D> " << v << " = ext_scale_mont<D>(" << out << ", kc[" << k << " * D]);\n";
+        else {
+          const std::string kv = load_slot(k);
+          code << "    const Ext<D> " << v << " = ext_mul_mont<D>(" << out << ", " << kv << ");\n";
+        }
+        out = v;
+      }
+    } else if (n.name == "EXPT" && n.args.size() == 2 && n.args[1]->kind == Node::INT && n.args[1]->value >= 1 &&
+               n.args[1]->value <= MAXDEG) {
+      const std::string a = gen(*n.args[0]);
+      out = a;
+      for (long long i = 1; i < n.args[1]->value; i++) {
+        const std::string v = fresh();
+        code << "    const Ext<D> " << v << " = ext_mul_mont<D>(" << out << ", " << a << ");\n";
+        out = v;
+      }
+    } else {
+      failed = true;
+      return "t[0]";
+    }
+    seen[key] = out;
+    return out;
+  }
+};
+
+}  // namespace
+
+bool make_direct(const Statement &st, int points, Statement *out) {
+  if (st.T() < 1 || st.T() > MAXT || points < 1 || points > MAXEV || points + 1 > MAXX + 1) return false;
+  Parser parser(st.text);
+  auto root = parser.parse();
+  if (!parser.ok || !root) return false;
+  DirectWalk walk(st);
+  const std::string result = walk.gen(*root);
+  if (walk.failed) return false;
+  Statement d = st;
+  d.direct = true;
+  d.direct_code = walk.code.str() + "    return " + result + ";\n";
+  d.direct_slots = walk.slots;
+  d.expanded_groups.clear(), d.factored_groups.clear(), d.factored_linear.clear(), d.linear.clear();
+  Group g;
+  g.tabs = {0};  // (not the constant group)
+  g.parts.push_back(Group::Part{1u, {}});
+  for (int k = 0; k < points; k++) g.evalx.push_back(k == 0 ? 0 : k + 1);
+  g.acc_base = 0;
+  d.groups = {g};
+  d.nacc = points;
+  d.planned_points = points;
+  d.direct_key = "direct:" + std::to_string(points) + "|";
+  for (auto &t : st.tables) d.direct_key += t + ",";
+  d.direct_key += "|";
+  for (auto &c : st.constants) d.direct_key += c + ",";
+  d.direct_key += "|" + walk.text(*root);
+  *out = d;
+  return true;
+}
+
+void direct_slot_values(const Statement &st, int D, const uint32_t *const_vals, uint32_t *out) {
+  Parser parser(st.text);
+  auto root = parser.parse();
+  DirectWalk walk(st);
+  walk.D = D, walk.const_vals = const_vals;
+  (void)walk.gen(*root);
+  for (size_t k = 0; k < walk.values.size(); k++) memcpy(out + k * D, walk.values[k].data(), 4 * (size_t)D);
+}
+
+std::string direct_source(const Statement &st, const StmtDesc &d, const std::string &name) {
+  // the descriptor's initialiser as desc_source writes it, inside a type that carries the evaluator
+  std::string plain = desc_source(d, name);
+  const size_t from = plain.find("= {") + 2, to = plain.rfind("};\n};");
+  const std::string init = plain.substr(from, to - from + 1);
+  std::ostringstream o;
+  o << "struct " << name << "Desc : StmtDesc {\n  static constexpr bool direct = true;\n"
+    << "  // the statement at the tables' values t (Montgomery form) with the constant slots kc (Montgomery form)\n"
+    << "  template <int D>\n  static __device__ __forceinline__ Ext<D> eval(const Ext<D> *t, const uint32_t *kc) {\n"
+    << st.direct_code << "  }\n};\n"
+    << "struct " << name << " {\n  static constexpr " << name << "Desc d = {" << init << "};\n};\n";
   return o.str();
 }
 

@@ -68,7 +68,24 @@ struct Statement {
   void plan_claim();
   int planned_points = -1;
   std::string key() const;  // canonical description of the table groups, for kernel lookup
+  // A statement in direct form (make_direct): no groups of table monomials; the kernels evaluate the written form
+  // itself at every wire point, into one accumulator per point.  `groups` then holds one stand-in group with
+  // coefficient 1 whose accumulators are the wire points.
+  bool direct = false;
+  std::string direct_code;  // the body of the generated evaluator: statements ending in `return v<N>;`
+  int direct_slots = 0;     // its constant slots: table-free subforms, evaluated on the host for every proof
+  std::string direct_key;
 };
+
+// The statement as a kernel evaluates it when it is too wide for the groups' accumulators: the written form as
+// straight-line code over the tables' values at a point (every value in Montgomery form), table-free subforms
+// collapsed into constant slots, repeated subforms computed once.  POINTS wire points (X = 0, 2, 3, ...).
+// False when the form has more than MAXT tables or more than MAXEV wire points.
+bool make_direct(const Statement &st, int points, Statement *out);
+// the direct statement's constant slots at the constants' values: out[slot * D ..), canonical
+void direct_slot_values(const Statement &st, int D, const uint32_t *const_vals, uint32_t *out);
+// `struct <name>` for a direct statement: the descriptor with its evaluator
+std::string direct_source(const Statement &st, const StmtDesc &d, const std::string &name);
 
 int compile_statement(const std::string &text, const std::vector<std::string> &tables,
                       const std::vector<std::string> &constants, Statement *out);

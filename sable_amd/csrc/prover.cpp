@@ -52,24 +52,22 @@ int adopt_device_state(Transcript &tr, const DevB3S &state) {
 // fit: the monomials are dealt into parts, every part is a session of its own over the same tables, the parts'
 // rounds run in step and a round's message is the sum of theirs.  Host-driven rounds: the reference's
 // GENERIC-ROUND-SUMS role (src/sumcheck.lisp:282-317), the way that always works, not the fast one.
-static bool fits_one_kernel(const Statement &st, int points) {
+static bool fits_one_kernel(const Statement &st, int points) {  // points < 0: planned for the honest claim
   Statement planned = st;
-  planned.plan(points);
+  if (points < 0)
+    planned.plan_claim();
+  else
+    planned.plan(points);
   StmtDesc d;
   return planned.T() <= MAXT && make_desc(planned, &d);
 }
 
-static int sumcheck_prove_wide(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables,
-                               const int *strides, const uint32_t *eq, const uint32_t *consts, const std::string &label,
-                               const uint32_t *bw, int K, int degree, int points, uint32_t *out_chal,
-                               uint32_t *out_finals, uint32_t *const *out_folded) {
-  const int D = tr.D;
+// the parts: as many of the expanded form's groups each as still fit one kernel
+static int deal_parts(const Statement &st, int points, std::vector<Statement> *parts) {
   if (st.T() > MAXT || points > 16) {
     set_error("invalid-parameter: statement beyond the kernels' limits");
     return E_PARAM;
   }
-  // the parts: as many of the expanded form's groups each as still fit
-  std::vector<Statement> parts;
   Statement part = st;
   part.factored_groups.clear(), part.factored_linear.clear(), part.expanded_groups.clear();
   auto with = [&](Statement base, const Group &g) {
@@ -83,7 +81,7 @@ static int sumcheck_prove_wide(Transcript &tr, int n, const Statement &st, const
       part = grown;
       continue;
     }
-    if (!part.expanded_groups.empty()) parts.push_back(part);
+    if (!part.expanded_groups.empty()) parts->push_back(part);
     part.expanded_groups.clear();
     part = with(part, g);
     if (!fits_one_kernel(part, points)) {
@@ -91,7 +89,36 @@ static int sumcheck_prove_wide(Transcript &tr, int n, const Statement &st, const
       return E_PARAM;
     }
   }
-  if (!part.expanded_groups.empty()) parts.push_back(part);
+  if (!part.expanded_groups.empty()) parts->push_back(part);
+  return OK;
+}
+
+// HYPERCUBE-SUM of a statement that one kernel does not hold: the sum of its parts' claims
+int hypercube_sum_wide(const Statement &st, int D, int n, const uint32_t *const *d_tables, const int *strides,
+                       const uint32_t *eq, const uint32_t *consts, uint32_t *out) {
+  std::vector<Statement> parts;
+  int status = deal_parts(st, -1, &parts);
+  if (status) return status;
+  std::vector<uint32_t> total((size_t)D, 0u);
+  for (Statement &p : parts) {
+    SumcheckSession s;
+    s.private_buffers = true;
+    if ((status = s.begin(p, D, n, d_tables, strides, eq, nullptr, 1, consts, -1, true))) return status;
+    uint32_t sums[16 * 8];
+    if ((status = s.round_sums(sums))) return status;
+    for (int k = 0; k < D; k++) total[(size_t)k] = fadd(total[(size_t)k], sums[k]);
+  }
+  memcpy(out, total.data(), 4 * (size_t)D);
+  return OK;
+}
+
+static int sumcheck_prove_wide(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables,
+                               const int *strides, const uint32_t *eq, const uint32_t *consts, const std::string &label,
+                               const uint32_t *bw, int K, int degree, int points, uint32_t *out_chal,
+                               uint32_t *out_finals, uint32_t *const *out_folded) {
+  const int D = tr.D;
+  std::vector<Statement> parts;
+  if (int dealt = deal_parts(st, points, &parts)) return dealt;
   std::vector<std::unique_ptr<SumcheckSession>> sessions;
   int status;
   for (Statement &p : parts) {
@@ -124,15 +151,28 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
   int D = tr.D;
   if (degree < 0) degree = st.degree;
   int points = degree > 1 ? degree : 1;
-  SumcheckSession s;
+  SumcheckSession first, second;
   const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS");
   // the device drives the rounds when it can: the session then sends all its constants in one copy
   const bool device_rounds = n > 0 && n <= MAXROUNDS && points <= MAXPTS && !(host_rounds && host_rounds[0] == '1');
-  int status = s.begin(st, D, n, d_tables, strides, eq, bw, K, consts, degree, false, device_rounds);
-  if (status == E_PARAM && s.beyond_limits)
-    return sumcheck_prove_wide(tr, n, st, d_tables, strides, eq, consts, label, bw, K, degree, points, out_chal,
-                               out_finals, out_folded);
+  int status = first.begin(st, D, n, d_tables, strides, eq, bw, K, consts, degree, false, device_rounds);
+  bool direct = false;
+  if (status == E_PARAM && first.beyond_limits) {
+    // Too wide for accumulators per table group.  The fast way: the statement in direct form, one session whose
+    // kernels evaluate the written form at every wire point (compiled at run time, once per form and degree);
+    // the way that always works: its monomials dealt into parts proved in step.
+    const char *no_direct = getenv("EXACTA_HIP_NO_DIRECT");
+    Statement direct_st;
+    if (!(no_direct && no_direct[0] == '1') && n > 0 && make_direct(st, points, &direct_st)) {
+      status = second.begin(direct_st, D, n, d_tables, strides, eq, bw, K, consts, degree, false, device_rounds);
+      direct = status == OK;
+    }
+    if (!direct)
+      return sumcheck_prove_wide(tr, n, st, d_tables, strides, eq, consts, label, bw, K, degree, points, out_chal,
+                                 out_finals, out_folded);
+  }
   if (status) return status;
+  SumcheckSession &s = direct ? second : first;
   absorb_header(tr, label, n, degree, bw ? K : 1);
   if (device_rounds && s.device_capable()) {
     // the rounds run back to back on the device, transcript included.  This transcript then takes the messages

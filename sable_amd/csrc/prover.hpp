@@ -11,6 +11,9 @@
 
 namespace exh {
 
+// HYPERCUBE-SUM (src/sumcheck.lisp:112-126) of a statement wider than one kernel holds: the sum of its parts' claims
+int hypercube_sum_wide(const Statement &st, int D, int n, const uint32_t *const *d_tables, const int *strides,
+                       const uint32_t *eq, const uint32_t *consts, uint32_t *out);
 // tables: device pointers, K * 2^n entries of stride 1 or D each, block-major.
 int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables, const int *strides,
                    const uint32_t *eq, const uint32_t *consts, const std::string &label, const uint32_t *bw, int K,

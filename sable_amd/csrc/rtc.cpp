@@ -46,6 +46,7 @@ struct Job {
   std::string key;
   int D = 4;
   StmtDesc desc;
+  std::string source;  // the text of struct RtStmt when it is not the plain descriptor's
   std::vector<Part> parts;
   std::vector<std::thread> threads;
   std::atomic<int> running{0};
@@ -70,7 +71,7 @@ void compile_part(Job *job, Part *part) {
   // the descriptor sits in an unnamed namespace, as in the sources generated at build time: with external linkage
   // its fields do not fold to constants before the loops over them are unrolled, and the compilation does not end
   std::string source = "#include \"sumcheck_kernels.hpp\"\nnamespace exh {\nnamespace {\n" +
-                       desc_source(job->desc, "RtStmt") + "}\n}\n";
+                       (job->source.empty() ? desc_source(job->desc, "RtStmt") : job->source) + "}\n}\n";
   const char *names[kNSources], *texts[kNSources];
   for (int i = 0; i < kNSources; i++) names[i] = kSources[i].name, texts[i] = kSources[i].text;
   hiprtcProgram prog = nullptr;
@@ -262,13 +263,13 @@ void prepare_compiler() {
 }
 }  // namespace
 
-void rtc_request(const std::string &key, const StmtDesc &desc, int D) {
+void rtc_request(const std::string &key, const StmtDesc &desc, int D, const std::string &source) {
   prepare_compiler();
   std::lock_guard<std::mutex> lock(g_mutex);
   auto at = std::make_pair(key, D);
   if (g_jobs.count(at)) return;
   auto job = std::make_unique<Job>();
-  job->key = key, job->D = D, job->desc = desc;
+  job->key = key, job->D = D, job->desc = desc, job->source = source;
   const std::string d = std::to_string(D), st = "exh::RtStmt";
   // one program with the set's kernels, compiled on one background thread
   job->parts.resize(1);
@@ -276,7 +277,8 @@ void rtc_request(const std::string &key, const StmtDesc &desc, int D) {
   for (const char *base : {"true", "false"})
     for (const char *fold : {"true", "false"})
       exprs.push_back("exh::round_kernel<" + d + ", " + base + ", " + fold + ", " + st + ">");
-  exprs.push_back("exh::round_kernel_fold2<" + d + ", " + st + ">");
+  // (the double fold follows the base-field sweep, which a statement in direct form does not take)
+  if (source.empty()) exprs.push_back("exh::round_kernel_fold2<" + d + ", " + st + ">");
   exprs.push_back("exh::tail_kernel<" + d + ", " + st + ">");
   int passes = node_slots(desc) <= MAXACC ? nodes_launches(desc, D) : 0;
   for (int p = 0; p < passes; p++)

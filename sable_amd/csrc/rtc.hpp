@@ -14,7 +14,8 @@ namespace exh {
 bool rtc_enabled();
 // Start compiling kernels for the planned statement (its key, descriptor and degree D) unless that was done or
 // asked before.  Returns at once.
-void rtc_request(const std::string &key, const StmtDesc &desc, int D);
+// `source` (optional): the text of `struct RtStmt` when it is more than the descriptor (a statement in direct form).
+void rtc_request(const std::string &key, const StmtDesc &desc, int D, const std::string &source = std::string());
 // Load the compilations that have finished into the registry.  Called by the thread that owns the device,
 // before it looks a statement up.  Returns E_DEVICE when a module does not load.
 int rtc_collect();

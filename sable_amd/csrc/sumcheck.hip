@@ -169,6 +169,23 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   (void)rtc_collect();
   kernels = find_kernels(st.key(), D);
   generated = kernels != nullptr;
+  if (st.direct) {
+    // a statement in direct form has no interpreter to fall back on: without its kernels the caller takes another
+    // way (beyond_limits: the statement in parts).  Like any unseen statement it is compiled in the background
+    // when the tables are large enough for the difference to matter, for the next proof; exh_stmt_generate asks
+    // for the kernels ahead of time and can wait for them.
+    if (claim_mode || st.nacc != points) {
+      set_error("invalid-parameter: a statement in direct form is proved at the wire points it was made for");
+      return E_PARAM;
+    }
+    if (!generated) {
+      static const int min_n = getenv("EXACTA_HIP_RTC_MIN_N") ? atoi(getenv("EXACTA_HIP_RTC_MIN_N")) : 20;
+      if (rtc_enabled() && n >= min_n) rtc_request(st.key(), desc, D, direct_source(st, desc, "RtStmt"));
+      set_error("invalid-parameter: the kernels of the statement in direct form are not compiled (yet)");
+      beyond_limits = true;
+      return E_PARAM;
+    }
+  }
   if (!generated && !claim_mode && rtc_enabled()) {
     // no kernel yet for this statement: the interpreter serves this proof; for tables large enough for the
     // difference to matter, kernels are compiled in the background for the next one
@@ -282,6 +299,8 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   if (any_base && !all_base)
     for (int t = 0; t < T; t++)
       if (strides[t] == 1) words += size * D;
+  const uint64_t direct_off = words;  // a direct statement's constant slots
+  if (st.direct) words += (uint64_t)std::max(st.direct_slots, 1) * D;
   if ((status = arena_misc().reserve(words * 4))) return status;
   uint32_t *base = (uint32_t *)arena_misc().ptr;
   d_weights = base;
@@ -293,6 +312,14 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   d_ctrl = reinterpret_cast<Ctrl *>(base + ctrl_off);
   d_mtilde = base + mt_off;
   d_c0 = base + c0_off;
+  d_direct = nullptr;
+  if (st.direct) {
+    d_direct = base + direct_off;
+    direct_host.assign((size_t)std::max(st.direct_slots, 1) * D, 0u);
+    if (st.direct_slots) direct_slot_values(st, D, consts, direct_host.data());
+    for (uint32_t &w : direct_host) w = to_mont(w);
+    EXH_HIP(hipMemcpyAsync(d_direct, direct_host.data(), direct_host.size() * 4, hipMemcpyHostToDevice, c.stream));
+  }
 
   cur.assign(T, nullptr);
   cur_base = all_base;
@@ -492,6 +519,7 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
   a.pstride = s.pstride;
   a.double_fold = double_fold ? 1 : 0;
   if (s.device_loop) a.ctrl = s.d_ctrl;
+  a.consts = s.d_direct;
   uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
   const bool own_epilogue = do_sums && s.device_loop && s.st.nacc > 0;
   if (own_epilogue) {
@@ -727,15 +755,16 @@ int SumcheckSession::round_sums(uint32_t *out) {
       for (int k = 0; k < points; k++) rows[k] = hf::add(rows[k], v);
       continue;
     }
-    uint32_t fix = fpow(R1, grp.tabs.size());  // the kernel's sums carry R^-degree
+    // the kernel's sums carry R^-degree (none for a statement in direct form)
+    uint32_t fix = st.direct ? 1u : fpow(R1, grp.tabs.size());
     std::vector<hf::E> vals;
     for (size_t k = 0; k < grp.evalx.size(); k++) {
       hf::E v(c.host_pinned + (size_t)(grp.acc_base + k) * D, c.host_pinned + (size_t)(grp.acc_base + k + 1) * D);
       vals.push_back(hf::scale(v, fix));
     }
-    bool direct = (int)grp.tabs.size() >= points;
+    bool at_wire = st.direct || (int)grp.tabs.size() >= points;  // evaluated at the wire points themselves
     for (int k = 0; k < points; k++) {
-      hf::E gv = direct ? vals[k] : hf::interpolate(grp.evalx, vals, hf::lift((uint32_t)wire[k], D));
+      hf::E gv = at_wire ? vals[k] : hf::interpolate(grp.evalx, vals, hf::lift((uint32_t)wire[k], D));
       rows[k] = hf::add(rows[k], hf::mul(coef, gv));
     }
   }
@@ -828,8 +857,9 @@ static uint64_t tail_pairs(int T, int D) {
 
 // the Lagrange basis of the group's node e over its nodes at wire point k (0, 2, 3, ...), times the power of R the
 // group's sums carry (R^-degree)
-static uint32_t map_scalar(const Group &grp, size_t e, int k, int points) {
-  const uint32_t fix = fpow(R1, grp.tabs.size());
+static uint32_t map_scalar(const Group &grp, size_t e, int k, int points, bool direct) {
+  // (a direct statement's accumulators hold w times the form's value in Montgomery form, reduced once: no power of R)
+  const uint32_t fix = direct ? 1u : fpow(R1, grp.tabs.size());
   if ((int)grp.tabs.size() >= points) return (int)e == k ? fix : 0u;  // evaluated at the wire points themselves
   const int wire = k == 0 ? 0 : k + 1;
   uint32_t num = 1, den = 1;
@@ -851,7 +881,7 @@ void SumcheckSession::message_map_scalars(std::vector<uint32_t> *lagfix, std::ve
     if (grp.tabs.empty()) continue;
     for (size_t e = 0; e < grp.evalx.size(); e++) {
       (*acc_group)[grp.acc_base + e] = (int)g;
-      for (int k = 0; k < points; k++) (*lagfix)[(size_t)k * nacc + grp.acc_base + e] = map_scalar(grp, e, k, points);
+      for (int k = 0; k < points; k++) (*lagfix)[(size_t)k * nacc + grp.acc_base + e] = map_scalar(grp, e, k, points, st.direct);
     }
   }
 }
@@ -899,7 +929,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     }
     for (size_t e = 0; e < grp.evalx.size(); e++) {
       for (int k = 0; k < points; k++) {
-        hf::E m = hf::scale(coef, map_scalar(grp, e, k, points));
+        hf::E m = hf::scale(coef, map_scalar(grp, e, k, points, st.direct));
         uint32_t *dst = mt + ((size_t)k * nacc + grp.acc_base + e) * D;
         for (int cc = 0; cc < D; cc++) dst[cc] = to_mont(m[cc]);
       }
@@ -1140,6 +1170,7 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
     a.groups = groups;
     a.spin_limit = 200000;
     a.host_log = host_log, a.host_flag_at = host_flag_at, a.host_seq = host_seq;
+    a.consts = d_direct;
     for (int jj = 0; jj < rounds; jj++) {
       a.low_off[jj] = low_off[j + jj];
       a.high_off[jj] = high_off[j + jj];

@@ -65,6 +65,9 @@ struct SumcheckSession {
   Ctrl *d_ctrl = nullptr;
   std::vector<uint32_t> final_cache;  // the tables as the device loop's tail left them, when read back with its logs
   uint32_t *d_mtilde = nullptr, *d_c0 = nullptr;
+  // a statement in direct form: its constant slots at this proof's constants (Montgomery form), host and device
+  uint32_t *d_direct = nullptr;
+  std::vector<uint32_t> direct_host;
   bool pending_fold = false;
   uint32_t pending_r[8];
   int generation = 0;

@@ -67,6 +67,7 @@ struct RoundArgs {
   uint32_t *arrivals;          // workgroups that have added their sums, zero before the launch
   uint32_t groups, points, spin_limit;
   const uint32_t *mtilde, *c0;  // the round's message map and constant terms
+  const uint32_t *consts;       // a statement in direct form: its constant slots (EXTs, Montgomery form)
 };
 
 // How the workgroups of a streaming launch finish a round without another launch.  Every workgroup adds its sums
@@ -117,6 +118,7 @@ struct TailArgs {
   // on the stream to read the logs (null: it does both)
   uint32_t *host_log;
   uint32_t host_flag_at, host_seq;
+  const uint32_t *consts;  // a statement in direct form: its constant slots (EXTs, Montgomery form)
 };
 
 template <int D>
@@ -204,6 +206,56 @@ __device__ __forceinline__ void v_mul_acc(Acc96 *acc, uint32_t a, uint32_t b) { 
 template <int D>
 __device__ __forceinline__ void v_mul_acc(Acc96 *acc, const Ext<D> &a, const Ext<D> &b) { ext_mul_acc<D>(acc, a, b); }
 
+// A statement too wide for accumulators per table group comes in direct form: its descriptor's type carries an
+// evaluator of the written form (generated code) and a flag, and the accumulators are the wire points.
+template <class T>
+struct is_direct {
+  template <class U>
+  static char test(decltype(U::direct) *);
+  template <class U>
+  static long test(...);
+  static constexpr bool value = sizeof(test<T>(nullptr)) == sizeof(char);
+};
+
+// The pair's contribution for a statement in direct form: the tables' lines in Montgomery form (so that sums and
+// products of any shape stay in one scale), the form evaluated at each wire point X = 0, 2, 3, ..., and w times
+// that value added to the point's accumulator.  The loop over the points is kept a loop: the evaluator is long,
+// and one copy of it per kernel keeps compile times and code size in hand; the accumulators stay in registers
+// because each is named by a constant inside the switch.
+template <int D, class V, class Desc, int PARTS, int PART>
+__device__ __forceinline__ void accumulate_direct(const Desc &d, const V *lo, const V *hi, const Ext<D> &w,
+                                                  Acc96 (*acc)[D], const uint32_t *kc) {
+  Ext<D> at0[MAXT], slope[MAXT];
+#pragma unroll
+  for (int t = 0; t < MAXT; t++)
+    if (t < d.T) {
+      if constexpr (std::is_same<V, uint32_t>::value) {
+        at0[t] = ext_lift<D>(mont_mul(lo[t], R2));
+        slope[t] = ext_lift<D>(mont_mul(fsub(hi[t], lo[t]), R2));
+      } else {
+        at0[t] = ext_scale_mont<D>(lo[t], R2);
+        slope[t] = ext_scale_mont<D>(ext_sub<D>(hi[t], lo[t]), R2);
+      }
+    }
+#pragma unroll 1
+  for (int k = PART; k < d.nacc; k += PARTS) {
+    const uint32_t x_mont = mont_mul(k == 0 ? 0u : (uint32_t)k + 1u, R2);
+    Ext<D> t[MAXT];
+#pragma unroll
+    for (int i = 0; i < MAXT; i++)
+      if (i < d.T) t[i] = ext_add<D>(at0[i], ext_scale_mont<D>(slope[i], x_mont));
+    const Ext<D> f = Desc::template eval<D>(t, kc);
+    switch (k) {
+      case 0: ext_mul_acc<D>(acc[0], f, w); break;
+      case 1: ext_mul_acc<D>(acc[1], f, w); break;
+      case 2: ext_mul_acc<D>(acc[2], f, w); break;
+      case 3: ext_mul_acc<D>(acc[3], f, w); break;
+      case 4: ext_mul_acc<D>(acc[4], f, w); break;
+      default: ext_mul_acc<D>(acc[5], f, w); break;
+    }
+  }
+}
+
 // With PARTS > 1 only the accumulators a with a % PARTS == PART are computed (a compile-time constant: with the
 // part as a run-time value, uniform as it is, the compiler folds the parts' branches into one path that indexes
 // the accumulators by it, and they move from registers to scratch memory): the last rounds, with a pair per lane
@@ -211,7 +263,11 @@ __device__ __forceinline__ void v_mul_acc(Acc96 *acc, const Ext<D> &a, const Ext
 // waits for a quarter of the products.
 template <int D, class V, class Desc, int PARTS = 1, int PART = 0>
 __device__ __forceinline__ void accumulate_pair(const Desc &d, const V *lo, const V *hi, const Ext<D> &w,
-                                                Acc96 (*acc)[D]) {
+                                                Acc96 (*acc)[D], const uint32_t *kc = nullptr) {
+  if constexpr (is_direct<Desc>::value) {
+    accumulate_direct<D, V, Desc, PARTS, PART>(d, lo, hi, w, acc, kc);
+    return;
+  }
   V cur[MAXT], slope[MAXT];
 #pragma unroll
   for (int t = 0; t < MAXT; t++)
@@ -730,6 +786,7 @@ struct RoundShape {
   uint32_t points;
   const uint32_t *mtilde, *c0;
   Ctrl *ctrl;
+  const uint32_t *consts;
 };
 
 template <int D, bool IN_BASE, bool FOLD, class Desc, bool FOLD2 = false, bool GENERATED = false>
@@ -752,7 +809,8 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
   // With a statement known at compile time and D = 4 the next pair's words are fetched before this pair's
   // arithmetic (two workgroups per compute unit leave the registers for it, and too few wavefronts to hide the
   // loads behind one another); the interpreter and D = 8 keep the plain order.
-  constexpr bool AHEAD = GENERATED && D == 4;
+  // (nor does a statement in direct form: it is wide, and its tables' words ahead would not fit the registers)
+  constexpr bool AHEAD = GENERATED && D == 4 && !is_direct<Desc>::value;
   if constexpr (AHEAD) {
     constexpr int Q = raw_quads<D, IN_BASE, FOLD, FOLD2>();
     uint4 raw[MAXT][Q], ahead[MAXT][Q];
@@ -768,7 +826,7 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
       pair_from_raw<D, IN_BASE, FOLD, V, FOLD2, Q>(d, raw, out, i, r, lo, hi, bw);
       if (sh.do_sums) {
         if (!sh.deferred) w = ext_mul_mont<D>(w, load_ext<D>(sh.high + (i >> sh.low_bits) * D));
-        accumulate_pair<D, V>(d, lo, hi, w, acc);
+        accumulate_pair<D, V>(d, lo, hi, w, acc, sh.consts);
       }
       if (more) {
 #pragma unroll
@@ -788,7 +846,7 @@ __device__ __forceinline__ void round_core(const Desc &d, const uint32_t *const 
       if (sh.do_sums) {
         Ext<D> w = load_ext<D>(sh.low + (i & low_mask) * D);
         if (!sh.deferred) w = ext_mul_mont<D>(w, load_ext<D>(sh.high + (i >> sh.low_bits) * D));
-        accumulate_pair<D, V>(d, lo, hi, w, acc);
+        accumulate_pair<D, V>(d, lo, hi, w, acc, sh.consts);
       }
     }
   }
@@ -860,7 +918,7 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
     BindWeights<D> bw = bind_weights<D>(r0, r1);
     RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
                      args.do_sums != 0, RoundTotals{args.totals, args.arrivals, args.groups, args.pstride, args.spin_limit},
-                     args.points, args.mtilde, args.c0, args.ctrl};
+                     args.points, args.mtilde, args.c0, args.ctrl, args.consts};
     round_core<D, true, true, Desc, true, GENERATED>(d, args.in, args.out, sh, r, blockIdx.x,
                                           args.partials + (uint64_t)blockIdx.x * args.pstride, &bw);
     return;
@@ -872,7 +930,7 @@ __device__ __forceinline__ void round_body(const Desc &d, const RoundArgs<D> &ar
   }
   RoundShape<D> sh{args.low, args.high, args.n_pairs, args.low_bits, args.pairs_per_thread, args.deferred != 0,
                    args.do_sums != 0, RoundTotals{args.totals, args.arrivals, args.groups, args.pstride, args.spin_limit},
-                   args.points, args.mtilde, args.c0, args.ctrl};
+                   args.points, args.mtilde, args.c0, args.ctrl, args.consts};
   round_core<D, IN_BASE, FOLD, Desc, false, GENERATED>(d, args.in, args.out, sh, r, blockIdx.x,
                                args.partials + (uint64_t)blockIdx.x * args.pstride);
 }
@@ -945,13 +1003,13 @@ __global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) 
 // wavefront into sums (LDS).  The accumulators are this function's own, so that they live in registers.
 template <int D, int PART, class Desc>
 __device__ __forceinline__ void small_round_sums(const Desc &d, const Ext<D> *lo, const Ext<D> *hi, const Ext<D> &w,
-                                                 uint32_t *sums) {
+                                                 uint32_t *sums, const uint32_t *kc) {
   Acc96 acc[MAXACC][D];
 #pragma unroll
   for (int a = 0; a < MAXACC; a++)
 #pragma unroll
     for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
-  accumulate_pair<D, Ext<D>, Desc, 4, PART>(d, lo, hi, w, acc);
+  accumulate_pair<D, Ext<D>, Desc, 4, PART>(d, lo, hi, w, acc, kc);
   part_wave_sums<D, PART, 4>(d, acc, sums);
 }
 
@@ -1053,13 +1111,13 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
         if (lane >= pairs) ww = ext_zero<D>();  // lanes without a pair add nothing
         if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
         if (wave == 0)
-          small_round_sums<D, 0>(d, lo, hi, ww, sums);
+          small_round_sums<D, 0>(d, lo, hi, ww, sums, args.consts);
         else if (wave == 1)
-          small_round_sums<D, 1>(d, lo, hi, ww, sums);
+          small_round_sums<D, 1>(d, lo, hi, ww, sums, args.consts);
         else if (wave == 2)
-          small_round_sums<D, 2>(d, lo, hi, ww, sums);
+          small_round_sums<D, 2>(d, lo, hi, ww, sums, args.consts);
         else
-          small_round_sums<D, 3>(d, lo, hi, ww, sums);
+          small_round_sums<D, 3>(d, lo, hi, ww, sums, args.consts);
         lds_barrier();
       } else {
         Acc96 acc[MAXACC][D];
@@ -1081,7 +1139,7 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
             wl = load_ext<D>(args.weights + (args.low_off[jj] + (gi & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
             wh = load_ext<D>(args.weights + (args.high_off[jj] + (gi >> args.low_bits[jj])) * D);
           }
-          accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc);
+          accumulate_pair<D, Ext<D>>(d, lo, hi, ext_mul_mont<D>(wl, wh), acc, args.consts);
         }
         if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
         block_sums<D, true>(d, acc, lds, sums);

@@ -16,6 +16,23 @@ SUMCHECK = {
                     seed=2),
     "config3": dict(form="(* (+ c0 3) (- c1 c0) c2 c3)", tables=["c0", "c1", "c2", "c3"], constants=[], n=26, d=8,
                     seed=3),
+    # A statement wider than the table groups' kernels hold: the leaf-layer and zerocheck statement of the
+    # reference's toy domain (tests/tests.lisp:487-512 through src/domain.lisp:95-114: three lookups, three
+    # constraints, every kind of column; 41 table monomials), over seeded tables instead of a witness -- the
+    # prover's work does not depend on the constraints holding.
+    "domain": dict(
+        form="(+ (* %A0 (+ (- %Z 5 (* %BETA0 A@0) (* %BETA1 B@0)) (- %Z 5 (* %BETA0 A@1) (* %BETA1 B@1))))"
+             " (* %AL0 (- %Z 5 (* %BETA0 A@0) (* %BETA1 B@0)) (- %Z 5 (* %BETA0 A@1) (* %BETA1 B@1)))"
+             " (* %A1 (+ (* (+ S@0 2) (- %Z 7 (* %BETA0 C@1) (* %BETA1 M@1) (* %BETA2 W)))"
+             " (* (+ S@1 2) (- %Z 7 (* %BETA0 C@0) (* %BETA1 M@0) (* %BETA2 W)))))"
+             " (* %AL1 (- %Z 7 (* %BETA0 C@0) (* %BETA1 M@0) (* %BETA2 W)) (- %Z 7 (* %BETA0 C@1) (* %BETA1 M@1) (* %BETA2 W)))"
+             " (* %A2 (+ (- %Z 9 (* %BETA0 KB)) (- %Z 9 (* %BETA0 KB)))) (* %AL2 (- %Z 9 (* %BETA0 KB)) (- %Z 9 (* %BETA0 KB)))"
+             " (* %GAM0 (* A@0 (- A@0 1))) (* %GETA0 (* A@1 (- A@1 1))) (* %GAM1 (- C@0 (* A@0 B@0)))"
+             " (* %GETA1 (- C@1 (* A@1 B@1))) (* %GAM2 (* S@0 (- S@0 1) M@0)) (* %GETA2 (* S@1 (- S@1 1) M@1)))",
+        tables=["A@0", "A@1", "B@0", "B@1", "C@0", "C@1", "M@0", "M@1", "S@0", "S@1", "W", "KB"],
+        constants=["%Z", "%BETA0", "%BETA1", "%BETA2", "%A0", "%AL0", "%A1", "%AL1", "%A2", "%AL2", "%GAM0", "%GETA0",
+                   "%GAM1", "%GETA1", "%GAM2", "%GETA2"],
+        n=20, d=4, seed=7),
 }
 
 

@@ -33,3 +33,23 @@ def vectors():
         return out
 
     return of
+
+
+def launch_names(step):
+    """The names of the launches `step` makes, from the library's own launch timing (GPU tests)."""
+    import ctypes as C
+
+    import sable_amd as sa
+    lib = sa.load()
+    sa.check(lib.exh_profile_enable(1))
+    try:
+        step()
+        names = []
+        for i in range(lib.exh_profile_count()):
+            name = C.create_string_buffer(64)
+            rnd, ms, nbytes = C.c_int(), C.c_float(), C.c_uint64()
+            sa.check(lib.exh_profile_entry(i, name, 64, C.byref(rnd), C.byref(ms), C.byref(nbytes)))
+            names.append(name.value.decode())
+    finally:
+        sa.check(lib.exh_profile_enable(0))
+    return names

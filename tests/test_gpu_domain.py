@@ -9,6 +9,7 @@ import sable_amd as sa
 from oracle import binding as orc
 from oracle import domain as od
 from sable_amd import domain as sd
+from conftest import launch_names
 from test_oracle_domain import CASES as ORACLE_CASES, lookup_challenges, toy_domain
 
 pytestmark = pytest.mark.gpu
@@ -181,3 +182,30 @@ def test_a_wide_statement_at_size():
     tr = sa.Transcript("dom-test", d)
     sd.prove_domain(tr, mine, z, betas)
     assert tr.proof() == otr.proof()
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("d,n,k", [(4, 7, 2), (4, 13, 1), (8, 5, 3)])
+def test_the_toy_domain_in_direct_form(d, n, k):
+    """The same wide statement once its direct-form kernels are there (exh_stmt_generate compiles them: the
+    written form evaluated per pair at every wire point, one accumulator per point): one device-driven session
+    instead of parts proved in step, and the same bytes as the oracle's."""
+    theirs = toy_domain(n=n, k=k, seed=300 + d + n)
+    mine = device_toy(theirs)
+    z, betas = lookup_challenges(d, n)
+    otr = orc.Transcript("dom-test", d)
+    want_claims = od.prove_domain(otr, theirs, z, betas)
+    st = sd._compiled(mine)
+    assert st.generate(d, degree=sd.domain_degree(mine), wait=True)
+    tr = sa.Transcript("dom-test", d)
+    out = {}
+    names = launch_names(lambda: out.setdefault("claims", sd.prove_domain(tr, mine, z, betas)))
+    assert tr.proof() == otr.proof() and same_claims(out["claims"], want_claims)
+    # with one block everything around the zerocheck is chained on the device, so the streaming round launches
+    # (named round_...) are the zerocheck's: in parts there is one per part and round, in one device-driven loop
+    # only the first few rounds stream before the tables fit the workgroups' LDS
+    if k == 1:
+        assert len([name for name in names if name.startswith("round_")]) < n, names
+    vtr = sa.Transcript("dom-test", d, proof=tr.proof())
+    got, _ = sd.verify_domain(vtr, mine, z, betas)
+    assert vtr.finished() and same_claims(got, out["claims"])

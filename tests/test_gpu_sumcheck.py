@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 
 import sable_amd as sa
+from conftest import launch_names
 from oracle import binding as orc
 
 pytestmark = pytest.mark.gpu
@@ -343,5 +344,62 @@ def test_host_replay_of_the_device_transcript(n, monkeypatch):
     otr = orc.Transcript("replay", 4)
     orc.prove(otr, n, orc.Statement(CONFIG2, ["t0", "t1", "t2"], ["alpha"]), tables, eq=eq, constants=alpha)
     assert same(otr.challenge(), outs[0][3])
+    for t in dev:
+        t.free()
+
+
+def _wide():
+    from sable_amd import workloads as wl
+    cfg = wl.SUMCHECK["domain"]
+    return cfg["form"], cfg["tables"], cfg["constants"]
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("d,n,base,with_eq,K", [(4, 6, True, True, 1), (4, 12, False, True, 1), (4, 9, True, False, 1),
+                                                (4, 5, True, True, 3), (8, 7, True, True, 1), (4, 18, True, True, 1)])
+def test_a_wide_statement_in_direct_form(d, n, base, with_eq, K):
+    """A statement of 41 table monomials over 12 tables (the toy domain's, over seeded tables): too wide for
+    accumulators per table group, so its kernels evaluate the written form itself at every wire point.  The honest
+    claim (summed over the statement's parts) and the proof are the oracle's, on base and extension tables, with
+    and without an eq point, with block weights, and at a size whose first rounds stream from memory; the same
+    proof comes out when the statement is dealt into parts instead."""
+    form, names, cnames = _wide()
+    st, ost = both(form, names, cnames)
+    rng = np.random.default_rng(4100 + d + n)
+    size = K << n
+    tables = [rng.integers(0, P, size, dtype=np.uint32) if base else rand_ext(rng, (size,), d) for _ in names]
+    eq = rand_ext(rng, (n,), d) if with_eq else None
+    cv = rand_ext(rng, (len(cnames),), d)
+    bw = rand_ext(rng, (K,), d) if K > 1 else None
+    dev = [sa.Table.upload(t) for t in tables]
+    assert st.generate(d, wait=True)
+    if K == 1:
+        assert same(sa.hypercube_sum(st, n, dev, d, eq=eq, constants=cv), orc.hypercube_sum(ost, n, tables, d, eq=eq, constants=cv))
+    tr, otr = sa.Transcript("wide", d), orc.Transcript("wide", d)
+    out = {}
+    names = launch_names(lambda: out.setdefault("got", sa.prove(tr, n, st, dev, eq=eq, constants=cv, block_weights=bw)))
+    got = out["got"]
+    want = orc.prove(otr, n, ost, tables, eq=eq, constants=cv, block_weights=bw)
+    assert tr.proof() == otr.proof()
+    assert same(got[0], want[0]) and same(got[1], want[1])
+    # one session: the few rounds that stream, then the tables in LDS (in parts: a launch per part and round)
+    assert len([name for name in names if name.startswith("round_")]) < n, names
+    for t in dev:
+        t.free()
+
+
+def test_a_wide_statement_in_parts_when_the_direct_form_is_switched_off(monkeypatch):
+    form, names, cnames = _wide()
+    st, ost = both(form, names, cnames)
+    rng = np.random.default_rng(4200)
+    d, n = 4, 8
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) for _ in names]
+    eq, cv = rand_ext(rng, (n,), d), rand_ext(rng, (len(cnames),), d)
+    dev = [sa.Table.upload(t) for t in tables]
+    monkeypatch.setenv("EXACTA_HIP_NO_DIRECT", "1")
+    tr, otr = sa.Transcript("wide", d), orc.Transcript("wide", d)
+    sa.prove(tr, n, st, dev, eq=eq, constants=cv)
+    orc.prove(otr, n, ost, tables, eq=eq, constants=cv)
+    assert tr.proof() == otr.proof()
     for t in dev:
         t.free()
