@@ -555,6 +555,7 @@ def main():
     ap.add_argument("--cpu-n", type=int, default=20, help="variables of the one-thread CPU baseline's sample (0: skip)")
     ap.add_argument("--others", type=int, default=1, help="0: leave the other configured workloads out of the headline's line")
     args = ap.parse_args()
+    sys.stdout.reconfigure(line_buffering=True)  # the line is out before the process ends, whatever ends it
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus above 1 is not supported (nothing here uses a "
                  "second device)")
@@ -642,8 +643,12 @@ def main():
         others["config5"]["basefold"] = {key: r[key] for key in ("workload", "ms_per_step", "proof_sha256",
                                                                  "proof_is_the_cpu_oracles", "kernel_ms_per_step",
                                                                  "timed_launches_per_step", "roofline")}
+        r = run_domain(sa, k, 2)
+        others["wide_statement"] = {key: r[key] for key in ("workload", "ms_per_step", "ms_per_step_in_parts",
+                                                            "entries_per_s", "proof_sha256", "proof_is_the_parts_paths",
+                                                            "timed_launches_per_step", "loop_hbm_fraction", "roofline")}
         out["other_configs"] = others
-    print(json.dumps(out))
+    print(json.dumps(out), flush=True)
 
 
 if __name__ == "__main__":
