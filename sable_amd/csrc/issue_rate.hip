@@ -30,14 +30,20 @@ enum IssueOp : int {
   OP_CVT_F64_U32,
   OP_MIN_U32,
   OP_CNDMASK_B32,
+  OP_PERM_B32,       // a rotation by whole bytes as a byte permutation
+  OP_ALIGNBYTE_B32,  // the same as a byte alignment of the word with itself
+  OP_LSHLREV_B32,
+  OP_LSHL_OR_B32,
+  OP_XAD_U32,
   OP_COUNT
 };
 
 static const char *const kOpNames[OP_COUNT] = {
     "v_fma_f64",     "v_add_f64",      "v_mul_f64",   "v_mul_lo_u32", "v_mul_hi_u32", "v_mad_u64_u32",
     "v_add_u32",     "v_sub_u32+v_min_u32", "v_xor_b32", "v_alignbit_b32", "v_add3_u32", "v_fma_f32",
-    "v_add_co_u32+v_addc_co_u32", "v_cvt_f64_u32", "v_min_u32", "v_cndmask_b32"};
-static const int kOpInstructions[OP_COUNT] = {1, 1, 1, 1, 1, 1, 1, 2, 1, 1, 1, 1, 2, 1, 1, 1};
+    "v_add_co_u32+v_addc_co_u32", "v_cvt_f64_u32", "v_min_u32", "v_cndmask_b32", "v_perm_b32", "v_alignbyte_b32",
+    "v_lshlrev_b32", "v_lshl_or_b32", "v_xad_u32"};
+static const int kOpInstructions[OP_COUNT] = {1, 1, 1, 1, 1, 1, 1, 2, 1, 1, 1, 1, 2, 1, 1, 1, 1, 1, 1, 1, 1};
 
 constexpr int ISSUE_BLOCK = 256;
 
@@ -88,6 +94,11 @@ __global__ __launch_bounds__(ISSUE_BLOCK) void issue_rate_kernel(uint32_t *out, 
         if constexpr (OP == OP_CVT_F64_U32) asm volatile("v_cvt_f64_u32 %0, %1" : "=v"(x[i]) : "v"(u[i]));
         if constexpr (OP == OP_MIN_U32) asm volatile("v_min_u32 %0, %0, %1" : "+v"(u[i]) : "v"(ia));
         if constexpr (OP == OP_CNDMASK_B32) asm volatile("v_cndmask_b32 %0, %0, %1, vcc" : "+v"(u[i]) : "v"(ia) : );
+        if constexpr (OP == OP_PERM_B32) asm volatile("v_perm_b32 %0, %0, %0, %1" : "+v"(u[i]) : "v"(ib));
+        if constexpr (OP == OP_ALIGNBYTE_B32) asm volatile("v_alignbyte_b32 %0, %0, %0, 1" : "+v"(u[i]));
+        if constexpr (OP == OP_LSHLREV_B32) asm volatile("v_lshlrev_b32 %0, 7, %0" : "+v"(u[i]));
+        if constexpr (OP == OP_LSHL_OR_B32) asm volatile("v_lshl_or_b32 %0, %0, 7, %1" : "+v"(u[i]) : "v"(ia));
+        if constexpr (OP == OP_XAD_U32) asm volatile("v_xad_u32 %0, %0, %1, %2" : "+v"(u[i]) : "v"(ia), "v"(ib));
       }
     }
   }
