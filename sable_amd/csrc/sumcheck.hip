@@ -1180,6 +1180,23 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
   if (grid > 1 && !slice_totals_clear)  // the rounds' totals start at zero (64-bit words)
     EXH_HIP(hipMemsetAsync(d_slice_totals, 0, (size_t)rounds * groups * pstride * 8, c.stream));
   if (grid > 1) slice_totals_clear = false;
+  const bool hold = held_tail && grid == 1 && generated && kernels->launch_tail_glue && j + rounds == n;
+  if (hold) {  // the caller launches it, with its own next step behind the rounds
+    if (D == 4) {
+      TailArgs<4> a;
+      fill(a);
+      held_tail->assign(reinterpret_cast<uint8_t *>(&a), reinterpret_cast<uint8_t *>(&a) + sizeof(a));
+    } else {
+      TailArgs<8> a;
+      fill(a);
+      held_tail->assign(reinterpret_cast<uint8_t *>(&a), reinterpret_cast<uint8_t *>(&a) + sizeof(a));
+    }
+    cur_base = false;
+    for (int t = 0; t < T; t++) cur[t] = (uint32_t *)dst.ptr + (uint64_t)t * final_size * D;
+    size = final_size;
+    generation += folds;
+    return OK;
+  }
   c.prof_begin(grid > 1 ? "slices" : "tail", j,
                (uint64_t)T * size * (cur_base ? 1 : D) * 4 + (uint64_t)T * final_size * D * 4);
   if (D == 4) {

@@ -23,6 +23,9 @@ struct KernelSet {  // the launchers generated for one statement and one degree 
   int nodes_passes = 0;  // launches of launch_nodes per round (0: not available)
   // workgroups of the tail kernel a compute unit holds at once with that much dynamic LDS (-1: unknown)
   std::function<int(uint32_t lds_bytes)> tail_blocks_per_cu;
+  // LogUp-GKR's layer statement only: the one-workgroup launch of the last rounds followed, in the same launch, by
+  // the step between two layers (TailArgs<D>, GlueArgs<D>)
+  std::function<void(const void *tail_args, const void *step_args, hipStream_t stream)> launch_tail_glue;
 };
 // EQ-TABLE of k coordinates (canonical, host) into 2^k elements of device memory
 int eq_table_device(int D, int k, const uint32_t *r, uint32_t *d_out);
@@ -90,6 +93,10 @@ struct SumcheckSession {
   // from the host; run_device enqueues its launches and returns without waiting or reading anything back, and the
   // control block (logs, finals) stays in device memory for the chain's next launch.
   std::function<int()> chain_hook;
+  // Set with chain_hook by a caller whose next step can ride on this session's last launch: that launch (one
+  // workgroup, the last rounds) is then not enqueued; its arguments are left here (a TailArgs<D>) for the caller to
+  // launch, after this session has returned and even after the next one has begun (they are plain addresses).
+  std::vector<uint8_t> *held_tail = nullptr;
   // the scalar (Lagrange basis times the power of R the sums carry) that maps accumulator `acc` to wire point k in
   // the message map: lagfix[k * nacc + acc], and the group each accumulator belongs to
   void message_map_scalars(std::vector<uint32_t> *lagfix, std::vector<int> *acc_group) const;
