@@ -29,21 +29,29 @@ enum IssueOp : int {
   OP_ADDC_PAIR,  // a 64-bit add: add with carry-out, add with carry-in (two instructions)
   OP_CVT_F64_U32,
   OP_MIN_U32,
-  OP_CNDMASK_B32,
+  OP_CNDMASK_B32,    // a select reading a vcc that no instruction near it wrote: 23 cycles each, unlike every real use below
   OP_PERM_B32,       // a rotation by whole bytes as a byte permutation
   OP_ALIGNBYTE_B32,  // the same as a byte alignment of the word with itself
   OP_LSHLREV_B32,
   OP_LSHL_OR_B32,
   OP_XAD_U32,
+  OP_CMP_CNDMASK,   // a comparison into vcc and the select that reads it (two instructions)
+  OP_CMP_U32,       // the comparison alone
+  OP_CNDMASK_SGPR,  // the select reading its mask from a scalar register pair
+  OP_CMP_2CNDMASK,  // one comparison, two selects that read it (three instructions)
+  OP_CMP_GAP_CNDMASK,  // a comparison, four other instructions, then the select (six instructions)
+  OP_CMP_SGPR_CNDMASK,  // the comparison into a scalar register pair and the select reading that (two instructions)
   OP_COUNT
 };
 
 static const char *const kOpNames[OP_COUNT] = {
     "v_fma_f64",     "v_add_f64",      "v_mul_f64",   "v_mul_lo_u32", "v_mul_hi_u32", "v_mad_u64_u32",
     "v_add_u32",     "v_sub_u32+v_min_u32", "v_xor_b32", "v_alignbit_b32", "v_add3_u32", "v_fma_f32",
-    "v_add_co_u32+v_addc_co_u32", "v_cvt_f64_u32", "v_min_u32", "v_cndmask_b32", "v_perm_b32", "v_alignbyte_b32",
-    "v_lshlrev_b32", "v_lshl_or_b32", "v_xad_u32"};
-static const int kOpInstructions[OP_COUNT] = {1, 1, 1, 1, 1, 1, 1, 2, 1, 1, 1, 1, 2, 1, 1, 1, 1, 1, 1, 1, 1};
+    "v_add_co_u32+v_addc_co_u32", "v_cvt_f64_u32", "v_min_u32", "v_cndmask_b32(vcc written once, long before)", "v_perm_b32", "v_alignbyte_b32",
+    "v_lshlrev_b32", "v_lshl_or_b32", "v_xad_u32", "v_cmp_lt_u32+v_cndmask_b32", "v_cmp_lt_u32", "v_cndmask_b32(sgpr mask)",
+    "v_cmp_lt_u32+2 v_cndmask_b32", "v_cmp_lt_u32+4 v_xor_b32+v_cndmask_b32", "v_cmp_lt_u32(sgpr)+v_cndmask_b32(sgpr)"};
+static const int kOpInstructions[OP_COUNT] = {1, 1, 1, 1, 1, 1, 1, 2, 1, 1, 1, 1, 2, 1, 1, 1,
+                                              1, 1, 1, 1, 1, 2, 1, 1, 3, 6, 2};
 
 constexpr int ISSUE_BLOCK = 256;
 
@@ -60,6 +68,8 @@ __global__ __launch_bounds__(ISSUE_BLOCK) void issue_rate_kernel(uint32_t *out, 
     f[i] = (float)(threadIdx.x + i);
   }
   const float ffa = (float)fa, ffb = (float)fb;
+  // (the selects below read vcc: written once here, by a vector comparison, as in real code)
+  if constexpr (OP == OP_CNDMASK_B32) asm volatile("v_cmp_lt_u32 vcc, %0, %1" : : "v"(u[0]), "v"(ia) : "vcc");
   for (uint32_t it = 0; it < iterations; it++) {
 #pragma unroll
     for (int rep = 0; rep < 8; rep++) {
@@ -99,6 +109,29 @@ __global__ __launch_bounds__(ISSUE_BLOCK) void issue_rate_kernel(uint32_t *out, 
         if constexpr (OP == OP_LSHLREV_B32) asm volatile("v_lshlrev_b32 %0, 7, %0" : "+v"(u[i]));
         if constexpr (OP == OP_LSHL_OR_B32) asm volatile("v_lshl_or_b32 %0, %0, 7, %1" : "+v"(u[i]) : "v"(ia));
         if constexpr (OP == OP_XAD_U32) asm volatile("v_xad_u32 %0, %0, %1, %2" : "+v"(u[i]) : "v"(ia), "v"(ib));
+        if constexpr (OP == OP_CMP_CNDMASK)
+          asm volatile("v_cmp_lt_u32 vcc, %0, %1\n\tv_cndmask_b32 %0, %0, %2, vcc" : "+v"(u[i]) : "v"(ia), "v"(ib) : "vcc");
+        if constexpr (OP == OP_CMP_U32) asm volatile("v_cmp_lt_u32 vcc, %0, %1" : : "v"(u[i]), "v"(ia) : "vcc");
+        if constexpr (OP == OP_CMP_2CNDMASK) {
+          uint32_t t = u[i];
+          asm volatile("v_cmp_lt_u32 vcc, %0, %2\n\tv_cndmask_b32 %0, %0, %3, vcc\n\tv_cndmask_b32 %1, %1, %2, vcc"
+                       : "+v"(u[i]), "+v"(t) : "v"(ia), "v"(ib) : "vcc");
+          u[i] ^= t;
+        }
+        if constexpr (OP == OP_CMP_GAP_CNDMASK) {
+          uint32_t t = u[i];
+          asm volatile("v_cmp_lt_u32 vcc, %0, %2\n\tv_xor_b32 %1, %1, %2\n\tv_xor_b32 %1, %1, %3\n\tv_xor_b32 %1, %1, %2\n\t"
+                       "v_xor_b32 %1, %1, %3\n\tv_cndmask_b32 %0, %0, %1, vcc"
+                       : "+v"(u[i]), "+v"(t) : "v"(ia), "v"(ib) : "vcc");
+        }
+        if constexpr (OP == OP_CMP_SGPR_CNDMASK) {
+          uint64_t mask;
+          asm volatile("v_cmp_lt_u32 %1, %0, %2\n\tv_cndmask_b32 %0, %0, %3, %1" : "+v"(u[i]), "=&s"(mask) : "v"(ia), "v"(ib));
+        }
+        if constexpr (OP == OP_CNDMASK_SGPR) {
+          uint64_t mask = 0x5555555555555555ull;
+          asm volatile("v_cndmask_b32 %0, %0, %1, %2" : "+v"(u[i]) : "v"(ia), "s"(mask));
+        }
       }
     }
   }
