@@ -71,11 +71,11 @@ EXH_HD uint32_t mont_reduce(uint64_t t) {
 // t / R mod p for any t < 4 p^2 < 2^64 (a sum of four products): result in [0, p)
 EXH_HD uint32_t mont_reduce4(uint64_t t) {
   uint32_t m = (uint32_t)t * PINV;
-  uint32_t u = (uint32_t)(((uint64_t)m * P) >> 32);
-  uint32_t hi = (uint32_t)(t >> 32);  // < 1.99 p
-  uint32_t r = hi - u;                // in (-p, 1.99 p)
-  r = hi < u ? r + P : r;
-  return umin32(r, r - P);
+  uint32_t u = (uint32_t)(((uint64_t)m * P) >> 32);  // < p
+  uint32_t hi = (uint32_t)(t >> 32);                 // < 1.99 p
+  hi = umin32(hi, hi - P);                           // < p (the wrapped alternative is the larger unsigned value)
+  uint32_t r = hi - u;                               // in (-p, p): no comparison, no select
+  return umin32(r, r + P);
 }
 EXH_HD uint32_t mont_mul(uint32_t a, uint32_t b) { return mont_reduce((uint64_t)a * b); }
 // exact a b mod p (two reductions; host-side helpers and rare device paths)
@@ -101,9 +101,12 @@ EXH_HD void acc_zero(Acc96 &a) {
   a.lo = 0;
   a.hi = 0;
 }
+// (the carry of the 64-bit addition taken from the addition itself: three additions chained by the carry; written
+// as a comparison of the sum with a term it costs a 64-bit comparison and a select on top)
 EXH_HD void acc_add(Acc96 &a, uint64_t t) {
-  uint64_t s = a.lo + t;
-  a.hi += s < t;
+  unsigned long long s;
+  const bool carry = __builtin_uaddll_overflow(a.lo, t, &s);
+  a.hi += carry ? 1u : 0u;
   a.lo = s;
 }
 EXH_HD void acc_mad(Acc96 &a, uint32_t x, uint32_t y) { acc_add(a, (uint64_t)x * y); }

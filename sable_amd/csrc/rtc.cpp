@@ -117,6 +117,12 @@ void compile_part(Job *job, Part *part) {
   job->running--;
 }
 
+// the one-workgroup kernel of a statement: with half the registers for a statement in direct form at F_p^8 (see
+// tail_kernel_narrow)
+std::string tail_expression(int D, bool direct) {
+  return std::string(direct && D == 8 ? "exh::tail_kernel_narrow<" : "exh::tail_kernel<") + std::to_string(D) + ", exh::RtStmt>";
+}
+
 // the kernel behind launcher arguments passed by value as one struct
 void launch_module(hipFunction_t f, const void *args, uint32_t grid, uint32_t lds_bytes, hipStream_t s) {
   void *params[] = {const_cast<void *>(args)};
@@ -170,7 +176,7 @@ int load_job(Job *job) {
       round[base][fold] = fn["exh::round_kernel<" + d + ", " + (base ? "true" : "false") + ", " + (fold ? "true" : "false") +
                              ", " + st + ">"];
   hipFunction_t fold2 = fn["exh::round_kernel_fold2<" + d + ", " + st + ">"];
-  hipFunction_t tail = fn["exh::tail_kernel<" + d + ", " + st + ">"];
+  hipFunction_t tail = fn[tail_expression(job->D, !job->source.empty())];
   int passes = node_slots(job->desc) <= MAXACC ? nodes_launches(job->desc, job->D) : 0;
   std::vector<hipFunction_t> nodes;
   for (int p = 0; p < passes; p++)
@@ -279,7 +285,7 @@ void rtc_request(const std::string &key, const StmtDesc &desc, int D, const std:
       exprs.push_back("exh::round_kernel<" + d + ", " + base + ", " + fold + ", " + st + ">");
   // (the double fold follows the base-field sweep, which a statement in direct form does not take)
   if (source.empty()) exprs.push_back("exh::round_kernel_fold2<" + d + ", " + st + ">");
-  exprs.push_back("exh::tail_kernel<" + d + ", " + st + ">");
+  exprs.push_back(tail_expression(D, !source.empty()));
   int passes = node_slots(desc) <= MAXACC ? nodes_launches(desc, D) : 0;
   for (int p = 0; p < passes; p++)
     exprs.push_back("exh::nodes_kernel<" + d + ", " + st + ", " + std::to_string(p) + ", " +

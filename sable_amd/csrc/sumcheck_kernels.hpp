@@ -1629,6 +1629,13 @@ template <int D, class S>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(1, 1))) void tail_kernel(TailArgs<D> args) {
   tail_body<D>(S::d, args);
 }
+// (the same with half the registers: a statement in direct form at F_p^8 needs more than the 512 either way, and the
+// compiler's use of the upper half of the register file for 64-bit values that it also spills has been seen to end
+// in registers it then rejects)
+template <int D, class S>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(2, 2))) void tail_kernel_narrow(TailArgs<D> args) {
+  tail_body<D>(S::d, args);
+}
 template <int D, class S>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(2, 2))) void round_kernel_fold2(RoundArgs<D> args) {
   round_body<D, true, true, decltype(S::d), true, true>(S::d, args);
