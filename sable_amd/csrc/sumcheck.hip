@@ -138,6 +138,8 @@ static inline uint32_t next_pow2(uint64_t v) {
   return p;
 }
 
+static uint32_t tile_pairs_per_thread(uint64_t n_pairs, uint64_t max_grid, uint64_t low_span);
+
 int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uint32_t *const *tables,
                            const int *strides, const uint32_t *eq, const uint32_t *bw, int K_, const uint32_t *consts,
                            int degree, bool claim_mode_, bool defer_setup) {
@@ -269,7 +271,13 @@ int SumcheckSession::begin(const Statement &statement, int D_, int n_, const uin
   node_slots_n = node_slots(desc);  // grid sums of the sweep that serves rounds 0 and 1 from the base tables
   pstride = next_pow2((uint64_t)std::max(std::max(st.nacc, 1), node_slots_n <= MAXACC ? node_slots_n : 0) * D);
   uint64_t partial_off = pos * D;  // from here in words
-  const uint64_t partial_rows = max_grid;
+  // (a workgroup's partial row per workgroup of the largest grid a round can take: tiles stop growing at the span
+  // of a HIGH weight, see tile_pairs_per_thread)
+  uint64_t partial_rows = max_grid;
+  for (int j = 0; j < n; j++) {
+    const uint64_t pairs = (size >> j) / 2, tile = (uint64_t)BLOCK * tile_pairs_per_thread(pairs, max_grid, (uint64_t)1 << low_bits[j]);
+    partial_rows = std::max(partial_rows, (pairs + tile - 1) / tile);
+  }
   uint64_t words = partial_off + (partial_rows + 1) * (uint64_t)pstride + 64;
   words += 64;
   words += words & 1;  // the 64-bit totals of the grid launch of slices: [MAXTAIL][SLICE_GROUPS][pstride]
@@ -493,6 +501,18 @@ int SumcheckSession::launch_setup() {
   return OK;
 }
 
+// Pairs per thread of a streaming launch over n_pairs pairs: a tile (BLOCK * pairs per thread) grows to fit the
+// grid's cap, but not beyond the span of one HIGH weight when it can stay within it -- the weight is then applied
+// once per workgroup, where a larger tile would pay an extension product per pair; the grid is larger instead, and
+// its workgroups follow one another.  low_span: 2^low_bits of the round, 0 when the launch does not sum.
+static uint32_t tile_pairs_per_thread(uint64_t n_pairs, uint64_t max_grid, uint64_t low_span) {
+  uint32_t ppt = 1;
+  while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > max_grid &&
+         !(low_span >= BLOCK && (uint64_t)BLOCK * ppt * 2 > low_span && (uint64_t)BLOCK * ppt <= low_span))
+    ppt *= 2;
+  return ppt;
+}
+
 template <int D>
 static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::vector<uint32_t *> &outs,
                         uint64_t n_pairs, int j, bool double_fold = false) {
@@ -512,7 +532,7 @@ static int launch_round(SumcheckSession &s, bool fold, bool do_sums, const std::
     a.high = s.d_weights + s.high_off[j] * D;
     a.low_bits = (uint32_t)s.low_bits[j];
   }
-  while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > s.max_grid) ppt *= 2;
+  ppt = tile_pairs_per_thread(n_pairs, s.max_grid, do_sums ? (uint64_t)1 << a.low_bits : 0);
   a.pairs_per_thread = ppt;
   a.deferred = do_sums && ((uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits)) ? 1 : 0;
   a.partials = s.d_partials;
@@ -610,7 +630,7 @@ static int launch_nodes_round(SumcheckSession &s, uint64_t n_pairs) {
   // (two workgroups fit a compute unit beside the accumulators: the session's grid cap has them all resident
   // at once, which spreads each workgroup's fixed work -- first loads, the reduction over lanes -- over the most pairs)
   uint32_t ppt = 1;
-  while ((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt) > s.max_grid) ppt *= 2;
+  ppt = tile_pairs_per_thread(n_pairs, s.max_grid, (uint64_t)1 << a.low_bits);
   a.pairs_per_thread = ppt;
   a.deferred = (uint64_t)BLOCK * ppt <= ((uint64_t)1 << a.low_bits) ? 1 : 0;
   uint32_t grid = (uint32_t)((n_pairs + (uint64_t)BLOCK * ppt - 1) / ((uint64_t)BLOCK * ppt));
