@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # The integer-multiply roofline's peak is measured by `--workload mulrate` (run_mulrate below; the issue-rate
 # kernel of sable_amd/csrc/issue_rate.hip): lanes x SIMDs x compute units x clock / cycles per wavefront instruction
 # of v_mad_u64_u32 with many wavefronts resident.  profiles/mulrate_kernel_stats.md holds the run this default is from.
-MULRATE_DEFAULT = {"cycles_per_wave_instruction": 4.7, "clock_ghz": 2.4, "compute_units": 256}
+MULRATE_DEFAULT = {"cycles_per_wave_instruction": 4.9, "clock_ghz": 2.4, "compute_units": 256}
 
 
 def int32_mul_peak(rate=None):
@@ -45,9 +45,11 @@ def int32_mul_peak(rate=None):
 # the same counter reads for the plain copy kernel of `--workload copy`), and 32-bit integer multiply instructions
 # per lane and prove from the kernels' instruction streams times their trip counts (profiles/ holds both summaries).
 MEASURED = {
-    "kernel_sources_sha256": "1613bf95a80d17178e51f2f030678ca66368cf43f4f3d37e2ec7c6b544cf17d0",
-    "traffic": {("round_nodes_base", 24): 203455684, ("round_fold2_base", 24): 403998986},
-    "int32_mul_per_prove": 2063597568,
+    "kernel_sources_sha256": "1cb054f0ec17f75b8c7482d0fb62814115899f5c1336fedbce43b8ab3f373466",
+    "traffic": {("round_nodes_base", 24): 204067331, ("round_fold2_base", 24): 403962385},
+    # per pair: 76 multiply-adds in the sweep (2^22 pairs of four entries), 272 multiply-adds and 96 multiplies of
+    # the reductions in the extension rounds (2^21 + 2^20 + ... pairs)
+    "int32_mul_per_prove": 76 * (1 << 22) + 368 * ((1 << 21) + (1 << 20) + (1 << 19) + (1 << 19)),
 }
 KERNEL_SOURCES = ["sumcheck_kernels.hpp", "field.hpp", "dev_transcript.hpp", "blake3.hpp", "stmtdesc.hpp"]
 
