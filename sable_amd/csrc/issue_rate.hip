@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "blake3.hpp"
 #include "context.hpp"
 
 namespace exh {
@@ -41,6 +42,8 @@ enum IssueOp : int {
   OP_CMP_2CNDMASK,  // one comparison, two selects that read it (three instructions)
   OP_CMP_GAP_CNDMASK,  // a comparison, four other instructions, then the select (six instructions)
   OP_CMP_SGPR_CNDMASK,  // the comparison into a scalar register pair and the select reading that (two instructions)
+  OP_B3_COMPRESS,  // a BLAKE3 compression as the Merkle kernels run it (compiled code, not assembly): its instructions
+                   // (230 v_xor, 224 v_alignbit, 116 v_add, 108 v_add3) in their real order and dependence
   OP_COUNT
 };
 
@@ -49,9 +52,10 @@ static const char *const kOpNames[OP_COUNT] = {
     "v_add_u32",     "v_sub_u32+v_min_u32", "v_xor_b32", "v_alignbit_b32", "v_add3_u32", "v_fma_f32",
     "v_add_co_u32+v_addc_co_u32", "v_cvt_f64_u32", "v_min_u32", "v_cndmask_b32(vcc written once, long before)", "v_perm_b32", "v_alignbyte_b32",
     "v_lshlrev_b32", "v_lshl_or_b32", "v_xad_u32", "v_cmp_lt_u32+v_cndmask_b32", "v_cmp_lt_u32", "v_cndmask_b32(sgpr mask)",
-    "v_cmp_lt_u32+2 v_cndmask_b32", "v_cmp_lt_u32+4 v_xor_b32+v_cndmask_b32", "v_cmp_lt_u32(sgpr)+v_cndmask_b32(sgpr)"};
+    "v_cmp_lt_u32+2 v_cndmask_b32", "v_cmp_lt_u32+4 v_xor_b32+v_cndmask_b32", "v_cmp_lt_u32(sgpr)+v_cndmask_b32(sgpr)",
+    "blake3 compression (678 instructions)"};
 static const int kOpInstructions[OP_COUNT] = {1, 1, 1, 1, 1, 1, 1, 2, 1, 1, 1, 1, 2, 1, 1, 1,
-                                              1, 1, 1, 1, 1, 2, 1, 1, 3, 6, 2};
+                                              1, 1, 1, 1, 1, 2, 1, 1, 3, 6, 2, 678};
 
 constexpr int ISSUE_BLOCK = 256;
 
@@ -128,6 +132,17 @@ __global__ __launch_bounds__(ISSUE_BLOCK) void issue_rate_kernel(uint32_t *out, 
           uint64_t mask;
           asm volatile("v_cmp_lt_u32 %1, %0, %2\n\tv_cndmask_b32 %0, %0, %3, %1" : "+v"(u[i]), "=&s"(mask) : "v"(ia), "v"(ib));
         }
+        if constexpr (OP == OP_B3_COMPRESS) {
+          if (i == 0) {  // one compression per link, whatever the number of chains: it has four of its own
+            uint32_t cv[8], m[16];
+#pragma unroll
+            for (int k = 0; k < 8; k++) cv[k] = u[0] + k;
+#pragma unroll
+            for (int k = 0; k < 16; k++) m[k] = ia + k;
+            b3_compress(cv, m, 0, 64, 11, cv, 0);
+            u[0] = cv[0] ^ cv[1] ^ cv[2] ^ cv[3] ^ cv[4] ^ cv[5] ^ cv[6] ^ cv[7];
+          }
+        }
         if constexpr (OP == OP_CNDMASK_SGPR) {
           uint64_t mask = 0x5555555555555555ull;
           asm volatile("v_cndmask_b32 %0, %0, %1, %2" : "+v"(u[i]) : "v"(ia), "s"(mask));
@@ -200,7 +215,9 @@ int issue_rate(int op, int chains, int workgroups, int iterations, const char **
   hipDeviceProp_t prop;
   EXH_HIP(hipGetDeviceProperties(&prop, c.device));
   if (name) *name = kOpNames[op];
-  if (instructions_per_wave) *instructions_per_wave = (double)iterations * 8.0 * chains * kOpInstructions[op];
+  // (a compression is one per link whatever the number of chains)
+  if (instructions_per_wave)
+    *instructions_per_wave = (double)iterations * 8.0 * (op == OP_B3_COMPRESS ? 1 : chains) * kOpInstructions[op];
   if (clock_khz) *clock_khz = prop.clockRate;
   if (compute_units) *compute_units = prop.multiProcessorCount;
   return OK;
