@@ -403,3 +403,52 @@ def test_a_wide_statement_in_parts_when_the_direct_form_is_switched_off(monkeypa
     assert tr.proof() == otr.proof()
     for t in dev:
         t.free()
+
+
+@pytest.mark.parametrize("host_rounds", [False, True])
+def test_many_blocks_keep_a_tile_within_a_block(host_rounds, monkeypatch):
+    """Block weights over many small blocks: a streaming launch's tile stops growing at the span of one HIGH weight
+    (a block), so the grid is larger than the resident cap and -- in host-driven rounds -- so is the table of
+    partial rows."""
+    if host_rounds:
+        monkeypatch.setenv("EXACTA_HIP_HOST_ROUNDS", "1")
+    K, n, d = 600, 10, 4
+    rng = np.random.default_rng(77)
+    tables = [rand_ext(rng, (K << n,), d) for _ in range(2)]
+    bw = rand_ext(rng, (K,), d)
+    prove_both("bw-many", d, n, "(* t0 t1)", ["t0", "t1"], tables, eq=rand_ext(rng, (n,), d), block_weights=bw,
+               degree=2, sc_label="gkr")
+
+
+WIDE_FORMS = [
+    # five-term sums are no linear forms for the kernels (four terms at most), so the products are multiplied out:
+    # 25 and 50 table monomials
+    ("(* (+ t0 t1 t2 t3 t4) (- t5 t6 t7 t8 t9))", 10, []),
+    ("(+ (* k0 (expt (+ t0 t1 t2 t3 t4) 2) (- t5)) (* 7 (+ t5 t6 t7 t8 t9) (+ t0 t2 t4 t6 t8)) (- k1 3))", 10, ["k0", "k1"]),
+]
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("form,nt,cnames", WIDE_FORMS)
+@pytest.mark.parametrize("d,n,mixed", [(4, 7, False), (4, 11, True)])
+def test_wide_forms_of_other_shapes_in_direct_form(form, nt, cnames, d, n, mixed):
+    """Powers, unary minus, integer factors, a table-free term, and base tables beside extension tables."""
+    names = [f"t{i}" for i in range(nt)]
+    st, ost = both(form, names, cnames)
+    rng = np.random.default_rng(4300 + n + nt)
+    tables = [rand_ext(rng, (1 << n,), d) if (mixed and i % 3 == 0) else rng.integers(0, P, 1 << n, dtype=np.uint32)
+              for i in range(nt)]
+    eq = rand_ext(rng, (n,), d)
+    cv = rand_ext(rng, (len(cnames),), d) if cnames else None
+    dev = [sa.Table.upload(t) for t in tables]
+    assert st.generate(d, wait=True)
+    assert same(sa.hypercube_sum(st, n, dev, d, eq=eq, constants=cv), orc.hypercube_sum(ost, n, tables, d, eq=eq, constants=cv))
+    tr, otr = sa.Transcript("wide2", d), orc.Transcript("wide2", d)
+    out = {}
+    names_launched = launch_names(lambda: out.setdefault("got", sa.prove(tr, n, st, dev, eq=eq, constants=cv)))
+    want = orc.prove(otr, n, ost, tables, eq=eq, constants=cv)
+    assert tr.proof() == otr.proof()
+    assert same(out["got"][0], want[0]) and same(out["got"][1], want[1])
+    assert len([name for name in names_launched if name.startswith("round_")]) < n, names_launched
+    for t in dev:
+        t.free()
