@@ -140,8 +140,8 @@ __device__ inline void dev_absorb_words(RunB3S &s, const uint32_t *words, uint32
   }
 }
 
-// K <= 8 base-field challenges (CHALLENGE-BASE, src/transcript.lisp:159-172): squeeze 4 (missing + 4)
-// bytes, keep the 31-bit words below p, repeat until K are kept; each squeeze then absorbs "squeeze" and
+// K <= 12 base-field challenges (CHALLENGE-BASE, src/transcript.lisp:159-172): squeeze 4 (missing + 4)
+// bytes (at most 64: one output block), keep the 31-bit words below p, repeat until K are kept; each squeeze then absorbs "squeeze" and
 // the first min(32, n) bytes of its output (src/transcript.lisp:152-157).  OUT is in LDS.
 // `ready` is called by the whole wavefront as soon as the K challenges are in OUT: what follows (absorbing the last
 // squeeze's bytes, a compression when they fill the block) is the transcript's own bookkeeping, which whoever waits
@@ -152,10 +152,10 @@ __device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out, F ready) {
   uint32_t *stage = s.ring + 32;
   int have = 0;
   while (have < k) {
-    const uint32_t n = 4u * (uint32_t)(k - have + 4);  // at most 48 bytes: one output block
+    const uint32_t n = 4u * (uint32_t)(k - have + 4);  // at most 64 bytes: one output block
     uint32_t w0, w1, w2, w3;
     b3_compress_quad(s.cv, s.ring + 16 * s.half, 0, s.used, B3_CHUNK_END | B3_ROOT, w0, w1, w2, w3);
-    if (lane < 4) stage[lane] = w0, stage[4 + lane] = w1, stage[8 + lane] = w2;
+    if (lane < 4) stage[lane] = w0, stage[4 + lane] = w1, stage[8 + lane] = w2, stage[12 + lane] = w3;
     __builtin_amdgcn_wave_barrier();
     // "squeeze", then the first min(32, n) bytes of the output
     const uint32_t fed = n < 32 ? n : 32;

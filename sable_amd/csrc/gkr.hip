@@ -432,7 +432,7 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
   {  // one block: the layers chained on the device, one wait for the whole proof
     const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS"), *no_chain = getenv("EXACTA_HIP_NO_GKR_CHAIN");
     const bool off = (host_rounds && host_rounds[0] == '1') || (no_chain && no_chain[0] == '1');
-    if (K == 1 && n >= 2 && n - 2 <= MAXROUNDS && L * D <= 8 && 2 * L <= GLUE_MAXCONST && !off) {
+    if (K == 1 && n >= 2 && n - 2 <= MAXROUNDS && L * D <= 12 && 2 * L <= GLUE_MAXCONST && !off) {
       status = D == 4 ? prove_upper_chained<4>(tr, n, L, layers, label, out_ri, out_cp, out_cq)
                       : prove_upper_chained<8>(tr, n, L, layers, label, out_ri, out_cp, out_cq);
       if (status) return status;

@@ -39,9 +39,9 @@ def test_reduce_layer(d, k, m):
 
 CASES = [(3, 1, 1, 4), (3, 3, 2, 4), (2, 4, 1, 8), (4, 5, 2, 4), (1, 2, 1, 4), (1, 1, 2, 8), (2, 2, 3, 4),
          (10, 1, 1, 4), (6, 1, 2, 8),
-         # one block: the layers chained on the device (up to eight base challenges per layer), from the smallest
+         # one block: the layers chained on the device (up to twelve base challenges per layer), from the smallest
          # tree that chains to one whose upper layers take the grid of slices
-         (2, 1, 1, 4), (5, 1, 2, 4), (7, 1, 1, 8), (13, 1, 1, 4), (12, 1, 2, 4)]
+         (2, 1, 1, 4), (5, 1, 2, 4), (7, 1, 1, 8), (13, 1, 1, 4), (12, 1, 2, 4), (6, 1, 3, 4), (11, 1, 3, 4)]
 
 
 @pytest.mark.parametrize("n,k,lookups,d", CASES)
@@ -72,7 +72,7 @@ def test_prove_upper_matches_the_oracle(n, k, lookups, d):
         p.free(), q.free()
 
 
-@pytest.mark.parametrize("n,lookups,d", [(9, 1, 4), (6, 2, 4), (8, 1, 8)])
+@pytest.mark.parametrize("n,lookups,d", [(9, 1, 4), (6, 2, 4), (8, 1, 8), (7, 3, 4)])
 def test_the_chained_layers_and_the_host_driven_layers_send_the_same_bytes(n, lookups, d, monkeypatch):
     rng = np.random.default_rng(100 + n)
     leaves = random_leaves(rng, lookups, n, 1, d)
