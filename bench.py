@@ -45,7 +45,7 @@ def int32_mul_peak(rate=None):
 # the same counter reads for the plain copy kernel of `--workload copy`), and 32-bit integer multiply instructions
 # per lane and prove from the kernels' instruction streams times their trip counts (profiles/ holds both summaries).
 MEASURED = {
-    "kernel_sources_sha256": "1cb054f0ec17f75b8c7482d0fb62814115899f5c1336fedbce43b8ab3f373466",
+    "kernel_sources_sha256": "4c6f57cee8b42c6c11d9c19efbda2ec74de56d3d30fea849ece36455fc392118",
     "traffic": {("round_nodes_base", 24): 204067331, ("round_fold2_base", 24): 403962385},
     # per pair: 76 multiply-adds in the sweep (2^22 pairs of four entries), 272 multiply-adds and 96 multiplies of
     # the reductions in the extension rounds (2^21 + 2^20 + ... pairs)
