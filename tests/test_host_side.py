@@ -168,3 +168,15 @@ def test_statement_compile_matches_expand():
         tv = rng.integers(0, sa.P, (len(names), 8), dtype=np.uint32)
         cv = rng.integers(0, sa.P, (max(len(cnames), 1), 8), dtype=np.uint32)
         assert sa.check_final(ost.evaluate(tv, cv, 8), st, tv, constants=cv if cnames else None)
+
+
+def test_the_bench_constants_go_with_the_present_kernel_sources():
+    """bench.py reports measured traffic and multiply counts only for the version of the kernels they were measured
+    on: the stamp has to be renewed (with the figures) when the kernels' sources change."""
+    import importlib.util
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert bench.MEASURED["kernel_sources_sha256"] == bench.kernel_sources_sha256()
