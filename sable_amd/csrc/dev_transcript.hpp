@@ -146,8 +146,18 @@ __device__ inline void dev_absorb_words(RunB3S &s, const uint32_t *words, uint32
 // `ready` is called by the whole wavefront as soon as the K challenges are in OUT: what follows (absorbing the last
 // squeeze's bytes, a compression when they fill the block) is the transcript's own bookkeeping, which whoever waits
 // for the challenge need not wait for.
+// With `pending` (not null) the bytes the last squeeze leaves to absorb are handed back instead of absorbed: the
+// caller absorbs them later (rb3s_flush), before anything else goes through the transcript -- in a round's serial
+// part they would stand between the challenge and the fold that waits for it.
+struct PendingAppend {
+  uint32_t byte, len;  // this lane's byte of the stream; bytes in all (0: nothing pending)
+};
+__device__ inline void rb3s_flush(RunB3S &s, PendingAppend &pending) {
+  if (pending.len) rb3s_append_bytes(s, pending.byte, pending.len);
+  pending.len = 0;
+}
 template <class F>
-__device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out, F ready) {
+__device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out, F ready, PendingAppend *pending = nullptr) {
   const uint32_t lane = threadIdx.x & 63;
   uint32_t *stage = s.ring + 32;
   int have = 0;
@@ -172,6 +182,10 @@ __device__ inline void dev_challenge(RunB3S &s, int k, uint32_t *out, F ready) {
     have += __popcll(ok);
     __builtin_amdgcn_wave_barrier();
     if (have >= k) ready();
+    if (have >= k && pending) {
+      pending->byte = byte, pending->len = 7 + fed;
+      return;
+    }
     rb3s_append_bytes(s, byte, 7 + fed);
   }
 }

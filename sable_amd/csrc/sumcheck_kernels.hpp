@@ -679,14 +679,16 @@ __device__ __forceinline__ void round_message(const uint32_t *sums, uint32_t nac
 // instead of a barrier and begin the fold while this one finishes the transcript's bookkeeping.
 template <int D>
 __device__ __forceinline__ void transcript_step(RunB3S &tr, Ctrl *ctrl, uint32_t round, uint32_t points,
-                                                EpilogueLds *e, bool log = true, uint32_t *publish = nullptr) {
+                                                EpilogueLds *e, bool log = true, uint32_t *publish = nullptr,
+                                                PendingAppend *pending = nullptr) {
   const uint32_t tid = threadIdx.x;
+  if (pending) rb3s_flush(tr, *pending);
   dev_absorb_words(tr, e->msg, points * D);
   dev_challenge(tr, D, e->chal, [&] {
     if (tid < (uint32_t)D) e->r_mont[tid] = to_mont(e->chal[tid]);
     __builtin_amdgcn_wave_barrier();
     if (publish && tid == 0) __hip_atomic_store(publish, round + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  });
+  }, pending);
   if (log)
     for (uint32_t o = tid; o < points * D; o += 64) ctrl->msg[round][o] = e->msg[o];
   if (log && tid < (uint32_t)D) ctrl->chal[round][tid] = e->chal[tid], ctrl->r_mont[tid] = e->r_mont[tid];
@@ -1001,7 +1003,7 @@ __global__ __launch_bounds__(EPI_BLOCK) void epilogue_kernel(EpilogueArgs args) 
 
 // A small round's sums on one wavefront: the accumulators PART, PART + 4, ... of the lane's pair, summed over the
 // wavefront into sums (LDS).  The accumulators are this function's own, so that they live in registers.
-template <int D, int PART, class Desc>
+template <int D, int PART, int PARTS, class Desc>
 __device__ __forceinline__ void small_round_sums(const Desc &d, const Ext<D> *lo, const Ext<D> *hi, const Ext<D> &w,
                                                  uint32_t *sums, const uint32_t *kc) {
   Acc96 acc[MAXACC][D];
@@ -1009,8 +1011,8 @@ __device__ __forceinline__ void small_round_sums(const Desc &d, const Ext<D> *lo
   for (int a = 0; a < MAXACC; a++)
 #pragma unroll
     for (int c = 0; c < D; c++) acc_zero(acc[a][c]);
-  accumulate_pair<D, Ext<D>, Desc, 4, PART>(d, lo, hi, w, acc, kc);
-  part_wave_sums<D, PART, 4>(d, acc, sums);
+  accumulate_pair<D, Ext<D>, Desc, PARTS, PART>(d, lo, hi, w, acc, kc);
+  part_wave_sums<D, PART, PARTS>(d, acc, sums);
 }
 
 // Load (folding or lifting on the way in) into LDS, then per round sums -> message -> challenge -> fold
@@ -1030,6 +1032,7 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   const uint32_t width = (uint32_t)d.nacc * D;
   if (args.ctrl->round != args.first_round) return;  // an earlier launch gave up: leave the count as it is
   RunB3S tr;
+  PendingAppend pending{0, 0};  // (the first wavefront's)
   if (tid < 64) rb3s_load(tr, epi.ring, &args.ctrl->tr);
   uint32_t entries = (args.first_fold ? args.entries / 2 : args.entries) / G;  // of this workgroup's slice
   {
@@ -1110,14 +1113,16 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
         Ext<D> ww = ext_mul_mont<D>(wl, wh);
         if (lane >= pairs) ww = ext_zero<D>();  // lanes without a pair add nothing
         if (jj + 1 < args.rounds) fetch_weight(jj + 1, pairs / 2);
+        // three wavefronts share the accumulators; the first, which ran the transcript, meanwhile absorbs what the
+        // last squeeze left to absorb (a compression every other round): nobody waits for that any more
         if (wave == 0)
-          small_round_sums<D, 0>(d, lo, hi, ww, sums, args.consts);
+          rb3s_flush(tr, pending);
         else if (wave == 1)
-          small_round_sums<D, 1>(d, lo, hi, ww, sums, args.consts);
+          small_round_sums<D, 0, 3>(d, lo, hi, ww, sums, args.consts);
         else if (wave == 2)
-          small_round_sums<D, 2>(d, lo, hi, ww, sums, args.consts);
+          small_round_sums<D, 1, 3>(d, lo, hi, ww, sums, args.consts);
         else
-          small_round_sums<D, 3>(d, lo, hi, ww, sums, args.consts);
+          small_round_sums<D, 2, 3>(d, lo, hi, ww, sums, args.consts);
         lds_barrier();
       } else {
         Acc96 acc[MAXACC][D];
@@ -1188,7 +1193,7 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
       // the first wavefront publishes the challenge the moment it is drawn and finishes the transcript's step while
       // the others, which wait for that word alone, are already folding
       if (tid < 64) {
-        transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi, wg == 0, &ready_round);
+        transcript_step<D>(tr, args.ctrl, args.first_round + jj, args.points, &epi, wg == 0, &ready_round, &pending);
       } else {
         while (__hip_atomic_load(&ready_round, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != args.first_round + jj + 1)
           __builtin_amdgcn_s_sleep(1);
@@ -1233,6 +1238,7 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
                      load_ext<D>(tail_tables + ((size_t)t * cap + x) * D));
   if (G == 1 && entries == 1 && tid < (uint32_t)d.T * D)  // the finals travel with the logs
     args.ctrl->finals[tid] = tail_tables[(size_t)(tid / D) * cap * D + tid % D];
+  if (tid < 64) rb3s_flush(tr, pending);
   if (wg == 0 && tid < 64) {
     rb3s_store(tr, &args.ctrl->tr);
     if (tid == 0) args.ctrl->round = args.first_round + args.rounds;
