@@ -473,16 +473,51 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
   std::vector<uint32_t> consts, finals((size_t)(NT + 1) * D), rho((size_t)(n + lk + 1) * D);
   std::vector<uint32_t> r, ri;
   uint64_t dims2[2] = {2, (uint64_t)D};
-  for (int l = 0; l < L; l++) {  // the roots
-    uint32_t root[16];
-    memcpy(root, top[0][2 * l].data(), 4 * D);
-    memcpy(root + D, top[0][2 * l + 1].data(), 4 * D);
-    if ((status = tr.send(root, 2, dims2, nullptr))) return status;
-    cp[l] = hf::from(root, D);
-    cq[l] = hf::from(root + D, D);
-  }
   std::vector<int> strides(NT + 1, D);
-  for (int j = 0; j < lk; j++) {  // the top tree
+  // The top tree is a tree of one block over the block index: its roots and layers are PROVE-UPPER's with one
+  // block under the label's "-top", so the chain above serves it as well (one wait instead of one per layer).
+  bool top_chained = false;
+  {
+    const char *host_rounds = getenv("EXACTA_HIP_HOST_ROUNDS"), *no_chain = getenv("EXACTA_HIP_NO_GKR_CHAIN");
+    const bool off = (host_rounds && host_rounds[0] == '1') || (no_chain && no_chain[0] == '1');
+    if (lk >= 1 && lk - 1 <= MAXROUNDS && L * D <= 12 && 2 * L <= GLUE_MAXCONST && !off) {
+      // every level of every lookup's top tree in one buffer, one copy
+      std::vector<std::vector<const uint32_t *>> top_layers(lk + 1, std::vector<const uint32_t *>(2 * L));
+      std::vector<uint32_t> all;
+      std::vector<std::vector<size_t>> at(lk + 1, std::vector<size_t>(2 * L));
+      for (int j = 0; j <= lk; j++)
+        for (int i = 0; i < 2 * L; i++) {
+          at[j][i] = all.size();
+          all.insert(all.end(), top[j][i].begin(), top[j][i].end());
+        }
+      uint32_t *d_top = bufs.alloc(all.size());
+      if (!d_top) return E_NOMEM;
+      EXH_HIP(hipMemcpyAsync(d_top, all.data(), all.size() * 4, hipMemcpyHostToDevice, c.stream));
+      for (int j = 0; j <= lk; j++)
+        for (int i = 0; i < 2 * L; i++) top_layers[j][i] = d_top + at[j][i];
+      r.assign((size_t)lk * D, 0);
+      std::vector<uint32_t> ocp((size_t)L * D), ocq((size_t)L * D);
+      status = D == 4 ? prove_upper_chained<4>(tr, lk + 1, L, top_layers, label + "-top", r.data(), ocp.data(), ocq.data())
+                      : prove_upper_chained<8>(tr, lk + 1, L, top_layers, label + "-top", r.data(), ocp.data(), ocq.data());
+      if (status) return status;
+      for (int l = 0; l < L; l++) {
+        cp[l] = hf::from(&ocp[(size_t)l * D], D);
+        cq[l] = hf::from(&ocq[(size_t)l * D], D);
+      }
+      top_chained = true;
+    }
+  }
+  if (!top_chained) {
+    for (int l = 0; l < L; l++) {  // the roots
+      uint32_t root[16];
+      memcpy(root, top[0][2 * l].data(), 4 * D);
+      memcpy(root + D, top[0][2 * l + 1].data(), 4 * D);
+      if ((status = tr.send(root, 2, dims2, nullptr))) return status;
+      cp[l] = hf::from(root, D);
+      cq[l] = hf::from(root + D, D);
+    }
+  }
+  for (int j = 0; j < lk && !top_chained; j++) {  // the top tree, layer by layer
     layer_challenges(tr, D, L, consts, as, lam);
     uint64_t size = (uint64_t)1 << j;
     std::vector<const uint32_t *> tabs(NT);
@@ -533,24 +568,23 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
           tabs[4 * l + 2 * w + 1] = hi;
         }
       }
-    std::vector<std::vector<uint32_t>> folded(NT, std::vector<uint32_t>(Kp * D, 0));  // zero padded to 2^lk
-    std::vector<uint32_t *> fptr(NT);
-    for (int t = 0; t < NT; t++) fptr[t] = folded[t].data();
+    // With several blocks the folded tables (one entry per block) stay on the device, zero padded to 2^lk, as the
+    // tables of the sumcheck over the block index; the weights, padded alike, go before them in one copy.
+    uint32_t *d_blk = nullptr;
+    if (lk > 0) {
+      if (!(d_blk = bufs.alloc((uint64_t)(NT + 1) * Kp * D))) return E_NOMEM;
+    }
     status = sumcheck_prove(tr, layer, st, tabs.data(), strides.data(), layer > 0 ? ri.data() : nullptr,
-                            consts.data(), label, bw.data(), K, layer > 0 ? 2 : 0, rho.data(), finals.data(),
-                            fptr.data());
+                            consts.data(), label, bw.data(), K, layer > 0 ? 2 : 0, rho.data(),
+                            lk > 0 ? nullptr : finals.data(), nullptr, lk > 0 ? d_blk + Kp * D : nullptr, Kp);
     if (status) return status;
     std::vector<uint32_t> rbn;
     if (lk > 0) {  // bind the block index: the blocks' values and weights, padded with zeros
       std::vector<const uint32_t *> btabs(NT + 1);
       std::vector<uint32_t> bwp(Kp * D, 0);
       memcpy(bwp.data(), bw.data(), (size_t)K * D * 4);
-      for (int t = 0; t <= NT; t++) {
-        uint32_t *d = bufs.alloc(Kp * D);
-        if (!d) return E_NOMEM;
-        EXH_HIP(hipMemcpy(d, t == 0 ? bwp.data() : folded[t - 1].data(), Kp * D * 4, hipMemcpyHostToDevice));
-        btabs[t] = d;
-      }
+      EXH_HIP(hipMemcpyAsync(d_blk, bwp.data(), Kp * D * 4, hipMemcpyHostToDevice, c.stream));
+      for (int t = 0; t <= NT; t++) btabs[t] = d_blk + (uint64_t)t * Kp * D;
       std::vector<uint32_t> f2((size_t)(NT + 1) * D);
       rbn.assign((size_t)lk * D, 0);
       status = sumcheck_prove(tr, lk, st_blk, btabs.data(), strides.data(), nullptr, consts.data(), label + "-blk",

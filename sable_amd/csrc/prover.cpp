@@ -115,7 +115,8 @@ int hypercube_sum_wide(const Statement &st, int D, int n, const uint32_t *const 
 static int sumcheck_prove_wide(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables,
                                const int *strides, const uint32_t *eq, const uint32_t *consts, const std::string &label,
                                const uint32_t *bw, int K, int degree, int points, uint32_t *out_chal,
-                               uint32_t *out_finals, uint32_t *const *out_folded) {
+                               uint32_t *out_finals, uint32_t *const *out_folded, uint32_t *d_folded,
+                               uint64_t d_folded_len) {
   const int D = tr.D;
   std::vector<Statement> parts;
   if (int dealt = deal_parts(st, points, &parts)) return dealt;
@@ -142,12 +143,15 @@ static int sumcheck_prove_wide(Transcript &tr, int n, const Statement &st, const
     for (auto &s : sessions)
       if ((status = s->fold(r))) return status;
   }
-  return sessions[0]->finish(out_finals, out_folded);  // every part folded the same tables
+  // every part folded the same tables
+  if (d_folded && (status = sessions[0]->finish_device(d_folded, d_folded_len))) return status;
+  return sessions[0]->finish(out_finals, out_folded);
 }
 
 int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables, const int *strides,
                    const uint32_t *eq, const uint32_t *consts, const std::string &label, const uint32_t *bw, int K,
-                   int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded) {
+                   int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded,
+                   uint32_t *d_folded, uint64_t d_folded_len) {
   int D = tr.D;
   if (degree < 0) degree = st.degree;
   int points = degree > 1 ? degree : 1;
@@ -169,7 +173,7 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
     }
     if (!direct)
       return sumcheck_prove_wide(tr, n, st, d_tables, strides, eq, consts, label, bw, K, degree, points, out_chal,
-                                 out_finals, out_folded);
+                                 out_finals, out_folded, d_folded, d_folded_len);
   }
   if (status) return status;
   SumcheckSession &s = direct ? second : first;
@@ -200,6 +204,7 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
       }
     }
     if (!replaying && (status = adopt_device_state(tr, final_state))) return status;
+    if (d_folded && (status = s.finish_device(d_folded, d_folded_len))) return status;
     return s.finish(out_finals, out_folded);
   }
   uint32_t sums[16 * 8];
@@ -211,6 +216,7 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
     tr.challenge(D, r);
     if ((status = s.fold(r))) return status;
   }
+  if (d_folded && (status = s.finish_device(d_folded, d_folded_len))) return status;
   return s.finish(out_finals, out_folded);
 }
 

@@ -17,7 +17,10 @@ int hypercube_sum_wide(const Statement &st, int D, int n, const uint32_t *const 
 // tables: device pointers, K * 2^n entries of stride 1 or D each, block-major.
 int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *const *d_tables, const int *strides,
                    const uint32_t *eq, const uint32_t *consts, const std::string &label, const uint32_t *bw, int K,
-                   int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded);
+                   int degree, uint32_t *out_chal, uint32_t *out_finals, uint32_t *const *out_folded,
+                   uint32_t *d_folded = nullptr, uint64_t d_folded_len = 0);
+// (d_folded: the folded tables are also left on the device, table t at d_folded + t * d_folded_len * D, zeros after
+// its K entries; with out_finals and out_folded null nothing of them comes to the host)
 int sumcheck_verify(Transcript &tr, int n, const Statement &st, const uint32_t *claim, const uint32_t *eq,
                     const uint32_t *consts, int blocks, const std::string &label, int degree, uint32_t *out_chal,
                     uint32_t *out_reduced);

@@ -836,12 +836,50 @@ int SumcheckSession::flush() {
   return OK;
 }
 
+// table t's entries (stride 1 or D) as `padded` extension elements at out + t * padded * D: lifted, then zeros
+struct PadArgs {
+  const uint32_t *in[MAXT];
+  uint32_t *out;
+  uint64_t size, padded;
+  uint32_t in_stride, D;
+};
+__global__ __launch_bounds__(BLOCK) void pad_tables_kernel(PadArgs a) {
+  const uint64_t u = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;  // word of table blockIdx.y's output
+  if (u >= a.padded * a.D) return;
+  const uint64_t x = u / a.D;
+  const uint32_t k = (uint32_t)(u % a.D);
+  uint32_t v = 0;
+  if (x < a.size) v = a.in_stride == 1 ? (k == 0 ? a.in[blockIdx.y][x] : 0u) : a.in[blockIdx.y][x * a.D + k];
+  a.out[((uint64_t)blockIdx.y * a.padded) * a.D + u] = v;
+}
+
+int SumcheckSession::finish_device(uint32_t *d_out, uint64_t padded) {
+  Context &c = ctx();
+  if (int owned = owns_arenas()) return owned;
+  int status = flush();
+  if (status) return status;
+  const int T = st.T();
+  if (padded < size || T < 1) {
+    set_error("invalid-parameter: the padded length of the folded tables");
+    return E_PARAM;
+  }
+  PadArgs a;
+  memset(&a, 0, sizeof(a));
+  for (int t = 0; t < T; t++) a.in[t] = cur[t];
+  a.out = d_out, a.size = size, a.padded = padded, a.in_stride = cur_base ? 1u : (uint32_t)D, a.D = (uint32_t)D;
+  const uint32_t grid = (uint32_t)((padded * D + BLOCK - 1) / BLOCK);
+  hipLaunchKernelGGL(pad_tables_kernel, dim3(grid, T), dim3(BLOCK), 0, c.stream, a);
+  EXH_HIP(hipGetLastError());
+  return OK;
+}
+
 int SumcheckSession::finish(uint32_t *finals, uint32_t *const *folded) {
   Context &c = ctx();
   if (int owned = owns_arenas()) return owned;
   int status = flush();
   if (status) return status;
   int T = st.T();
+  if (!finals && !folded) return OK;
   // each table's current entries (K of them after n rounds), lifted if still base
   const uint64_t words = size * (cur_base ? 1 : D);
   const bool cached = !cur_base && final_cache.size() == (size_t)T * words;

@@ -132,6 +132,10 @@ struct SumcheckSession {
   int fold(const uint32_t *r /* D */);
   // finals: T * D; folded[t] (optional): K * D each
   int finish(uint32_t *finals, uint32_t *const *folded);
+  // the same tables left on the device instead: table t's entries at d_out + t * padded * D, lifted if still base,
+  // zeros from its last entry up to `padded` (what a sumcheck over the block index takes as its tables).  Enqueued
+  // on the session's stream; nothing is copied to the host.
+  int finish_device(uint32_t *d_out, uint64_t padded);
   // device pointers of the current (fully or partly folded) tables, after any pending fold
   int flush();
 };

@@ -39,6 +39,9 @@ def test_reduce_layer(d, k, m):
 
 CASES = [(3, 1, 1, 4), (3, 3, 2, 4), (2, 4, 1, 8), (4, 5, 2, 4), (1, 2, 1, 4), (1, 1, 2, 8), (2, 2, 3, 4),
          (10, 1, 1, 4), (6, 1, 2, 8),
+         # several blocks at sizes where the layers' sumchecks run on the device-driven loop, the top tree on the
+         # chain and the folded tables stay on the device for the sumcheck over the block index
+         (9, 3, 1, 4), (8, 2, 2, 4), (7, 6, 1, 8), (11, 4, 3, 4),
          # one block: the layers chained on the device (up to twelve base challenges per layer), from the smallest
          # tree that chains to one whose upper layers take the grid of slices
          (2, 1, 1, 4), (5, 1, 2, 4), (7, 1, 1, 8), (13, 1, 1, 4), (12, 1, 2, 4), (6, 1, 3, 4), (11, 1, 3, 4)]
