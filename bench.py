@@ -45,7 +45,7 @@ def int32_mul_peak(rate=None):
 # the same counter reads for the plain copy kernel of `--workload copy`), and 32-bit integer multiply instructions
 # per lane and prove from the kernels' instruction streams times their trip counts (profiles/ holds both summaries).
 MEASURED = {
-    "kernel_sources_sha256": "130da64e4926ed6efcfd37d20ea85183aaba229e7c86631139222e3c81f22e85",
+    "kernel_sources_sha256": "84841755ff915996f2c965a0c6de1e5fbe22a98773f07c1cce7a8c3f1a8ddc0f",
     "traffic": {("round_nodes_base", 24): 204067331, ("round_fold2_base", 24): 403962385},
     # per pair: 76 multiply-adds in the sweep (2^22 pairs of four entries), 272 multiply-adds and 96 multiplies of
     # the reductions in the extension rounds (2^21 + 2^20 + ... pairs)

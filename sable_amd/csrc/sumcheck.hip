@@ -472,6 +472,7 @@ int SumcheckSession::launch_setup() {
   uint64_t zero_words = size / 2 > tail_pairs(st.T(), D) ? zeroed_words : 0;
   const uint32_t zero_grid = (uint32_t)((zero_words + 4 * BLOCK - 1) / (4 * BLOCK));  // four words a thread
   bool cleared = false;
+  c.prof_begin("weights", 0, 0);
   if (setup.total_eq) {
     uint32_t grid = std::max((uint32_t)((setup.total_eq + BLOCK - 1) / BLOCK), zero_grid);
     // tables are laid out in launch order, so thread gid maps to table k by running sums; the
@@ -496,6 +497,7 @@ int SumcheckSession::launch_setup() {
     cleared = cleared || zero_words > 0;
     zero_words = 0;
   }
+  c.prof_end();
   slice_totals_clear = cleared;  // else (no set-up kernel ran) the grid launch clears them itself
   EXH_HIP(hipGetLastError());
   return OK;
@@ -993,6 +995,14 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       }
     }
   }
+  // A session whose every round runs in the one-workgroup launch needs no set-up launch: that launch builds the
+  // weight tables itself from the eq point's factors, which lead the session's constants (EXACTA_HIP_NO_OWN_WEIGHTS=1:
+  // never)
+  {
+    const char *no_own = getenv("EXACTA_HIP_NO_OWN_WEIGHTS");
+    own_weights = setup_deferred && has_eq && !has_bw && setup.total_eq > 0 && !setup.ones_len &&
+                  size / 2 <= tail_pairs(T, D) && n <= MAXTAIL && !(no_own && no_own[0] == '1');
+  }
   if (chain_hook) {  // the chain's launch writes what the copy below would bring
     if (!setup_deferred) {
       set_error("invalid-parameter: a chained session defers its set-up");
@@ -1001,12 +1011,12 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     int st_hook = chain_hook();
     if (st_hook) return st_hook;
     setup_deferred = false;
-    if ((st_hook = launch_setup())) return st_hook;
+    if (!own_weights && (st_hook = launch_setup())) return st_hook;
   } else if (setup_deferred) {  // one copy for the session's constants and the loop's, then the weight tables
     EXH_HIP(hipMemcpyAsync(d_weights, c.host_pinned + PIN_BEGIN, (setup_words + up_words) * 4, hipMemcpyHostToDevice,
                            c.stream));
     setup_deferred = false;
-    int st_setup = launch_setup();
+    int st_setup = own_weights ? OK : launch_setup();
     if (st_setup) return st_setup;
   } else {
     EXH_HIP(hipMemcpyAsync(d_mtilde, up, up_words * 4, hipMemcpyHostToDevice, c.stream));
@@ -1233,6 +1243,12 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
       a.low_off[jj] = low_off[j + jj];
       a.high_off[jj] = high_off[j + jj];
       a.low_bits[jj] = (uint32_t)low_bits[j + jj];
+    }
+    if (own_weights && grid == 1 && j == 0 && rounds == n) {  // the launch builds the weight tables behind its tables
+      uint64_t own_entries = (uint64_t)2 * n;
+      for (int jj = 0; jj < n; jj++) own_entries += ((uint64_t)1 << low_bits[jj]) + n_high[jj];
+      a.factors = d_weights, a.n_vars = (uint32_t)n;
+      a.lds_bytes += (uint32_t)(own_entries * D * 4);
     }
   };
   if (grid > 1 && !slice_totals_clear)  // the rounds' totals start at zero (64-bit words)

@@ -110,6 +110,7 @@ struct SumcheckSession {
   // OK while this is the latest session begun (its arenas have not been handed to another one)
   int owns_arenas() const;
   bool setup_deferred = false;
+  bool own_weights = false;  // the one launch that runs every round builds the weight tables itself
   size_t setup_words = 0;
   struct {
     uint64_t total_eq = 0, ones_off = 0, ones_len = 0;

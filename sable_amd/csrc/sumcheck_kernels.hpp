@@ -119,6 +119,12 @@ struct TailArgs {
   uint32_t *host_log;
   uint32_t host_flag_at, host_seq;
   const uint32_t *consts;  // a statement in direct form: its constant slots (EXTs, Montgomery form)
+  // A session whose every round runs in this one launch builds its weight tables itself, in LDS behind the tables
+  // (no set-up launch): `factors` holds (r_v R, (1 - r_v) R) for the eq point's n_vars variables; round jj's LOW
+  // table covers the low_bits[jj] variables from first_round + jj + 1 on, its HIGH table the rest.  Null: the
+  // tables are read from `weights`.
+  const uint32_t *factors;
+  uint32_t n_vars;
 };
 
 template <int D>
@@ -1068,6 +1074,45 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
     for (uint32_t u = tid; u < args.points * width; u += BLOCK) epi.mtilde[u] = args.mtilde[u];
     for (uint32_t u = tid; u < args.rounds * args.points * D; u += BLOCK) c0s[u] = args.c0[u];
   }
+  // The session's own weight tables (see TailArgs::factors), in LDS behind the tables: the factors first, then
+  // per round its LOW and its HIGH table.  An entry is a chain of at most n_vars products, one entry per thread
+  // and trip: entry x of a table over the variables [first, first + bits) is prod_b (x_b ? r_b : 1 - r_b).
+  const bool own_weights = args.factors != nullptr;
+  uint32_t *const own_factors = tail_tables + (size_t)d.T * cap * D;
+  uint32_t *const own_tables = own_factors + (size_t)2 * args.n_vars * D;
+  auto own_high_bits = [&](uint32_t jj) { return args.n_vars - (args.first_round + jj + 1) - args.low_bits[jj]; };
+  auto own_at = [&](uint32_t jj, bool high) {  // where round jj's LOW (HIGH) table begins, in elements
+    uint32_t at = 0;
+    for (uint32_t q = 0; q < jj; q++) at += (1u << args.low_bits[q]) + (1u << own_high_bits(q));
+    return high ? at + (1u << args.low_bits[jj]) : at;
+  };
+  if (own_weights) {
+    for (uint32_t u = tid; u < 2 * args.n_vars * D; u += BLOCK) own_factors[u] = args.factors[u];
+    __syncthreads();
+    const uint32_t total = own_at(args.rounds, false);
+    for (uint32_t u = tid; u < total; u += BLOCK) {
+      uint32_t jj = 0, start = 0, first = 0, bits = 0;
+      for (;; jj++) {  // (u < total: the scan ends inside the rounds)
+        const uint32_t lb = args.low_bits[jj], hb = own_high_bits(jj);
+        if (u < start + (1u << lb)) {
+          first = args.first_round + jj + 1, bits = lb;
+          break;
+        }
+        start += 1u << lb;
+        if (u < start + (1u << hb)) {
+          first = args.first_round + jj + 1 + lb, bits = hb;
+          break;
+        }
+        start += 1u << hb;
+      }
+      const uint32_t x = u - start;
+      Ext<D> e = ext_lift<D>(1);
+      for (uint32_t b = 0; b < bits; b++)
+        e = ext_mul_mont<D>(e, load_ext<D>(own_factors + ((size_t)(first + b) * 2 + (((x >> b) & 1) ? 0 : 1)) * D));
+      store_ext<D>(own_tables + (size_t)u * D, e);
+    }
+    __syncthreads();
+  }
   // the weight factors of this thread's first pair of a round, fetched one round ahead
   Ext<D> wl = ext_zero<D>(), wh = ext_zero<D>();
   // (a round of at most 64 pairs runs with a pair per lane on all four wavefronts, each computing a share of the
@@ -1078,6 +1123,11 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
   auto fetch_weight = [&](uint32_t jj, uint32_t pairs) {
     const uint32_t me = pairs <= 64 ? lane : tid;
     const uint64_t i = (uint64_t)wg * pairs + (me < pairs ? me : pairs - 1);
+    if (own_weights) {
+      wl = load_ext<D>(own_tables + (size_t)(own_at(jj, false) + (uint32_t)(i & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
+      wh = load_ext<D>(own_tables + (size_t)(own_at(jj, true) + (uint32_t)(i >> args.low_bits[jj])) * D);
+      return;
+    }
     wl = load_ext<D>(args.weights + (args.low_off[jj] + (i & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
     wh = load_ext<D>(args.weights + (args.high_off[jj] + (i >> args.low_bits[jj])) * D);
   };
@@ -1139,7 +1189,8 @@ __device__ __forceinline__ void tail_body(const Desc &d, const TailArgs<D> &args
               lo[t] = load_ext<D>(p);
               hi[t] = load_ext<D>(p + D);
             }
-          if (i >= BLOCK) {  // beyond the prefetched pair
+          if (i >= BLOCK) {  // beyond the prefetched pair (never with the session's own tables: one launch's
+                             // rounds have a pair per thread at most)
             const uint64_t gi = (uint64_t)wg * pairs + i;
             wl = load_ext<D>(args.weights + (args.low_off[jj] + (gi & (((uint64_t)1 << args.low_bits[jj]) - 1))) * D);
             wh = load_ext<D>(args.weights + (args.high_off[jj] + (gi >> args.low_bits[jj])) * D);

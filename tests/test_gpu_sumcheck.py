@@ -322,6 +322,35 @@ def test_base_field_sweep_with_block_weights(K, n, d, with_eq, monkeypatch):
                block_weights=bw)
 
 
+@pytest.mark.parametrize("form,names,cnames,d,n,base", [
+    (CONFIG2, ["t0", "t1", "t2"], ["alpha"], 4, 8, True),
+    (CONFIG2, ["t0", "t1", "t2"], ["alpha"], 4, 3, False),
+    (CONFIG3, ["c0", "c1", "c2", "c3"], [], 8, 6, True),
+    ("(* t0 t1)", ["t0", "t1"], [], 8, 1, False),
+    ("(* t0 t1)", ["t0", "t1"], [], 4, 9, False),
+])
+def test_a_small_session_builds_its_weight_tables_in_its_one_launch(form, names, cnames, d, n, base, monkeypatch):
+    """A proof whose every round fits the one-workgroup launch has no set-up launch: that launch forms the eq
+    weights itself in LDS (the largest such sizes for each table count here, and one round).  Same bytes as the
+    oracle, and as with the set-up launch (EXACTA_HIP_NO_OWN_WEIGHTS=1); the launches differ by that one."""
+    rng = np.random.default_rng(n * 31 + d)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) if base else rand_ext(rng, (1 << n,), d) for _ in names]
+    eq = rand_ext(rng, (n,), d)
+    consts = rand_ext(rng, (len(cnames),), d) if cnames else None
+    st, _, proof, _ = prove_both("own-weights", d, n, form, names, tables, eq=eq, constants=consts, cnames=cnames)
+    dev = [sa.Table.upload(t) for t in tables]
+    counts = []
+    for off in ("0", "1"):
+        monkeypatch.setenv("EXACTA_HIP_NO_OWN_WEIGHTS", off)
+        tr = sa.Transcript("own-weights", d)
+        names_of = launch_names(lambda: sa.prove(tr, n, st, dev, eq=eq, constants=consts))
+        assert tr.proof() == proof
+        counts.append(len(names_of))
+    assert counts[1] == counts[0] + 1
+    for t in dev:
+        t.free()
+
+
 @pytest.mark.parametrize("n", [6, 19])
 def test_host_replay_of_the_device_transcript(n, monkeypatch):
     """By default the host transcript takes the device transcript's final hash state; with EXACTA_HIP_REPLAY=1 it
