@@ -6,12 +6,14 @@ vanish everywhere) and lookups (tag, values, numerator forms).  Its proof is one
 n-1 (oracle gkr_prove_upper), one sumcheck over the halves of the columns that proves the trees' leaf layer and
 the zerocheck (oracle prove), and a fresh point that turns the halves' finals into column claims.
 
-The sumcheck and GKR underneath are pinned by the reference's golden vectors.  For this layer the reference holds
-no bytes (its frozen domain cases need SBCL's PRNG stream): parity of this file is pinned by what the protocol
-fixes -- the verifier accepts the prover's proof, its claims are the columns' multilinear extensions at the claimed
-points, the roots are the sums of the leaf fractions, a broken constraint and every perturbed message are rejected
-(tests/test_oracle_domain.py, after tests/tests.lisp:485-575) -- and by the statement's value at random points
-against the formula in the doc string of domain-statement (src/domain.lisp:95-114).
+The sumcheck underneath is pinned by the reference's golden vectors.  This layer is pinned by the reference's
+frozen domain cases (tests/tests.lisp:587-624, digest at :904): the sixteen proofs of EXPORT-DOMAIN-CASES, made here
+over the reference's own inputs (SBCL's seeded generator restated in tests/golden/sbcl_random.py), with the
+verifier's claims and roots, hash to the SHA-256 the reference holds (tests/test_oracle_frozen_cases.py).  Beside
+that, what the protocol fixes: the verifier accepts the prover's proof, its claims are the columns' multilinear
+extensions at the claimed points, the roots are the sums of the leaf fractions, a broken constraint and every
+perturbed message are rejected (tests/test_oracle_domain.py, after tests/tests.lisp:485-575), and the statement's
+value at random points equals the formula in the doc string of domain-statement (src/domain.lisp:95-114).
 
 Forms are nested lists as in oracle/forms.py: an int, an upper-case name, or [op, arg...].
 """

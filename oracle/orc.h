@@ -19,10 +19,12 @@
  *   sumcheck with base tables / constants     invariants: base == lifted proof bytes, brute-force
  *                                             round sums on tiny n, linearity in the statement,
  *                                             verifier acceptance (no golden bytes exist)
- *   GKR fraction trees, prove-upper           PARITY UNPINNED BY BYTES (the reference's frozen cases need
- *                                             SBCL's PRNG); pinned by root = sum of leaf fractions,
- *                                             claims = MLE of the parents, verifier acceptance,
- *                                             forgery rejection, every layer being a pinned sumcheck
+ *   GKR fraction trees, prove-upper,          the reference's frozen GKR cases (tests/tests.lisp:464-483, digest at
+ *   verify-upper                              :903): the eight proofs of EXPORT-GKR-CASES (one block and several, one to
+ *                                             three lookups, F_p^4 and F_p^8) over the reference's own inputs (SBCL's
+ *                                             seeded generator, tests/golden/sbcl_random.py) with the verifier's outputs
+ *                                             hash to the SHA-256 the reference holds; also root = sum of leaf fractions,
+ *                                             claims = MLE of the parents, forgery rejection
  *   leaf digest, Merkle, cap, BaseFold        PARITY UNPINNED BY BYTES; pinned by the :blake3 vectors for
  *                                             every hash shape used, path checks against the cap,
  *                                             fold(encode(m)) = encode(fold(m)), final table = message

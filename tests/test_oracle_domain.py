@@ -1,5 +1,5 @@
-"""The oracle's domain layer (oracle/domain.py, after src/domain.lisp).  The reference holds no bytes for it (its
-frozen domain proofs need SBCL's PRNG); these tests pin it by what the protocol fixes, following
+"""The oracle's domain layer (oracle/domain.py, after src/domain.lisp).  Its bytes are pinned by the reference's frozen
+domain cases (tests/test_oracle_frozen_cases.py); these tests hold it to what the protocol fixes, following
 tests/tests.lisp:485-575: the toy domain with every kind of column, the verifier accepting the prover's proof with
 the same claims, a full column's claim being its multilinear extension at the claimed point, the roots being the
 sums of the leaf fractions, a broken constraint rejected and every perturbed message rejected."""
