@@ -860,3 +860,20 @@ def pcs_verify_opening(tr, nv, keys, rr, v, grind_bits=4, queries=6):
     rr, v = _u32(rr).reshape(-1, 8), _u32(v)
     _check(lib().orc_pcs_verify_opening(tr.h, nv, len(keys), arr, _p(rr), _p(v), grind_bits, queries), "pcs")
     return True
+
+
+def basefold_classes(tr, nv, classes, rr, v, grind_bits=4, queries=6):
+    """basefold (src/pcs.lisp:581-657) alone over the classes' combined columns: classes = [(c, h (2^c, 8)), ...]
+    in ascending c, the largest being nv.  Returns the query positions."""
+    arr = (OpenKey * len(classes))()
+    keep = []
+    for k, (c, h) in enumerate(classes):
+        h = _u32(h).reshape(-1, 8)
+        assert len(h) == 1 << c
+        keep.append(h)
+        arr[k].c, arr[k].ncols, arr[k].h = c, 0, _p(h)
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    qs = np.zeros(queries, np.uint64)
+    _check(lib().orc_basefold_classes(tr.h, nv, len(classes), arr, _p(rr), _p(v), grind_bits, queries,
+                                      qs.ctypes.data_as(u64p)), "basefold")
+    return [int(q) for q in qs]

@@ -284,6 +284,8 @@ typedef struct {
    sum_c H_c(the last c coordinates of rr) = v */
 int orc_pcs_open(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr, const uint32_t *v,
                  int grind_bits, int queries, uint64_t *out_qs);
+int orc_basefold_classes(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr, const uint32_t *v,
+                 int grind_bits, int queries, uint64_t *out_qs);
 /* BASEFOLD's verifier side and VERIFY-QUERIES; ORC_E_REJECT when a check fails */
 int orc_pcs_verify_opening(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr,
                            const uint32_t *v, int grind_bits, int queries);

@@ -91,8 +91,8 @@ static void add_table(uint32_t *acc, const uint32_t *h, uint64_t len) {
 
 /* BASEFOLD, prover side, src/pcs.lisp:581-657; classes ascending, class c joins at level nv - c; then OPEN-QUERIES
    (:721-734) over the keys, each the last (and only) unit of its set */
-int orc_pcs_open(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr, const uint32_t *v,
-                 int grind_bits, int queries, uint64_t *out_qs) {
+static int open_classes(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr, const uint32_t *v,
+                        int grind_bits, int queries, uint64_t *out_qs, int open_keys) {
   int fl = nv - FLOG > 0 ? nv - FLOG : 0, status = ORC_OK;
   uint64_t len = (uint64_t)1 << nv;
   for (int k = 0; k < nkeys; k++)
@@ -230,7 +230,7 @@ int orc_pcs_open(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const 
     }
   }
   /* OPEN-QUERIES, :721-734: each key's queried leaves, then (it is its set's last) its tree's paths */
-  for (int k = 0; k < nkeys && !status; k++) {
+  for (int k = 0; k < nkeys && !status && open_keys; k++) {
     const orc_open_key *key = &keys[k];
     int c = key->c, depth = orc_cap_level((uint64_t)1 << (c - 1));
     uint64_t *leaves = (uint64_t *)malloc(8 * (size_t)queries);
@@ -257,6 +257,18 @@ done:
   free(cw);
   free(tw);
   return status;
+}
+
+int orc_pcs_open(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr, const uint32_t *v,
+                 int grind_bits, int queries, uint64_t *out_qs) {
+  return open_classes(tr, nv, nkeys, keys, rr, v, grind_bits, queries, out_qs, 1);
+}
+
+/* BASEFOLD alone (src/pcs.lisp:581-657) over the classes' combined columns (a key's c and h; nothing else of it is
+   read): what a caller that opens merged sets and mixed trees itself (tests/golden/pcs_cases.py) builds on */
+int orc_basefold_classes(orc_tr *tr, int nv, int nkeys, const orc_open_key *keys, const uint32_t *rr, const uint32_t *v,
+                         int grind_bits, int queries, uint64_t *out_qs) {
+  return open_classes(tr, nv, nkeys, keys, rr, v, grind_bits, queries, out_qs, 0);
 }
 
 /* BASEFOLD's verifier side and VERIFY-QUERIES (src/pcs.lisp:581-657, 752-843) over the same keys (class, column

@@ -1,7 +1,9 @@
 """The oracle against the reference's frozen cases (tests/tests.lisp:902-925): the SHA-256 of the case files that
-EXPORT-GKR-CASES and EXPORT-DOMAIN-CASES write -- eight PROVE-UPPER proofs (one block and several, one to three
-lookups, F_p^4 and F_p^8) and sixteen PROVE-DOMAIN proofs (every kind of column, merged blocks, with and without
-lookups and constraints), with the verifiers' outputs -- over inputs from SBCL's seeded generator
+EXPORT-GKR-CASES, EXPORT-DOMAIN-CASES and EXPORT-PCS-CASES write -- eight PROVE-UPPER proofs (one block and
+several, one to three lookups, F_p^4 and F_p^8), sixteen PROVE-DOMAIN proofs (every kind of column, merged blocks,
+with and without lookups and constraints) with the verifiers' outputs, and the three commitment proofs (size
+classes 5 to 10, columns split at cmax, merged sets with mixed-height trees, a segment, point reductions in batches,
+BaseFold with one and two oracle levels, grinding, six queries) -- over inputs from SBCL's seeded generator
 (tests/golden/sbcl_random.py).  A digest matches only if the generator, the inputs, every message of every proof,
 the verifier's claims and the proof encoding are the reference's, byte for byte."""
 import hashlib
@@ -51,3 +53,12 @@ def test_prove_domain_makes_the_frozen_domain_cases():
 
     text = fc.domain_cases_text(od.Domain, od.Column, prove, verify)
     assert hashlib.sha256(text.encode()).hexdigest() == fc.DOMAIN_SHA256
+
+
+def test_the_commitment_makes_the_frozen_pcs_cases():
+    """The reference's commitment scheduler (src/pcs.lisp, prover side) restated over the oracle's primitives in
+    tests/golden/pcs_cases.py: RS encoding, leaf digests chained over merged units, Merkle levels with injections and
+    caps, the point reductions' sumchecks, combine-columns, the cross-unit sumcheck's dot-pairs / fold-table /
+    lagrange, BaseFold over classes, grinding and the query openings."""
+    import pcs_cases as pc
+    assert hashlib.sha256(pc.pcs_cases_text().encode()).hexdigest() == pc.PCS_SHA256
