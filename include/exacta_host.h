@@ -113,6 +113,13 @@ int exh_basefold_prove(exh_transcript tr, int nv, const uint32_t *rr, const uint
 int exh_basefold_prove_encoded(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, exh_table h,
                                exh_table codeword, int grind_bits, int queries, uint64_t *out_qs,
                                uint32_t *out_challenges, uint32_t *out_final);
+/* BASEFOLD over several size classes (src/pcs.lisp:581-657 with its CLASSES and H arguments as PCS-FINISH passes
+   them, :714-716): classes[k] ascending, the last one nv; hs[k] the class's combined column H_c, 2^classes[k]
+   EXT8s on the device, joining at level nv - classes[k] (:590-600, :635-639).  The oracle openings are recorded
+   on the transcript as BASEFOLD does; the query openings of the committed trees (OPEN-QUERIES, :721-734) stay with
+   the caller, who knows its merge sets. */
+int exh_basefold_prove_classes(exh_transcript tr, int nv, int n_classes, const int *classes, const exh_table *hs,
+                               const uint32_t *rr, const uint32_t *v, int grind_bits, int queries, uint64_t *out_qs);
 int exh_basefold_verify(exh_transcript tr, int nv, const uint32_t *rr, const uint32_t *v, int grind_bits,
                         int queries, uint64_t *out_qs);
 

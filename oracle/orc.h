@@ -25,15 +25,19 @@
  *                                             seeded generator, tests/golden/sbcl_random.py) with the verifier's outputs
  *                                             hash to the SHA-256 the reference holds; also root = sum of leaf fractions,
  *                                             claims = MLE of the parents, forgery rejection
- *   leaf digest, Merkle, cap, BaseFold        PARITY UNPINNED BY BYTES; pinned by the :blake3 vectors for
- *                                             every hash shape used, path checks against the cap,
- *                                             fold(encode(m)) = encode(fold(m)), final table = message
- *                                             folded at the challenges
+ *   leaf digest, Merkle (with injections),    the reference's frozen commitment cases (tests/tests.lisp:728-758, digest at
+ *   cap, combine-columns, dot-pairs,          :905): the reference's scheduler restated over these primitives
+ *   fold-table, BaseFold over classes         (tests/golden/pcs_cases.py: units, merge sets, mixed trees, point
+ *                                             reductions, segment, finish, query openings) makes the three proofs of
+ *                                             EXPORT-PCS-CASES byte for byte; also the :blake3 vectors for every hash
+ *                                             shape used, path checks against the cap, fold(encode(m)) =
+ *                                             encode(fold(m)), final table = message folded at the challenges
  *   dot-pairs, fold-table, scale-add          their definitions in an independent pure-Python field on small tables;
  *                                             the round identity g(0) + g(1) of the folded tables = g(x)
  *   open-queries (leaves, paths)              numpy indexing of the codewords by the definition; every opened leaf,
  *                                             hashed and walked up its path, lands on the committed cap
- *   opening over several classes, verify-      PARITY UNPINNED BY BYTES; prover -> verifier acceptance, rejection of every
+ *   opening over several classes, verify-      its BaseFold and trees by the frozen cases above; its own query openings
+ *   queries, mixed-height Merkle trees        and the verifier by: prover -> verifier acceptance, rejection of every
  *   queries, mixed-height Merkle trees        flipped opened symbol / path / cap / final-table word, the single-class case
  *                                             being orc_basefold_prove byte for byte, injected levels against a
  *                                             definition-level Python tree

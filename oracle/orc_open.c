@@ -7,7 +7,10 @@
  * with the coefficients the caller gives (UC-COEF).  Merge sets, segments and the cross-unit sumcheck are not
  * restated.
  *
- * PARITY UNPINNED BY BYTES (the reference's frozen cases need SBCL's PRNG); pinned by: prover -> verifier
+ * Pinned by the reference's frozen commitment cases (tests/tests.lisp:728-758, digest at :905): under the reference's
+ * scheduler restated in tests/golden/pcs_cases.py, orc_basefold_classes and the Merkle levels with injections
+ * produce the three proofs of EXPORT-PCS-CASES byte for byte (tests/test_oracle_frozen_cases.py).  orc_pcs_open's
+ * own query openings (one tree per key) and the verifier's side are held to: prover -> verifier
  * acceptance; rejection of every flipped opened symbol, path byte, cap byte and final-table entry; each opened
  * leaf hashing up its path to the committed cap; fold(encode(m)) = encode(fold(m)) through the oracles down to
  * the final table's codeword, which is what VERIFY-QUERIES itself recomputes; the single-class case being

@@ -549,6 +549,17 @@ def basefold_prove(tr, nv, rr, v, h, grind_bits=4, queries=6, codeword=None):
     return [int(q) for q in qs], chal[:fl], final
 
 
+def basefold_prove_classes(tr, nv, classes, rr, v, grind_bits=4, queries=6):
+    """basefold over size classes: classes = [(c, Table of 2^c EXT8s), ...] ascending, the last c = nv."""
+    rr, v = _u32(rr).reshape(-1, 8), _u32(v)
+    cs = (C.c_int * len(classes))(*[c for c, _ in classes])
+    hs = (C.c_uint64 * len(classes))(*[t.handle for _, t in classes])
+    qs = np.zeros(queries, np.uint64)
+    check(load().exh_basefold_prove_classes(tr.h, nv, len(classes), cs, hs, _p(rr), _p(v), grind_bits, queries,
+                                            qs.ctypes.data_as(u64p)))
+    return [int(q) for q in qs]
+
+
 def basefold_verify(tr, nv, rr, v, grind_bits=4, queries=6):
     rr, v = _u32(rr).reshape(-1, 8), _u32(v)
     qs = np.zeros(queries, np.uint64)

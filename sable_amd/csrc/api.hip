@@ -1127,6 +1127,26 @@ int exh_basefold_prove(exh_transcript h, int nv, const uint32_t *rr, const uint3
   }
   return basefold_prove(*tr, nv, rr, v, dt->ptr, grind_bits, queries, out_qs, out_chal, out_final);
 }
+int exh_basefold_prove_classes(exh_transcript h, int nv, int n_classes, const int *classes, const exh_table *hs,
+                               const uint32_t *rr, const uint32_t *v, int grind_bits, int queries, uint64_t *out_qs) {
+  ApiLock api_lock;
+  Transcript *tr = tr_of(h);
+  if (!tr || n_classes < 1 || n_classes > 32 || !classes || !hs || nv < 1 || nv > 23) {
+    set_error("invalid-parameter: BaseFold over 1 to 32 classes, 1 <= nv <= 23");
+    return E_PARAM;
+  }
+  std::vector<const uint32_t *> tables(n_classes);
+  for (int k = 0; k < n_classes; k++) {
+    DeviceTable *dt = table_of(hs[k]);
+    if (!dt || classes[k] < 1 || classes[k] > nv || dt->stride != 8 || dt->n_u32 != ((uint64_t)8 << classes[k])) {
+      set_error("invalid-parameter: a class's combined column is 2^c EXT8s");
+      return E_PARAM;
+    }
+    tables[k] = dt->ptr;
+  }
+  return basefold_prove_classes(*tr, nv, n_classes, classes, tables.data(), rr, v, grind_bits, queries, out_qs, nullptr,
+                                nullptr, nullptr);
+}
 int exh_basefold_prove_encoded(exh_transcript h, int nv, const uint32_t *rr, const uint32_t *v, exh_table table,
                                exh_table codeword, int grind_bits, int queries, uint64_t *out_qs, uint32_t *out_chal,
                                uint32_t *out_final) {

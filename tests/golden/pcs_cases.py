@@ -48,6 +48,56 @@ def ext_sum(items, d):
     return acc
 
 
+class OracleBackend:
+    """The primitives the scheduler stands on, over host arrays: the oracle's here; tests/test_gpu_frozen_cases.py
+    has the device's behind the same names.  (The arithmetic on single field elements around them -- claims,
+    Lagrange interpolation of three values, eq of two points -- is the oracle's in both.)"""
+    def transcript(self, label, d):
+        return orc.Transcript(label, d)
+
+    def encode(self, columns, c):
+        return [orc.rs_encode(column, c + 1) for column in columns]
+
+    def leaf_digests(self, codewords, c, previous):
+        digests = np.zeros((1 << (c - 1), 32), np.uint8)
+        for l in range(1 << (c - 1)):
+            rows = np.array([cw[4 * l:4 * l + 4] for cw in codewords], np.uint32)
+            digests[l] = np.frombuffer(orc.leaf_digest(rows, None if previous is None else bytes(previous[l])), np.uint8)
+        return digests
+
+    def merkle_levels(self, leaves, injections):
+        return orc.merkle_levels_injected(leaves, injections)
+
+    def prove_reduction(self, tr, c, form, names, tables):
+        rho, _, _ = orc.prove(tr, c, orc.Statement(form, names), tables, label="pcs-red", degree=2)
+        return [r for r in rho]
+
+    def mle_eval(self, table, point, d):
+        return orc.mle_eval(table, np.array(point), d)
+
+    def combine_columns(self, columns, coefficients):
+        return orc.combine_columns(np.array(columns), coefficients)
+
+    def eq_table(self, point, d):
+        return orc.eq_table(np.array(point), d)
+
+    def scale_add(self, h, scale, column):
+        column = np.asarray(column, np.uint32)
+        return orc.scale_add(np.zeros_like(column) if h is None else h, scale, column)
+
+    def dot_pairs(self, e, v):
+        return orc.dot_pairs(e, v)
+
+    def fold_table(self, table, x):
+        return orc.fold_table(table, x)
+
+    def basefold_classes(self, tr, nv, classes, rr, v, grind_bits, queries):
+        return orc.basefold_classes(tr, nv, classes, rr, v, grind_bits=grind_bits, queries=queries)
+
+    def gather_leaves(self, codewords, c, leaves):
+        return np.array([[cw[4 * l:4 * l + 4] for cw in codewords] for l in leaves], np.uint32)
+
+
 # ------------------------------------------------------------------ inputs (tests/tests.lisp:647-668)
 def pcs_data(units, state):
     return {tensor: np.array([state.random(P) for _ in range(k << c0)], np.uint32)
@@ -155,8 +205,9 @@ class Pu:
 
 
 class Pcs:
-    def __init__(self, tr, cmax, queries, grind, max_points=64):
+    def __init__(self, tr, cmax, queries, grind, max_points=64, backend=None):
         self.tr, self.cmax, self.queries, self.grind, self.max_reduction_points = tr, cmax, queries, grind, max_points
+        self.b = backend or OracleBackend()
         self.units, self.order, self.ucs = {}, [], {}
         self.msets, self.mset_of, self.seg_decl, self.seg_of, self.segs = [], {}, [], {}, []
         self.states, self.codewords, self.trees = {}, {}, {}
@@ -204,23 +255,18 @@ class Pcs:
 
     def tree_levels(self, tid):
         if tid[0] == "single":
-            return orc.merkle_levels_injected(self.states[(tid[1], tid[2])], {})
+            return self.b.merkle_levels(self.states[(tid[1], tid[2])], {})
         sid = tid[1]
         cm, mixed = self.set_mixed(sid)
-        return orc.merkle_levels_injected(self.states[(sid, cm)], {cm - c: self.states[(sid, c)] for c in mixed if c != cm})
+        return self.b.merkle_levels(self.states[(sid, cm)], {cm - c: self.states[(sid, c)] for c in mixed if c != cm})
 
     def commit(self, name, tensors):
         unit, sid = self.units[name], self.set_id(name)
         unit.tensors = tensors
         for c, _ in unit.classes:
-            codewords = [orc.rs_encode(column, c + 1) for column in unit.columns(c, self.cmax)]
-            previous = self.states.get((sid, c))
+            codewords = self.b.encode(unit.columns(c, self.cmax), c)
             self.codewords[(name, c)] = codewords
-            digests = np.zeros((1 << (c - 1), 32), np.uint8)
-            for l in range(1 << (c - 1)):
-                rows = np.array([cw[4 * l:4 * l + 4] for cw in codewords], np.uint32)
-                digests[l] = np.frombuffer(orc.leaf_digest(rows, None if previous is None else bytes(previous[l])), np.uint8)
-            self.states[(sid, c)] = digests
+            self.states[(sid, c)] = self.b.leaf_digests(codewords, c, self.states.get((sid, c)))
         if name == self.set_members(sid)[-1]:
             for tid in self.set_trees(sid):
                 levels = self.tree_levels(tid)
@@ -245,15 +291,12 @@ class Pcs:
             combined.append((z, comb))
         names, tables = [], []
         for i, (z, comb) in enumerate(combined):
-            g = np.zeros((1 << c, 4), np.uint64)
-            for k, cf in comb:  # ext-scale cf (aref column x): coordinate-wise
-                g = (g + columns[k].astype(np.uint64)[:, None] * cf.astype(np.uint64)[None, :] % P) % P
+            # g[x] = sum_k (ext-scale cf (aref column_k x)): combine-columns at F_p^4
+            g = self.b.combine_columns([columns[k] for k, _ in comb], np.array([cf for _, cf in comb], np.uint32))
             names += ["E%d" % i, "G%d" % i]
-            tables += [orc.eq_table(np.array(z), 4), g.astype(np.uint32)]
+            tables += [self.b.eq_table(z, 4), g]
         form = "(+ " + " ".join("(* E%d G%d)" % (i, i) for i in range(len(combined))) + ")"
-        st = orc.Statement(form, names)
-        rho, _, _ = orc.prove(self.tr, c, st, tables, label="pcs-red", degree=2)
-        return [r for r in rho]
+        return self.b.prove_reduction(self.tr, c, form, names, tables)
 
     def max_points(self, c):
         return max(2, min(self.max_reduction_points, (8 << 30) // (2 * (1 << c) * 4 * 4)))
@@ -268,7 +311,7 @@ class Pcs:
             groups = by_point(by_class.get(c, []))
 
             def receive(keys, rho):
-                values = [(k, orc.mle_eval(columns[k], np.array(rho), 4)) for k in keys]
+                values = [(k, self.b.mle_eval(columns[k], rho, 4)) for k in keys]
                 self.tr.send(np.array([v for _, v in values], np.uint32).reshape(len(keys), 4))
                 return values
 
@@ -286,7 +329,7 @@ class Pcs:
             alpha = self.tr.challenges(ncols, 8)
             y = ext_sum([orc.ext_mul(a, embed(v)) for a, (_, v) in zip(alpha, values)], 8)
             uc = Uc(unit, c, rho, alpha, y, ncols)
-            uc.column = orc.combine_columns(np.array(columns), alpha)
+            uc.column = self.b.combine_columns(columns, alpha)
             self.ucs[(name, c)] = uc
 
     # -------------------------------------------------------------- the cross-unit sumcheck (src/pcs.lisp:445-516)
@@ -298,8 +341,8 @@ class Pcs:
         for c in sorted({u.c for u in us}):
             members = [u for u in us if u.c == c]
             const = ext_sum([self.lam_scaled(u.lam, u.y, c, nv) for u in members], 8)
-            e = np.concatenate([np.array([orc.ext_mul(x, u.lam) for x in orc.eq_table(np.array([embed(x) for x in u.rho]), 8)])
-                                for u in members])
+            # (e * lambda per entry of eq-table: lambda times the table)
+            e = np.concatenate([self.b.scale_add(None, u.lam, self.b.eq_table([embed(x) for x in u.rho], 8)) for u in members])
             v = np.concatenate([np.asarray(u.column, np.uint32).reshape(-1, 8) for u in members])
             states.append({"c": c, "const": const, "e": e, "v": v})
         return states
@@ -312,7 +355,7 @@ class Pcs:
                 if j < nv - s["c"]:
                     ev = [orc.ext_add(e, orc.ext_scale(s["const"], inverse_2)) for e in ev]
                 else:
-                    dp = orc.dot_pairs(s["e"], s["v"])
+                    dp = self.b.dot_pairs(s["e"], s["v"])
                     ev = [orc.ext_add(e, dp[parity]) for parity, e in enumerate(ev)]
             self.tr.send(np.array(ev, np.uint32))
             assert np.array_equal(orc.ext_add(ev[0], ev[1]), claim), "cross-unit sumcheck round %d" % j
@@ -323,7 +366,7 @@ class Pcs:
                 if j < nv - s["c"]:
                     s["const"] = orc.ext_scale(s["const"], inverse_2)
                 else:
-                    s["e"], s["v"] = orc.fold_table(s["e"], x), orc.fold_table(s["v"], x)
+                    s["e"], s["v"] = self.b.fold_table(s["e"], x), self.b.fold_table(s["v"], x)
         return r, claim
 
     def segment(self, i):
@@ -339,17 +382,17 @@ class Pcs:
         r, claim = self.cross_rounds(states, nv, claim)
         coefficients = [orc.ext_mul(u.lam, orc.ext_eq(np.array([embed(x) for x in u.rho]), np.array(r[nv - u.c:]), 8))
                         for u in ucs]
-        ys = [ext_sum([orc.ext_mul(e, orc.mle_eval(u.column, np.array(r[nv - c:]), 8))
+        ys = [ext_sum([orc.ext_mul(e, self.b.mle_eval(u.column, r[nv - c:], 8))
                        for u, e in zip(ucs, coefficients) if u.c == c], 8) for c in classes]
         self.tr.send(np.array(ys, np.uint32).reshape(len(classes), 8))
         assert np.array_equal(ext_sum(ys, 8), claim), "segment reduction"
         pus = []
         for c, y in zip(classes, ys):
             pu = Pu(c, r[nv - c:], y)
-            h = np.zeros((1 << c, 8), np.uint32)
+            h = None
             for u, e in zip(ucs, coefficients):
                 if u.c == c:
-                    h = orc.scale_add(h, e, u.column)
+                    h = self.b.scale_add(h, e, u.column)
             pu.column = h
             pus.append(pu)
         self.segs.append({"keys": keys, "coefficients": dict(zip(keys, coefficients)), "pus": pus})
@@ -370,12 +413,12 @@ class Pcs:
             u.sc = orc.ext_mul(u.lam, orc.ext_eq(np.array([embed(x) for x in u.rho]), np.array(rr[nv - u.c:]), 8))
         h = []
         for c in classes:
-            hc = np.zeros((1 << c, 8), np.uint32)
+            hc = None
             for u in members:
                 if u.c == c:
-                    hc = orc.scale_add(hc, u.sc, u.column)
+                    hc = self.b.scale_add(hc, u.sc, u.column)
             h.append((c, hc))
-        qs = orc.basefold_classes(self.tr, nv, h, np.array(rr), v, grind_bits=self.grind, queries=self.queries)
+        qs = self.b.basefold_classes(self.tr, nv, h, np.array(rr), v, self.grind, self.queries)
         self.open_queries(keys, qs, nv)
 
     def open_queries(self, keys, qs, nv):
@@ -384,8 +427,7 @@ class Pcs:
             last[self.set_id(k[0])] = k
         for name, c in keys:
             codewords = self.codewords[(name, c)]
-            leaves = np.array([[cw[4 * (q >> (nv - c)):4 * (q >> (nv - c)) + 4] for cw in codewords] for q in qs], np.uint32)
-            self.tr.record(leaves)
+            self.tr.record(self.b.gather_leaves(codewords, c, [q >> (nv - c) for q in qs]))
             if last[self.set_id(name)] == (name, c):
                 for tid in self.set_trees(self.set_id(name)):
                     tc, levels = self.tree_class(tid), self.trees[tid]
@@ -399,13 +441,14 @@ class Pcs:
                     self.tr.record_bytes(octets)
 
 
-def pcs_proof(scenario):
+def pcs_proof(scenario, backend=None):
     """PCS-PROOF (tests/tests.lisp:688-696): the claims and the proof bytes."""
+    backend = backend or OracleBackend()
     state = SbclRandom(scenario["seed"])
     data = pcs_data(scenario["units"], state)
     claims = pcs_claims(scenario["units"], data, state)
-    tr = orc.Transcript("pcs-test", 4)
-    pcs = Pcs(tr, scenario["cmax"], 6, 4, scenario.get("max_points", 64))
+    tr = backend.transcript("pcs-test", 4)
+    pcs = Pcs(tr, scenario["cmax"], 6, 4, scenario.get("max_points", 64), backend)
     for name, items in scenario["units"]:
         pcs.declare(name, items)
     if scenario["merge"]:
@@ -430,11 +473,11 @@ def _exts(es):
     return "[" + ",".join(_ints(e) for e in es) + "]"
 
 
-def pcs_cases_text():
+def pcs_cases_text(backend=None):
     """EXPORT-PCS-CASES (tests/tests.lisp:728-758)."""
     out = ["[\n"]
     for i, sc in enumerate(SCENARIOS):
-        claims, proof = pcs_proof(sc)
+        claims, proof = pcs_proof(sc, backend)
         units = ",".join('{"name": "%s", "items": [%s]}' % (name, ",".join('["%s", %d, %d]' % item for item in items))
                          for name, items in sc["units"])
         claimed = ",".join('{"unit": "%s", "claims": [%s]}' % (name, ",".join(

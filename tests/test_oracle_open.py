@@ -1,7 +1,8 @@
 """The oracle's final opening over several size classes (oracle/orc_open.c): BaseFold with classes joining at later
 levels, open-queries, verify-queries and Merkle trees of mixed height (src/pcs.lisp:64-95, 581-657, 721-843).
-No golden bytes exist for these (the reference's frozen cases need SBCL's PRNG); they are pinned by what the
-protocol itself fixes: the verifier accepts the prover's proof, rejects every perturbed opening, and the
+Its BaseFold over classes and its trees with injections are pinned by the reference's frozen commitment cases
+(tests/test_oracle_frozen_cases.py); the opening as a whole and the verifier are held here to what the protocol
+itself fixes: the verifier accepts the prover's proof, rejects every perturbed opening, and the
 single-class case is the one-class prover byte for byte."""
 import numpy as np
 import pytest
