@@ -170,6 +170,21 @@ def test_statement_compile_matches_expand():
         assert sa.check_final(ost.evaluate(tv, cv, 8), st, tv, constants=cv if cnames else None)
 
 
+def test_gkr_layer_statements_have_build_time_kernels():
+    """LAYER-STATEMENT (src/gkr.lisp:30-41) for one to three lookups, and (* bw statement) for the sumcheck over the
+    block index, as the library forms them: each has kernels generated at build time for F_p^4 (a statement without
+    them runs on the interpreter kernels, several times slower)."""
+    for lookups in (1, 2, 3):
+        tables, constants, terms = [], [], []
+        for l in range(lookups):
+            tables += ["P0-%d" % l, "P1-%d" % l, "Q0-%d" % l, "Q1-%d" % l]
+            constants += ["A%d" % l, "AL%d" % l]
+            terms += ["(* A%d P0-%d Q1-%d)" % (l, l, l), "(* A%d P1-%d Q0-%d)" % (l, l, l), "(* AL%d Q0-%d Q1-%d)" % (l, l, l)]
+        form = "(+ " + " ".join(terms) + ")"
+        assert sa.Statement(form, tables, constants).has_generated_kernel(4), lookups
+        assert sa.Statement("(* BW " + form + ")", ["BW"] + tables, constants).has_generated_kernel(4), lookups
+
+
 def test_the_bench_constants_go_with_the_present_kernel_sources():
     """bench.py reports measured traffic and multiply counts only for the version of the kernels they were measured
     on: the stamp has to be renewed (with the figures) when the kernels' sources change."""
