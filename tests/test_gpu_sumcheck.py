@@ -351,6 +351,22 @@ def test_a_small_session_builds_its_weight_tables_in_its_one_launch(form, names,
         t.free()
 
 
+@pytest.mark.parametrize("points,n", [(2, 7), (2, 15), (3, 14), (4, 13), (4, 19)])
+def test_point_reductions_of_an_opening(points, n):
+    """REDUCE-POINTS' sumcheck (src/pcs.lisp:333-373): sum_z eq(z, x) g_z(x) over extension tables, no eq weights,
+    wire degree 2, label "pcs-red" -- on the kernels generated for two to four points, from one workgroup's sizes
+    to streaming rounds."""
+    d = 4
+    rng = np.random.default_rng(points * 100 + n)
+    names = [v for i in range(points) for v in ("E%d" % i, "G%d" % i)]
+    form = "(+ " + " ".join("(* E%d G%d)" % (i, i) for i in range(points)) + ")"
+    tables = []
+    for i in range(points):
+        tables += [orc.eq_table(rand_ext(rng, (n,), d), d), rand_ext(rng, (1 << n,), d)]
+    st, _, _, _ = prove_both("pcs-test", d, n, form, names, tables, degree=2, sc_label="pcs-red")
+    assert st.has_generated_kernel(d)
+
+
 @pytest.mark.parametrize("n", [6, 19])
 def test_host_replay_of_the_device_transcript(n, monkeypatch):
     """By default the host transcript takes the device transcript's final hash state; with EXACTA_HIP_REPLAY=1 it

@@ -185,6 +185,14 @@ def test_gkr_layer_statements_have_build_time_kernels():
         assert sa.Statement("(* BW " + form + ")", ["BW"] + tables, constants).has_generated_kernel(4), lookups
 
 
+def test_point_reduction_statements_have_build_time_kernels():
+    """REDUCE-POINTS' statement (src/pcs.lisp:344-347) for one to four points, as an opening forms it."""
+    for points in (1, 2, 3, 4):
+        names = [n for i in range(points) for n in ("E%d" % i, "G%d" % i)]
+        form = "(+ " + " ".join("(* E%d G%d)" % (i, i) for i in range(points)) + ")"
+        assert sa.Statement(form, names).has_generated_kernel(4), points
+
+
 def test_the_bench_constants_go_with_the_present_kernel_sources():
     """bench.py reports measured traffic and multiply counts only for the version of the kernels they were measured
     on: the stamp has to be renewed (with the figures) when the kernels' sources change."""
