@@ -296,6 +296,32 @@ def run_gkr(sa, steps, warmup, gold):
             "roofline_by_time": by_time(by)[:8]}
 
 
+def run_gkr_shapes(sa, steps, warmup):
+    """PROVE-UPPER at the shapes a domain gives it (src/domain.lisp:346-349): several lookups proved together and
+    several blocks (block weights, a sumcheck over the block index after every layer), trees of 2^14 leaves per block
+    and lookup.  Each proof is checked by the library's verifier."""
+    d, n, out = 4, 14, {}
+    for name, k, lookups in (("one_block_three_lookups", 1, 3), ("three_blocks_one_lookup", 3, 1),
+                             ("three_blocks_two_lookups", 3, 2)):
+        dev = [(sa.Table.random(700 + 2 * l, k << n, d), sa.Table.random(701 + 2 * l, k << n, d))
+               for l in range(lookups)]
+
+        def step():
+            tr = sa.Transcript("gkr-shapes", d)
+            return tr, sa.prove_upper(tr, n, k, dev)
+
+        dt, (tr, proved) = timed(sa, step, steps, warmup)
+        vtr = sa.Transcript("gkr-shapes", d, proof=tr.proof())
+        _, ri, rb, cp, cq = sa.verify_upper(vtr, n, k, lookups)
+        if not (vtr.finished() and all(np.array_equal(a, b) for a, b in zip((ri, rb, cp, cq), proved))):
+            sys.exit("bench.py: the library's verifier does not agree with the proved claims (%s)" % name)
+        for p, q in dev:
+            p.free(), q.free()
+        out[name] = {"n": n, "blocks": k, "lookups": lookups, "ms_per_step": 1e3 * dt,
+                     "ms_per_layer": 1e3 * dt / (n - 1), "verifier_accepts": True}
+    return out
+
+
 # ------------------------------------------------------------------ config 5: commitment
 def run_commit(sa, steps, warmup, gold):
     cm = wl.COMMIT
@@ -642,6 +668,7 @@ def main():
         others["config4"] = {key: r[key] for key in ("workload", "ms_per_step", "ms_per_step_one_after_the_other",
                                                      "lookups_per_s", "proof_sha256", "proof_is_the_cpu_oracles",
                                                      "timed_launches_per_step", "roofline")}
+        others["config4"]["domain_shapes"] = run_gkr_shapes(sa, k, 2)
         r = run_commit(sa, k, 2, gold)
         others["config5"] = {key: r[key] for key in ("workload", "ms_per_step", "cap_sha256", "cap_is_the_cpu_oracles",
                                                      "roofline")}
