@@ -1051,17 +1051,26 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     // once every workgroup of a resident grid can hold its slice of the tables in LDS, the rounds down
     // to where one workgroup suffices run in one launch
     const bool pow2 = (size & (size - 1)) == 0;
+    // (several blocks: the pairs are an odd multiple of a power of two, and the grid that multiple of one, so that
+    // every workgroup's slice is a power of two of pairs and halves with the rounds; a fold pairs neighbours, so a
+    // slice need not lie in one block)
+    uint64_t odd = n_pairs;
+    while (odd > 1 && odd % 2 == 0) odd /= 2;
     uint64_t slice_max = SLICE_LDS_BYTES / ((uint64_t)T * 2 * D * 4);
     if (const char *cap = getenv("EXACTA_HIP_MAX_SLICE_PAIRS"))  // tests: keep more rounds on the streaming kernels
       slice_max = std::min<uint64_t>(slice_max, strtoull(cap, nullptr, 10));
     // (proofs running side by side share the device: each one's grid takes its part, a power of two)
     const uint64_t grid_max =
         std::min<uint64_t>(256, c.compute_units > 0 ? c.compute_units : 1) / (c.share > 1 ? 2 : 1);
-    if (pow2 && n_pairs > tail_pairs(T, D) && n_pairs <= slice_max * grid_max) {
+    if (odd > 1) {  // (EXACTA_HIP_NO_BLOCK_SLICES=1: tables of several blocks stay on the streaming kernels)
+      const char *no_block_slices = getenv("EXACTA_HIP_NO_BLOCK_SLICES");
+      if (no_block_slices && no_block_slices[0] == '1') odd = 17;
+    }
+    if (odd <= 16 && odd <= grid_max && n_pairs > tail_pairs(T, D) && n_pairs <= slice_max * grid_max) {
       int count = 0;
       while ((n_pairs >> count) > tail_pairs(T, D) && count < MAXTAIL && j + count < n) count++;
       const uint64_t left = 2 * (n_pairs >> count);  // entries per table after these rounds
-      uint64_t grid = 1;
+      uint64_t grid = odd;
       while (grid * 2 <= grid_max && grid * 2 <= left && (n_pairs / (grid * 2)) >= BLOCK) grid *= 2;
       while (n_pairs / grid > slice_max && grid * 2 <= grid_max && grid * 2 <= left) grid *= 2;
       // the grid's workgroups wait for one another: all of them must be resident at once.  The runtime says how
@@ -1216,7 +1225,7 @@ int SumcheckSession::launch_tail(int j, int rounds, uint32_t grid, bool first_fo
   // groups of workgroups share a row of totals: few enough that a workgroup polls all the rows' words at
   // once, one per thread (a second pass of polls is a second trip to memory in every round)
   uint32_t groups = 1;
-  while (groups * 2 <= SLICE_GROUPS && groups * 2 <= grid && groups * 2 * (uint32_t)st.nacc * D <= BLOCK) groups *= 2;
+  while (groups * 2 <= SLICE_GROUPS && grid % (groups * 2) == 0 && groups * 2 * (uint32_t)st.nacc * D <= BLOCK) groups *= 2;
   auto fill = [&](auto &a) {
     memset(&a, 0, sizeof(a));
     for (int t = 0; t < T; t++) a.in[t] = cur[t];

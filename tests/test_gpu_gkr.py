@@ -75,6 +75,26 @@ def test_prove_upper_matches_the_oracle(n, k, lookups, d):
         p.free(), q.free()
 
 
+@pytest.mark.parametrize("n,k,lookups,d", [(12, 3, 1, 4), (11, 5, 2, 4), (10, 3, 3, 4), (10, 6, 1, 8), (9, 12, 1, 4)])
+def test_several_blocks_on_the_grid_of_slices_and_on_the_streaming_rounds(n, k, lookups, d, monkeypatch):
+    """Tables of K 2^m entries (K not a power of two) take the grid of LDS-resident slices with a multiple of K's odd
+    part of workgroups; with the switch they stay on the streaming rounds.  Both are the oracle's proof."""
+    rng = np.random.default_rng(7 * n + k)
+    leaves = random_leaves(rng, lookups, n, k, d)
+    dev = [(sa.Table.upload(p), sa.Table.upload(q)) for p, q in leaves]
+    otr = orc.Transcript("gkr-blocks", d)
+    want = orc.gkr_prove_upper(otr, n, k, leaves)
+    for off in ("0", "1"):
+        monkeypatch.setenv("EXACTA_HIP_NO_BLOCK_SLICES", off)
+        tr = sa.Transcript("gkr-blocks", d)
+        got = sa.prove_upper(tr, n, k, dev)
+        assert tr.proof() == otr.proof(), off
+        for a, b in zip(got, want):
+            assert same(a, b)
+    for p, q in dev:
+        p.free(), q.free()
+
+
 @pytest.mark.parametrize("n,lookups,d", [(9, 1, 4), (6, 2, 4), (8, 1, 8), (7, 3, 4)])
 def test_the_chained_layers_and_the_host_driven_layers_send_the_same_bytes(n, lookups, d, monkeypatch):
     rng = np.random.default_rng(100 + n)
