@@ -196,6 +196,8 @@ struct DeviceBuffers {  // frees what it allocated when the proof ends
 };
 
 
+constexpr size_t GKR_BW_PIN = 8192, GKR_BW_PIN_WORDS = 1024;  // words of the context's pinned buffer (see below)
+
 // what the chain's sticky word means for the proof (host side)
 int chain_outcome(uint32_t failed) {
   if (!failed) return OK;
@@ -583,8 +585,16 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
       std::vector<const uint32_t *> btabs(NT + 1);
       std::vector<uint32_t> bwp(Kp * D, 0);
       memcpy(bwp.data(), bw.data(), (size_t)K * D * 4);
-      EXH_HIP(hipMemcpyAsync(d_blk, bwp.data(), Kp * D * 4, hipMemcpyHostToDevice, c.stream));
       for (int t = 0; t <= NT; t++) btabs[t] = d_blk + (uint64_t)t * Kp * D;
+      // the weights' table: read by the sumcheck's first launch from pinned memory where the host puts it (a part
+      // of the context's buffer nothing else uses; the host waits for this sumcheck before it writes there again),
+      // or copied beside the blocks' values when it is longer than that part
+      if (Kp * D <= GKR_BW_PIN_WORDS && c.host_pinned_dev) {
+        memcpy(c.host_pinned + GKR_BW_PIN, bwp.data(), Kp * D * 4);
+        btabs[0] = c.host_pinned_dev + GKR_BW_PIN;
+      } else {
+        EXH_HIP(hipMemcpy(d_blk, bwp.data(), Kp * D * 4, hipMemcpyHostToDevice));
+      }
       std::vector<uint32_t> f2((size_t)(NT + 1) * D);
       rbn.assign((size_t)lk * D, 0);
       status = sumcheck_prove(tr, lk, st_blk, btabs.data(), strides.data(), nullptr, consts.data(), label + "-blk",

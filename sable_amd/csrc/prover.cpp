@@ -185,6 +185,10 @@ int sumcheck_prove(Transcript &tr, int n, const Statement &st, const uint32_t *c
     // transcripts are the same function, and the tests hold the device's to the oracle's bytes)
     DevB3S state = device_state(tr), final_state;
     std::vector<uint32_t> messages((size_t)n * points * D), challenges((size_t)n * D);
+    {  // (EXACTA_HIP_FETCH_FINALS=1: fetch the folded tables with the logs all the same)
+      const char *fetch = getenv("EXACTA_HIP_FETCH_FINALS");
+      s.finals_stay = d_folded && !out_finals && !out_folded && !(fetch && fetch[0] == '1');
+    }
     if ((status = s.run_device(state, messages.data(), challenges.data(), &final_state))) return status;
     const char *replay = getenv("EXACTA_HIP_REPLAY");
     const bool replaying = replay && replay[0] == '1';

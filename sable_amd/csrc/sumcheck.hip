@@ -28,12 +28,21 @@ struct EqTables {
 
 // (both set-up kernels also clear the totals of the grid launch of LDS-resident slices: the first launch of a
 // session is the one place that comes before every use)
+// `staged` (null: none): the session's constants as the host staged them in pinned memory, `staged_words` of them,
+// factors first; the launch brings them to `staged_dst` for the launches behind it (in place of a copy on the
+// stream before it) and takes the factors from there itself.
 template <int D>
 __global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const uint32_t *factors,
                                                           uint32_t n_factor_words, uint32_t *out, uint64_t total,
-                                                          uint32_t *zero, uint64_t zero_words) {
+                                                          uint32_t *zero, uint64_t zero_words,
+                                                          const uint32_t *staged = nullptr, uint32_t staged_words = 0,
+                                                          uint32_t *staged_dst = nullptr) {
   uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
   for (uint64_t z = gid; z < zero_words; z += (uint64_t)gridDim.x * BLOCK) zero[z] = 0;
+  if (staged) {
+    for (uint64_t z = gid; z < staged_words; z += (uint64_t)gridDim.x * BLOCK) staged_dst[z] = staged[z];
+    factors = staged;
+  }
   // every variable's two factors into LDS first: an entry is a chain of up to `bits` products, and a load from
   // memory inside each link is most of the kernel's time
   __shared__ uint32_t lds_factors[2 * MAXROUNDS * 8];
@@ -59,9 +68,13 @@ __global__ __launch_bounds__(BLOCK) void eq_tables_kernel(EqTables tabs, const u
 }
 
 template <int D>
-__global__ __launch_bounds__(BLOCK) void fill_ones_kernel(uint32_t *out, uint64_t n, uint32_t *zero, uint64_t zero_words) {
+__global__ __launch_bounds__(BLOCK) void fill_ones_kernel(uint32_t *out, uint64_t n, uint32_t *zero, uint64_t zero_words,
+                                                          const uint32_t *staged = nullptr, uint32_t staged_words = 0,
+                                                          uint32_t *staged_dst = nullptr) {
   uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
   for (uint64_t z = gid; z < zero_words; z += (uint64_t)gridDim.x * BLOCK) zero[z] = 0;
+  if (staged)
+    for (uint64_t z = gid; z < staged_words; z += (uint64_t)gridDim.x * BLOCK) staged_dst[z] = staged[z];
   if (gid < n) store_ext<D>(out + gid * D, ext_lift<D>(1));
 }
 
@@ -462,7 +475,7 @@ int eq_tables_launch(int D, int count, const int *first, const int *bits, const 
 
 static uint64_t tail_pairs(int T, int D);
 
-int SumcheckSession::launch_setup() {
+int SumcheckSession::launch_setup(const uint32_t *staged, size_t staged_words) {
   Context &c = ctx();
   uint32_t *base = d_weights;
   EqTables eqt;
@@ -479,27 +492,33 @@ int SumcheckSession::launch_setup() {
     // offsets themselves may skip other regions, so they are taken from eqt.off
     if (D == 4)
       hipLaunchKernelGGL(eq_tables_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, (uint32_t)(2 * n * D), base,
-                         setup.total_eq, zero, zero_words);
+                         setup.total_eq, zero, zero_words, staged, (uint32_t)staged_words, base);
     else
       hipLaunchKernelGGL(eq_tables_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, eqt, base, (uint32_t)(2 * n * D), base,
-                         setup.total_eq, zero, zero_words);
+                         setup.total_eq, zero, zero_words, staged, (uint32_t)staged_words, base);
     cleared = zero_words > 0;
     zero_words = 0;
+    staged = nullptr;
   }
   if (setup.ones_len) {
     uint32_t grid = std::max((uint32_t)((setup.ones_len + BLOCK - 1) / BLOCK), zero_words ? zero_grid : 0u);
     if (D == 4)
       hipLaunchKernelGGL(fill_ones_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, base + setup.ones_off * D,
-                         setup.ones_len, zero, zero_words);
+                         setup.ones_len, zero, zero_words, staged, (uint32_t)staged_words, base);
     else
       hipLaunchKernelGGL(fill_ones_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, base + setup.ones_off * D,
-                         setup.ones_len, zero, zero_words);
+                         setup.ones_len, zero, zero_words, staged, (uint32_t)staged_words, base);
+    staged = nullptr;
     cleared = cleared || zero_words > 0;
     zero_words = 0;
   }
   c.prof_end();
   slice_totals_clear = cleared;  // else (no set-up kernel ran) the grid launch clears them itself
   EXH_HIP(hipGetLastError());
+  if (staged) {  // (no set-up kernel ran)
+    set_error("device-error: the session's staged constants were left behind");
+    return E_DEVICE;
+  }
   return OK;
 }
 
@@ -1012,11 +1031,20 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
     if (st_hook) return st_hook;
     setup_deferred = false;
     if (!own_weights && (st_hook = launch_setup())) return st_hook;
-  } else if (setup_deferred) {  // one copy for the session's constants and the loop's, then the weight tables
-    EXH_HIP(hipMemcpyAsync(d_weights, c.host_pinned + PIN_BEGIN, (setup_words + up_words) * 4, hipMemcpyHostToDevice,
-                           c.stream));
+  } else if (setup_deferred) {
+    // the session's constants and the loop's, staged in pinned memory, reach the device with the set-up launch,
+    // which reads them where they lie; with one copy on the stream when there is no such launch
+    // (EXACTA_HIP_COPY_CONSTANTS=1: always by that copy, the set-up launch behind it)
+    const char *copy_constants = getenv("EXACTA_HIP_COPY_CONSTANTS");
+    const bool by_launch = !own_weights && (setup.total_eq || setup.ones_len) && c.host_pinned_dev &&
+                           !(copy_constants && copy_constants[0] == '1');
+    if (!by_launch)
+      EXH_HIP(hipMemcpyAsync(d_weights, c.host_pinned + PIN_BEGIN, (setup_words + up_words) * 4, hipMemcpyHostToDevice,
+                             c.stream));
     setup_deferred = false;
-    int st_setup = own_weights ? OK : launch_setup();
+    int st_setup = own_weights ? OK
+                   : by_launch ? launch_setup(c.host_pinned_dev + PIN_BEGIN, setup_words + up_words)
+                               : launch_setup();
     if (st_setup) return st_setup;
   } else {
     EXH_HIP(hipMemcpyAsync(d_mtilde, up, up_words * 4, hipMemcpyHostToDevice, c.stream));
@@ -1136,7 +1164,8 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   if (status == OK && j < n) {  // the tail: rounds j .. n-1 and the last fold, in one workgroup
     // when a single entry per table is left at the end (the finals travel in the control block), the launch
     // itself delivers the control block to pinned host memory
-    const bool deliver = !c.profiling && !chain_hook && (size >> ((folds_due > 0 ? 1 : 0) + (n - j))) == 1;
+    const bool deliver =
+        !c.profiling && !chain_hook && ((size >> ((folds_due > 0 ? 1 : 0) + (n - j))) == 1 || finals_stay);
     if (deliver) {
       if (++c.log_seq == 0) ++c.log_seq;  // 0 is what the flag is reset to
       host_log = c.host_pinned_dev + PIN_DOWN, host_flag_at = (uint32_t)ctrl_words, host_seq = c.log_seq;
@@ -1163,7 +1192,7 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
   const size_t final_words = (size_t)T * size * D;
   final_cache.clear();
   const bool in_ctrl = tail_done && size == 1;  // the tail left the finals in the control block
-  const bool with_finals = tail_done && !in_ctrl && ctrl_words + final_words <= PIN_DOWN_WORDS;
+  const bool with_finals = tail_done && !in_ctrl && !finals_stay && ctrl_words + final_words <= PIN_DOWN_WORDS;
   if (logged_to_host) {
     // the flag follows the block through the same path, so seeing it means the block is there; a stream that
     // ends without raising it (a launch gave up) is caught by the query

@@ -87,6 +87,10 @@ struct SumcheckSession {
   // context's, so that several sessions can be open side by side (the parts of a statement too wide for one
   // kernel, proved in step).  Such a session runs host-driven rounds.
   bool private_buffers = false;
+  // The caller takes what the rounds leave of the tables on the device (finish_device) and never asks for them on
+  // the host: the device-driven loop then need not fetch them with its logs, and its last launch can deliver the
+  // logs to pinned memory itself whatever the tables' final length.
+  bool finals_stay = false;
   // Set before run_device by a caller that chains several sumchecks on the device (the layers of LogUp-GKR): the
   // loop's constants (eq factors, message map, constant terms, the head of the control block with the transcript's
   // state) are then written in device memory by the launch this hook enqueues, instead of being staged and copied
@@ -116,7 +120,7 @@ struct SumcheckSession {
     uint64_t total_eq = 0, ones_off = 0, ones_len = 0;
     unsigned char eqt[1536];  // the EqTables argument of eq_tables_kernel
   } setup;
-  int launch_setup();
+  int launch_setup(const uint32_t *staged = nullptr, size_t staged_words = 0);
   // claim mode: round_sums returns the honest claim sum_x w(x) F(tables(x)) in out[0..D) (n >= 1)
   bool claim_mode = false;
   std::vector<uint32_t> eq0;  // the eq point's first coordinate, for the claim
