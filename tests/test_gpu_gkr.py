@@ -84,11 +84,15 @@ def test_several_blocks_on_the_grid_of_slices_and_on_the_streaming_rounds(n, k, 
     dev = [(sa.Table.upload(p), sa.Table.upload(q)) for p, q in leaves]
     otr = orc.Transcript("gkr-blocks", d)
     want = orc.gkr_prove_upper(otr, n, k, leaves)
-    for off in ("0", "1"):
-        monkeypatch.setenv("EXACTA_HIP_NO_BLOCK_SLICES", off)
+    # (and with the older ways of moving a layer's constants and logs: a copy on the stream before the set-up launch,
+    # the folded tables fetched with the logs)
+    for switches in ({}, {"EXACTA_HIP_NO_BLOCK_SLICES": "1"}, {"EXACTA_HIP_COPY_CONSTANTS": "1"},
+                     {"EXACTA_HIP_FETCH_FINALS": "1"}):
+        for name in ("EXACTA_HIP_NO_BLOCK_SLICES", "EXACTA_HIP_COPY_CONSTANTS", "EXACTA_HIP_FETCH_FINALS"):
+            monkeypatch.setenv(name, switches.get(name, "0"))
         tr = sa.Transcript("gkr-blocks", d)
         got = sa.prove_upper(tr, n, k, dev)
-        assert tr.proof() == otr.proof(), off
+        assert tr.proof() == otr.proof(), switches
         for a, b in zip(got, want):
             assert same(a, b)
     for p, q in dev:

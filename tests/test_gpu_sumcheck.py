@@ -351,6 +351,29 @@ def test_a_small_session_builds_its_weight_tables_in_its_one_launch(form, names,
         t.free()
 
 
+@pytest.mark.parametrize("form,names,d,n,base,with_eq", [
+    ("(* t0 t1 t2)", ["t0", "t1", "t2"], 4, 17, True, True),
+    ("(* t0 t1)", ["t0", "t1"], 8, 12, False, True),
+    ("(* t0 t1)", ["t0", "t1"], 4, 11, False, False),
+])
+def test_a_session_takes_its_constants_with_the_set_up_launch_or_by_a_copy(form, names, d, n, base, with_eq, monkeypatch):
+    """The constants a session stages in pinned memory reach the device with its set-up launch (weight tables, or
+    ones without an eq point), which reads them where they lie; EXACTA_HIP_COPY_CONSTANTS=1 sends them with a copy
+    on the stream first.  Same bytes as the oracle either way."""
+    rng = np.random.default_rng(n * 17 + d)
+    tables = [rng.integers(0, P, 1 << n, dtype=np.uint32) if base else rand_ext(rng, (1 << n,), d) for _ in names]
+    eq = rand_ext(rng, (n,), d) if with_eq else None
+    st, _, proof, _ = prove_both("constants", d, n, form, names, tables, eq=eq)
+    dev = [sa.Table.upload(t) for t in tables]
+    for copy in ("0", "1"):
+        monkeypatch.setenv("EXACTA_HIP_COPY_CONSTANTS", copy)
+        tr = sa.Transcript("constants", d)
+        sa.prove(tr, n, st, dev, eq=eq)
+        assert tr.proof() == proof, copy
+    for t in dev:
+        t.free()
+
+
 @pytest.mark.parametrize("points,n", [(2, 7), (2, 15), (3, 14), (4, 13), (4, 19)])
 def test_point_reductions_of_an_opening(points, n):
     """REDUCE-POINTS' sumcheck (src/pcs.lisp:333-373): sum_z eq(z, x) g_z(x) over extension tables, no eq weights,
