@@ -78,12 +78,21 @@ int gkr_reduce_layer(int D, int K, int m, const uint32_t *p, const uint32_t *q, 
 
 // the lower and upper halves of each block, as K contiguous blocks each (HALVES-PER-BLOCK,
 // src/gkr.lisp:190-197); only needed when K > 1: with one block the halves are views
+// (every vector of a layer in one launch: blockIdx.y picks the vector; the halves of vector i go to
+// out + (2 i) n_out D and out + (2 i + 1) n_out D)
+struct HalvesArgs {
+  const uint32_t *v[MAXT];
+  uint32_t *out;
+  uint32_t size_bits;
+  uint64_t n_out;
+};
 template <int D>
-__global__ __launch_bounds__(BLOCK) void halves_kernel(const uint32_t *v, uint32_t *lower, uint32_t *upper,
-                                                       uint32_t size_bits, uint64_t n_out) {
+__global__ __launch_bounds__(BLOCK) void halves_kernel(HalvesArgs a) {
   uint64_t o = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
-  if (o >= n_out) return;
-  uint64_t size = (uint64_t)1 << size_bits, b = o >> size_bits, x = o & (size - 1);
+  if (o >= a.n_out) return;
+  const uint32_t *v = a.v[blockIdx.y];
+  uint32_t *lower = a.out + (uint64_t)(2 * blockIdx.y) * a.n_out * D, *upper = lower + a.n_out * D;
+  uint64_t size = (uint64_t)1 << a.size_bits, b = o >> a.size_bits, x = o & (size - 1);
   store_ext<D>(lower + o * D, load_ext<D>(v + (b * 2 * size + x) * D));
   store_ext<D>(upper + o * D, load_ext<D>(v + (b * 2 * size + size + x) * D));
 }
@@ -549,27 +558,31 @@ int gkr_prove_upper(Transcript &tr, int n, int K, int L, const uint32_t *const *
     std::vector<uint32_t> bw = block_weights(D, K, rb);
     uint64_t size = (uint64_t)1 << layer;
     std::vector<const uint32_t *> tabs(NT);
-    for (int l = 0; l < L; l++)
-      for (int w = 0; w < 2; w++) {
-        const uint32_t *v = layers[layer + 1][2 * l + w];
-        if (K == 1) {  // the halves are views
+    if (K == 1) {  // the halves are views
+      for (int l = 0; l < L; l++)
+        for (int w = 0; w < 2; w++) {
+          const uint32_t *v = layers[layer + 1][2 * l + w];
           tabs[4 * l + 2 * w] = v;
           tabs[4 * l + 2 * w + 1] = v + size * D;
-        } else {
-          uint32_t *lo = bufs.alloc(K * size * D), *hi = bufs.alloc(K * size * D);
-          if (!lo || !hi) return E_NOMEM;
-          uint64_t n_out = K * size;
-          uint32_t grid = (uint32_t)((n_out + BLOCK - 1) / BLOCK);
-          if (D == 4)
-            hipLaunchKernelGGL(halves_kernel<4>, dim3(grid), dim3(BLOCK), 0, c.stream, v, lo, hi, (uint32_t)layer,
-                               n_out);
-          else
-            hipLaunchKernelGGL(halves_kernel<8>, dim3(grid), dim3(BLOCK), 0, c.stream, v, lo, hi, (uint32_t)layer,
-                               n_out);
-          tabs[4 * l + 2 * w] = lo;
-          tabs[4 * l + 2 * w + 1] = hi;
         }
+    } else {  // one launch splits the layer's 2 L vectors
+      const uint64_t n_out = K * size;
+      HalvesArgs h;
+      memset(&h, 0, sizeof(h));
+      if (!(h.out = bufs.alloc((uint64_t)NT * n_out * D))) return E_NOMEM;
+      h.size_bits = (uint32_t)layer, h.n_out = n_out;
+      for (int i = 0; i < 2 * L; i++) {
+        h.v[i] = layers[layer + 1][i];
+        tabs[2 * i] = h.out + (uint64_t)(2 * i) * n_out * D;
+        tabs[2 * i + 1] = h.out + (uint64_t)(2 * i + 1) * n_out * D;
       }
+      const dim3 grid((uint32_t)((n_out + BLOCK - 1) / BLOCK), (uint32_t)(2 * L));
+      if (D == 4)
+        hipLaunchKernelGGL(halves_kernel<4>, grid, dim3(BLOCK), 0, c.stream, h);
+      else
+        hipLaunchKernelGGL(halves_kernel<8>, grid, dim3(BLOCK), 0, c.stream, h);
+      EXH_HIP(hipGetLastError());
+    }
     // With several blocks the folded tables (one entry per block) stay on the device, zero padded to 2^lk, as the
     // tables of the sumcheck over the block index; the weights, padded alike, go before them in one copy.
     uint32_t *d_blk = nullptr;
