@@ -573,7 +573,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="config2",
                     choices=["config1", "config2", "config3", "config4", "config5", "basefold", "domain", "combine",
-                             "combine128", "copy", "mulrate"],
+                             "combine128", "copy", "mulrate", "gkr_shapes"],
                     help="config2 (default) is the headline; the others are the remaining configured workloads; "
                          "copy is the known-size kernel the traffic counters are calibrated on")
     ap.add_argument("--gpus", type=int, default=1)
@@ -615,6 +615,15 @@ def main():
         print(json.dumps(line("LogUp-GKR prove-upper lookups/s (config 4)", res["lookups_per_s"], "lookups/s", True,
                               "u32 (Montgomery KoalaBear, F_p^4 tower)",
                               "synthetic (seeded uniform int8 lookups, exact multiplicities)", res, steps, warmup)))
+        return
+    if args.workload == "gkr_shapes":
+        shapes = run_gkr_shapes(sa, steps, warmup)
+        blocks = shapes["three_blocks_one_lookup"]
+        res = {"workload": "LogUp-GKR prove-upper at the shapes a domain gives it: 2^14 leaves per block and lookup, "
+                           "one block with three lookups, three blocks with one and with two; `value` is three blocks "
+                           "with one lookup", "ms_per_step": blocks["ms_per_step"], "shapes": shapes}
+        print(json.dumps(line("LogUp-GKR prove-upper lookups/s (3 blocks of 2^14)", 3 * (1 << 14) / (blocks["ms_per_step"] * 1e-3),
+                              "lookups/s", True, "u32 (Montgomery KoalaBear, F_p^4 tower)", SEEDED, res, steps, warmup)))
         return
     if args.workload == "config5":
         res = run_commit(sa, steps, warmup, gold)

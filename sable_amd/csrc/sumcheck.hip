@@ -1101,6 +1101,9 @@ int SumcheckSession::run_device(const DevB3S &state, uint32_t *messages, uint32_
       uint64_t grid = odd;
       while (grid * 2 <= grid_max && grid * 2 <= left && (n_pairs / (grid * 2)) >= BLOCK) grid *= 2;
       while (n_pairs / grid > slice_max && grid * 2 <= grid_max && grid * 2 <= left) grid *= 2;
+      // (fewer pairs than two workgroups have threads, yet more than the one-workgroup launch holds -- statements
+      // of many tables: two workgroups' rounds still cost a fraction of a streaming launch per round)
+      if (grid == 1 && grid_max >= 2 && left >= 2) grid = 2;
       // the grid's workgroups wait for one another: all of them must be resident at once.  The runtime says how
       // many of this kernel a compute unit holds with the slices' LDS; a grid beyond that stays on the streaming
       // kernels (asked once per kernel and size)
