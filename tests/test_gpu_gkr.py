@@ -44,7 +44,10 @@ CASES = [(3, 1, 1, 4), (3, 3, 2, 4), (2, 4, 1, 8), (4, 5, 2, 4), (1, 2, 1, 4), (
          (9, 3, 1, 4), (8, 2, 2, 4), (7, 6, 1, 8), (11, 4, 3, 4),
          # one block: the layers chained on the device (up to twelve base challenges per layer), from the smallest
          # tree that chains to one whose upper layers take the grid of slices
-         (2, 1, 1, 4), (5, 1, 2, 4), (7, 1, 1, 8), (13, 1, 1, 4), (12, 1, 2, 4), (6, 1, 3, 4), (11, 1, 3, 4)]
+         (2, 1, 1, 4), (5, 1, 2, 4), (7, 1, 1, 8), (13, 1, 1, 4), (12, 1, 2, 4), (6, 1, 3, 4), (11, 1, 3, 4),
+         # statements of many tables in F_p^8: few pairs fit the one-workgroup launch, and the rounds just above it
+         # go to two workgroups' slices
+         (9, 1, 3, 8), (10, 1, 2, 8), (8, 3, 2, 8)]
 
 
 @pytest.mark.parametrize("n,k,lookups,d", CASES)
